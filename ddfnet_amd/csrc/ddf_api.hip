@@ -1,0 +1,196 @@
+// C ABI of the DDF HIP library: argument validation and kernel-family choice.
+// Declarations and the reference entry points each call replaces are in
+// include/ddf_hip.h.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "ddf_common.h"
+
+namespace {
+
+thread_local char g_last_error[512] = "";
+
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int fail_hip(hipError_t err, const char *what) {
+    return fail(DDF_ERR_HIP, "%s: %s", what, hipGetErrorString(err));
+}
+
+// Checks shared by forward and backward.  Mirrors the argument contract of
+// DDFFunction.forward (ddf/ddf.py:45-65 of the reference): odd k >= 1,
+// d >= 1, s >= 1, known combine; sizes must be non-negative.
+int check_problem(int64_t N, int64_t C, int64_t H, int64_t W, int k, int d, int s,
+                  int combine, int dtype, int variant) {
+    if (N < 0 || C < 0 || H < 0 || W < 0)
+        return fail(DDF_ERR_BAD_ARG, "negative tensor size (N=%lld C=%lld H=%lld W=%lld)",
+                    (long long)N, (long long)C, (long long)H, (long long)W);
+    if (k < 1 || (k - 1) % 2 != 0 || d < 1 || s < 1)
+        return fail(DDF_ERR_BAD_ARG,
+                    "kernel_size must be odd and >= 1, dilation and stride >= 1 "
+                    "(got k=%d d=%d s=%d)", k, d, s);
+    if (combine != DDF_MUL && combine != DDF_ADD)
+        return fail(DDF_ERR_BAD_ARG, "combine must be DDF_MUL or DDF_ADD (got %d)", combine);
+    if (dtype != DDF_F16 && dtype != DDF_F32 && dtype != DDF_F64)
+        return fail(DDF_ERR_BAD_ARG, "unknown dtype %d", dtype);
+    if (variant != DDF_VARIANT_AUTO && variant != DDF_VARIANT_GENERIC &&
+        variant != DDF_VARIANT_TILED)
+        return fail(DDF_ERR_BAD_ARG, "unknown variant %d", variant);
+    // Index arithmetic inside the kernels is 64-bit, but a single (n, c) plane
+    // and the tap window must fit 32-bit offsets.
+    if (H > (1 << 24) || W > (1 << 24) || (int64_t)k * d > (1 << 20))
+        return fail(DDF_ERR_UNSUPPORTED, "plane or window too large");
+    return DDF_OK;
+}
+
+template <typename T>
+int forward_typed(const ddf::Problem &p, const void *x, const void *cf, const void *sf,
+                  void *out, int dtype, int variant, hipStream_t stream) {
+    const bool tiled_ok = ddf::tiled_forward_supported(p, dtype);
+    if (variant == DDF_VARIANT_TILED && !tiled_ok)
+        return fail(DDF_ERR_UNSUPPORTED,
+                    "tiled forward does not cover k=%d d=%d s=%d H=%lld W=%lld", p.k, p.d,
+                    p.s, (long long)p.H, (long long)p.W);
+    hipError_t err;
+    if (tiled_ok && variant != DDF_VARIANT_GENERIC)
+        err = ddf::tiled_forward<T>(p, (const T *)x, (const T *)cf, (const T *)sf, (T *)out,
+                                    stream);
+    else
+        err = ddf::generic_forward<T>(p, (const T *)x, (const T *)cf, (const T *)sf,
+                                      (T *)out, stream);
+    return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_forward launch");
+}
+
+template <typename T>
+int backward_typed(const ddf::Problem &p, const void *go, const void *x, const void *cf,
+                   const void *sf, void *dx, void *dcf, void *dsf, void *ws,
+                   size_t ws_bytes, int dtype, unsigned need, int variant,
+                   hipStream_t stream) {
+    const bool tiled_ok = ddf::tiled_backward_supported(p, dtype);
+    if (variant == DDF_VARIANT_TILED && !tiled_ok)
+        return fail(DDF_ERR_UNSUPPORTED,
+                    "tiled backward does not cover k=%d d=%d s=%d H=%lld W=%lld", p.k, p.d,
+                    p.s, (long long)p.H, (long long)p.W);
+    hipError_t err;
+    if (tiled_ok && variant != DDF_VARIANT_GENERIC) {
+        const size_t want = ddf::tiled_backward_workspace(p, dtype, need);
+        if (want > 0 && (ws == nullptr || ws_bytes < want))
+            return fail(DDF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", want,
+                        ws == nullptr ? (size_t)0 : ws_bytes);
+        if (want > 0 && ((uintptr_t)ws & 255u) != 0)
+            return fail(DDF_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+        err = ddf::tiled_backward<T>(p, (const T *)go, (const T *)x, (const T *)cf,
+                                     (const T *)sf, (T *)dx, (T *)dcf, (T *)dsf, ws, need,
+                                     stream);
+    } else {
+        err = ddf::generic_backward<T>(p, (const T *)go, (const T *)x, (const T *)cf,
+                                       (const T *)sf, (T *)dx, (T *)dcf, (T *)dsf, need,
+                                       stream);
+    }
+    return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_backward launch");
+}
+
+}  // namespace
+
+extern "C" {
+
+int ddf_hip_version(void) { return 100; }
+
+const char *ddf_hip_status_string(int status) {
+    switch (status) {
+        case DDF_OK: return "ok";
+        case DDF_ERR_BAD_ARG: return "bad argument";
+        case DDF_ERR_UNSUPPORTED: return "unsupported configuration";
+        case DDF_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case DDF_ERR_HIP: return "hip runtime error";
+        default: return "unknown status";
+    }
+}
+
+const char *ddf_hip_last_error(void) { return g_last_error; }
+
+int ddf_hip_forward(const void *features, const void *channel_filter,
+                    const void *spatial_filter, void *output, int64_t N, int64_t C,
+                    int64_t H, int64_t W, int kernel_size, int dilation, int stride,
+                    int combine, int dtype, int variant, void *stream) {
+    int rc = check_problem(N, C, H, W, kernel_size, dilation, stride, combine, dtype, variant);
+    if (rc != DDF_OK) return rc;
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
+    if (N * C * p.Ho * p.Wo == 0) return DDF_OK;  // nothing to write
+    if (!features || !channel_filter || !spatial_filter || !output)
+        return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DDF_F16:
+            return forward_typed<__half>(p, features, channel_filter, spatial_filter, output,
+                                         dtype, variant, st);
+        case DDF_F32:
+            return forward_typed<float>(p, features, channel_filter, spatial_filter, output,
+                                        dtype, variant, st);
+        default:
+            return forward_typed<double>(p, features, channel_filter, spatial_filter, output,
+                                         dtype, variant, st);
+    }
+}
+
+size_t ddf_hip_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W,
+                                        int kernel_size, int dilation, int stride,
+                                        int combine, int dtype, unsigned need_mask,
+                                        int variant) {
+    if (check_problem(N, C, H, W, kernel_size, dilation, stride, combine, dtype, variant) !=
+        DDF_OK)
+        return 0;
+    if (variant == DDF_VARIANT_GENERIC) return 0;
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
+    if (!ddf::tiled_backward_supported(p, dtype)) return 0;
+    return ddf::tiled_backward_workspace(p, dtype, need_mask & DDF_NEED_ALL);
+}
+
+int ddf_hip_backward(const void *grad_output, const void *features,
+                     const void *channel_filter, const void *spatial_filter,
+                     void *grad_features, void *grad_channel_filter,
+                     void *grad_spatial_filter, void *workspace, size_t workspace_bytes,
+                     int64_t N, int64_t C, int64_t H, int64_t W, int kernel_size,
+                     int dilation, int stride, int combine, int dtype, unsigned need_mask,
+                     int variant, void *stream) {
+    int rc = check_problem(N, C, H, W, kernel_size, dilation, stride, combine, dtype, variant);
+    if (rc != DDF_OK) return rc;
+    const unsigned need = need_mask & DDF_NEED_ALL;
+    if (need == 0) return DDF_OK;
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
+    if (N * C == 0) return DDF_OK;  // every gradient is empty
+    if (!grad_output && N * C * p.Ho * p.Wo != 0)
+        return fail(DDF_ERR_BAD_ARG, "null grad_output");
+    if (!features || !channel_filter || !spatial_filter)
+        if (N * C * H * W != 0) return fail(DDF_ERR_BAD_ARG, "null input tensor pointer");
+    if (((need & DDF_NEED_DX) && !grad_features && N * C * H * W != 0) ||
+        ((need & DDF_NEED_DCF) && !grad_channel_filter) ||
+        ((need & DDF_NEED_DSF) && !grad_spatial_filter && p.Ho * p.Wo != 0))
+        return fail(DDF_ERR_BAD_ARG, "null pointer for a requested gradient");
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DDF_F16:
+            return backward_typed<__half>(p, grad_output, features, channel_filter,
+                                          spatial_filter, grad_features, grad_channel_filter,
+                                          grad_spatial_filter, workspace, workspace_bytes,
+                                          dtype, need, variant, st);
+        case DDF_F32:
+            return backward_typed<float>(p, grad_output, features, channel_filter,
+                                         spatial_filter, grad_features, grad_channel_filter,
+                                         grad_spatial_filter, workspace, workspace_bytes,
+                                         dtype, need, variant, st);
+        default:
+            return backward_typed<double>(p, grad_output, features, channel_filter,
+                                          spatial_filter, grad_features, grad_channel_filter,
+                                          grad_spatial_filter, workspace, workspace_bytes,
+                                          dtype, need, variant, st);
+    }
+}
+
+}  // extern "C"

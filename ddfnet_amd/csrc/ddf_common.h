@@ -1,0 +1,71 @@
+// Shared declarations of the DDF HIP library (gfx950 only, wave64).
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "ddf_hip.h"
+
+namespace ddf {
+
+constexpr int kWave = 64;
+
+// Problem description handed to every launcher.  Ho/Wo use floor division
+// (ddf/ddf.py:56 of the reference), r is the tap radius in taps.
+struct Problem {
+    int64_t N, C, H, W, Ho, Wo;
+    int k, d, s, r, kk;
+    bool mul;
+};
+
+inline Problem make_problem(int64_t N, int64_t C, int64_t H, int64_t W, int k,
+                            int d, int s, int combine) {
+    Problem p;
+    p.N = N; p.C = C; p.H = H; p.W = W;
+    p.Ho = H / s; p.Wo = W / s;
+    p.k = k; p.d = d; p.s = s; p.r = (k - 1) / 2; p.kk = k * k;
+    p.mul = (combine == DDF_MUL);
+    return p;
+}
+
+// Accumulator type: fp16 and fp32 storage accumulate in fp32, fp64 in fp64.
+template <typename T> struct Acc { using type = float; };
+template <> struct Acc<double> { using type = double; };
+
+__device__ __forceinline__ float ld(const __half *p) { return __half2float(*p); }
+__device__ __forceinline__ float ld(const float *p) { return *p; }
+__device__ __forceinline__ double ld(const double *p) { return *p; }
+__device__ __forceinline__ void st(__half *p, float v) { *p = __float2half(v); }
+__device__ __forceinline__ void st(float *p, float v) { *p = v; }
+__device__ __forceinline__ void st(double *p, double v) { *p = v; }
+
+template <bool MUL, typename A>
+__device__ __forceinline__ A comb(A a, A b) { return MUL ? a * b : a + b; }
+
+inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Launchers.  Each returns a hipError_t from the launch (hipSuccess when the
+// tensor is empty and nothing was launched).  `supported` queries tell the
+// API layer whether the tiled family covers a problem.
+template <typename T>
+hipError_t generic_forward(const Problem &p, const T *x, const T *cf, const T *sf,
+                           T *out, hipStream_t st);
+template <typename T>
+hipError_t generic_backward(const Problem &p, const T *go, const T *x, const T *cf,
+                            const T *sf, T *dx, T *dcf, T *dsf, unsigned need,
+                            hipStream_t st);
+
+bool tiled_forward_supported(const Problem &p, int dtype);
+template <typename T>
+hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,
+                         T *out, hipStream_t st);
+
+bool tiled_backward_supported(const Problem &p, int dtype);
+size_t tiled_backward_workspace(const Problem &p, int dtype, unsigned need);
+template <typename T>
+hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf,
+                          const T *sf, T *dx, T *dcf, T *dsf, void *ws,
+                          unsigned need, hipStream_t st);
+
+}  // namespace ddf

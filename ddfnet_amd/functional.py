@@ -1,0 +1,181 @@
+"""The ``ddf`` autograd operator on the gfx950 HIP kernels.
+
+Host-side mirror of ``DDFFunction`` / ``ddf`` / ``OP_DICT`` of the reference
+(``ddf/ddf.py:19-122``): same positional signature, same assertion messages,
+same 8-tuple from ``backward``.  All arithmetic of the operator happens in
+``libddf_hip.so``; nothing here computes it in PyTorch and there is no
+fallback when the library is missing.
+
+Deliberate differences from the reference, each a superset of its behaviour:
+
+* fp16 runs natively (fp16 in and out, fp32 accumulation) rather than being
+  widened to fp32 first (``ddf/ddf.py:36-42``, ``:74``).  Operands of different
+  dtypes are promoted to the widest one, which is what the reference's
+  per-tensor widening amounts to.
+* Non-contiguous operands are made contiguous instead of raising
+  (``ddf/src/cuda/ddf_mul_cuda.cpp:27-32``).
+* Only the gradients autograd asks for are computed, and none of the six
+  zero-filled tensors of ``ddf/ddf.py:106-111`` is allocated.
+"""
+import torch
+from torch.autograd import Function
+
+from . import _lib
+
+__all__ = ['DDFFunction', 'ddf', 'OP_DICT']
+
+
+def _require_device_contiguous(named_tensors):
+    """What CHECK_INPUT enforces in ddf/src/cuda/ddf_mul_cuda.cpp:25-32, and the
+    CPU rejection of ddf/src/ddf_mul_ext.cpp:33."""
+    for name, t in named_tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            if name in ('features', 'top_grad'):
+                raise RuntimeError('ddf operation is not implemented on CPU')
+            raise RuntimeError(name + ' must be a CUDA tensor ')
+        if not t.is_contiguous():
+            raise RuntimeError(name + ' must be contiguous ')
+
+
+class _NativeOp(object):
+    """Stand-in for one of the reference's four extension modules
+    (``ddf/src/ddf_mul_ext.cpp:57-60``, ``ddf_mul_faster_ext.cpp:28-30``):
+    caller-allocated outputs, positional arguments in the reference's order,
+    return value 1."""
+
+    def __init__(self, combine, variant, with_backward=True):
+        self.combine, self.variant = combine, variant
+        if not with_backward:  # the faster modules export forward only
+            self.backward = None
+
+    def forward(self, features, channel_filter, spatial_filter,
+                kernel_size, dilation, stride, output):
+        _require_device_contiguous((('features', features),
+                                    ('channel_filter', channel_filter),
+                                    ('spatial_filter', spatial_filter),
+                                    ('output', output)))
+        with torch.cuda.device(features.device):
+            _lib.forward(features, channel_filter, spatial_filter, output,
+                         kernel_size, dilation, stride, self.combine, self.variant)
+        return 1
+
+    def backward(self, top_grad, features, channel_filter, spatial_filter,
+                 kernel_size, dilation, stride,
+                 rtop_grad, rbottom_grad, rspatial_filter_grad,
+                 bottom_grad, channel_filter_grad, spatial_filter_grad):
+        """``rtop_grad``, ``rbottom_grad`` and ``rspatial_filter_grad`` were
+        NHWC scratch in the reference (``ddf/src/cuda/ddf_mul_cuda.cpp:82-87``);
+        they are accepted and never touched.  A gradient passed as ``None`` is
+        not computed."""
+        grads = (('bottom_grad', bottom_grad, _lib.NEED_DX),
+                 ('channel_filter_grad', channel_filter_grad, _lib.NEED_DCF),
+                 ('spatial_filter_grad', spatial_filter_grad, _lib.NEED_DSF))
+        _require_device_contiguous((('top_grad', top_grad), ('features', features),
+                                    ('channel_filter', channel_filter),
+                                    ('spatial_filter', spatial_filter)) +
+                                   tuple((n, t) for n, t, _ in grads))
+        need = sum(bit for _, t, bit in grads if t is not None)
+        with torch.cuda.device(features.device):
+            nbytes = _lib.backward_workspace_bytes(
+                features.shape, kernel_size, dilation, stride, self.combine,
+                features.dtype, need, self.variant)
+            workspace = (torch.empty(nbytes, dtype=torch.uint8, device=features.device)
+                         if nbytes else None)
+            _lib.backward(top_grad, features, channel_filter, spatial_filter,
+                          bottom_grad, channel_filter_grad, spatial_filter_grad,
+                          kernel_size, dilation, stride, self.combine, need,
+                          workspace, self.variant)
+        return 1
+
+
+# Keys as in ddf/ddf.py:19-24.  The '*_faster' entries force the tiled kernels.
+OP_DICT = {
+    'mul': _NativeOp('mul', ''),
+    'mul_faster': _NativeOp('mul', 'f', with_backward=False),
+    'add': _NativeOp('add', ''),
+    'add_faster': _NativeOp('add', 'f', with_backward=False),
+}
+# version='o': the generic kernels, forward and backward.
+_ORIGINAL = {'mul': _NativeOp('mul', 'o'), 'add': _NativeOp('add', 'o')}
+
+
+class DDFFunction(Function):
+    @staticmethod
+    def forward(ctx, features, channel_filter, spatial_filter,
+                kernel_size=3, dilation=1, stride=1, kernel_combine='mul', version=''):
+        assert features.is_cuda, 'input feature must be a CUDA tensor.'
+        assert channel_filter.is_cuda, 'channel_filter must be a CUDA tensor.'
+        assert spatial_filter.is_cuda, 'spatial_filter must be a CUDA tensor.'
+
+        # one working dtype for the three operands
+        dtype = features.dtype
+        for other in (channel_filter, spatial_filter):
+            dtype = torch.promote_types(dtype, other.dtype)
+        assert dtype in _lib.DTYPE, 'unsupported dtype {}'.format(dtype)
+        features, channel_filter, spatial_filter = (
+            t.to(dtype).contiguous() for t in (features, channel_filter, spatial_filter))
+
+        b, c, h, w = features.size()
+        out_h, out_w = h // stride, w // stride
+        bc, cc, hc, wc = channel_filter.size()
+        assert bc == b and cc == c,\
+            "channel_filter size {} does not match feature size {}".format(
+                channel_filter.size(), features.size())
+        assert hc == kernel_size and wc == kernel_size,\
+            "channel_filter size {} does not match kernel size {}".format(
+                channel_filter.size(), kernel_size)
+        bs, cs, hs, ws = spatial_filter.size()
+        assert bs == b and hs == out_h and ws == out_w,\
+            "spatial_filter size {} does not match feature size {} with stride {}".format(
+                spatial_filter.size(), features.size(), stride)
+        assert cs == kernel_size ** 2,\
+            "spatial_filter size {} does not match kernel size {}".format(
+                spatial_filter.size(), kernel_size)
+        assert (kernel_size - 1) % 2 == 0 and kernel_size >= 1 and dilation >= 1 and stride >= 1
+        assert kernel_combine in {'mul', 'add'}, \
+            'only support mul or add combination, instead of {}'.format(kernel_combine)
+        assert version in {'', 'o', 'f'}, \
+            "version must be '', 'o' or 'f', instead of {}".format(version)
+
+        ctx.kernel_size, ctx.dilation, ctx.stride = kernel_size, dilation, stride
+        ctx.op_type = kernel_combine
+        ctx.version = version
+
+        # 'f' forces the tiled kernels, 'o' the generic ones, '' lets the
+        # library choose (the reference's own rule is at ddf/ddf.py:77-84).
+        if version == 'f':
+            op = OP_DICT[kernel_combine + '_faster']
+        elif version == 'o':
+            op = _ORIGINAL[kernel_combine]
+        else:
+            op = OP_DICT[kernel_combine]
+
+        # the kernels write every element, so no zero fill
+        output = features.new_empty((b, c, out_h, out_w))
+        op.forward(features, channel_filter, spatial_filter,
+                   kernel_size, dilation, stride, output)
+        if features.requires_grad or channel_filter.requires_grad or spatial_filter.requires_grad:
+            ctx.save_for_backward(features, channel_filter, spatial_filter)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        assert grad_output.is_cuda
+        features, channel_filter, spatial_filter = ctx.saved_tensors
+        grad_output = grad_output.to(features.dtype).contiguous()
+
+        wanted = ctx.needs_input_grad[:3]
+        grad_input, grad_channel_filter, grad_spatial_filter = (
+            torch.empty_like(t) if w else None
+            for t, w in zip((features, channel_filter, spatial_filter), wanted))
+
+        op = _ORIGINAL[ctx.op_type] if ctx.version == 'o' else OP_DICT[ctx.op_type]
+        op.backward(grad_output, features, channel_filter, spatial_filter,
+                    ctx.kernel_size, ctx.dilation, ctx.stride, None, None, None,
+                    grad_input, grad_channel_filter, grad_spatial_filter)
+        return grad_input, grad_channel_filter, grad_spatial_filter, None, None, None, None, None
+
+
+ddf = DDFFunction.apply

@@ -1,0 +1,177 @@
+"""Callers of the ``ddf`` operator: filter normalisation, the two filter
+branches, ``DDFPack`` and ``DDFUpPack``.
+
+These are ordinary PyTorch modules around the HIP operator.  Constructor
+arguments, sub-module names and parameter names follow the reference
+(``ddf/ddf.py:125-272``) so that its checkpoints load and its callers
+(``ddf_resnet.py:46-47``, ``test_time.py:56``) construct them unchanged.
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch.nn.init import calculate_gain
+
+from .functional import ddf
+
+__all__ = ['FilterNorm', 'build_spatial_branch', 'build_channel_branch',
+           'DDFPack', 'DDFUpPack']
+
+
+def _standardize(x, dim):
+    """(x - mean) / (unbiased std + 1e-10) over ``dim``
+    (``ddf/ddf.py:149-150``, ``:162-163``)."""
+    var, mean = torch.var_mean(x, dim=dim, keepdim=True)  # unbiased by default
+    return (x - mean) / (var.sqrt() + 1e-10)
+
+
+class FilterNorm(nn.Module):
+    """Standardise every predicted filter over its ``kernel_size**2`` taps, then
+    scale by a gain: the constant ``calculate_gain(nonlinearity) / kernel_size``
+    or, with ``running_std``, a learned per-tap vector initialised around it;
+    ``running_mean`` adds a learned per-tap offset (``ddf/ddf.py:125-173``).
+
+    ``'spatial'`` input is ``(b, in_channels * k*k, h, w)`` with taps on dim 1;
+    ``'channel'`` input is anything reshapeable to ``(b, in_channels, k*k)``
+    and comes back as ``(b, in_channels * k*k)``.
+    """
+
+    def __init__(self, in_channels, kernel_size, filter_type,
+                 nonlinearity='linear', running_std=False, running_mean=False):
+        assert filter_type in ('spatial', 'channel')
+        assert in_channels >= 1
+        super(FilterNorm, self).__init__()
+        self.in_channels = in_channels
+        self.filter_type = filter_type
+        # attribute spellings kept from the reference (ddf/ddf.py:133-134)
+        self.runing_std = running_std
+        self.runing_mean = running_mean
+        taps = in_channels * kernel_size ** 2
+        gain = calculate_gain(nonlinearity) / kernel_size
+        self.std = nn.Parameter(torch.randn(taps) * gain) if running_std else gain
+        if running_mean:
+            self.mean = nn.Parameter(torch.randn(taps))
+
+    def _affine(self, x, shape):
+        x = x * (self.std.view(shape) if self.runing_std else self.std)
+        if self.runing_mean:
+            x = x + self.mean.view(shape)
+        return x
+
+    def forward(self, x):
+        if self.filter_type == 'spatial':
+            b, ch, h, w = x.size()
+            x = _standardize(x.reshape(b, self.in_channels, -1, h, w), 2)
+            return self._affine(x.reshape(b, ch, h, w), (1, -1, 1, 1))
+        if self.filter_type == 'channel':
+            b = x.size(0)
+            x = _standardize(x.reshape(b, self.in_channels, -1), 2)
+            return self._affine(x.reshape(b, -1), (1, -1))
+        raise RuntimeError('Unsupported filter type {}'.format(self.filter_type))
+
+
+def build_spatial_branch(in_channels, kernel_size, head=1,
+                         nonlinearity='relu', stride=1):
+    """1x1 convolution (strided like the operator) to ``head * k*k`` taps per
+    pixel, then FilterNorm (``ddf/ddf.py:176-180``)."""
+    return nn.Sequential(
+        nn.Conv2d(in_channels, head * kernel_size ** 2, 1, stride=stride),
+        FilterNorm(head, kernel_size, 'spatial', nonlinearity))
+
+
+def build_channel_branch(in_channels, kernel_size,
+                         nonlinearity='relu', se_ratio=0.2):
+    """Squeeze-and-excite style branch: global average pool, bottleneck MLP of
+    1x1 convolutions, FilterNorm with a learned gain (``ddf/ddf.py:183-192``)."""
+    assert se_ratio > 0
+    mid_channels = int(in_channels * se_ratio)
+    return nn.Sequential(
+        nn.AdaptiveAvgPool2d((1, 1)),
+        nn.Conv2d(in_channels, mid_channels, 1),
+        nn.ReLU(True),
+        nn.Conv2d(mid_channels, in_channels * kernel_size ** 2, 1),
+        FilterNorm(in_channels, kernel_size, 'channel', nonlinearity, running_std=True))
+
+
+class DDFPack(nn.Module):
+    """Replacement for a ``k x k`` convolution: predicts both filters from the
+    input and applies them with ``ddf`` (``ddf/ddf.py:195-222``).  ``head > 1``
+    splits the channels into groups that each get their own spatial filter."""
+
+    def __init__(self, in_channels, kernel_size=3, stride=1, dilation=1, head=1,
+                 se_ratio=0.2, nonlinearity='relu', kernel_combine='mul'):
+        super(DDFPack, self).__init__()
+        assert kernel_size > 1
+        self.kernel_size = kernel_size
+        self.stride = stride
+        self.dilation = dilation
+        self.head = head
+        self.kernel_combine = kernel_combine
+        self.spatial_branch = build_spatial_branch(
+            in_channels, kernel_size, head, nonlinearity, stride)
+        self.channel_branch = build_channel_branch(
+            in_channels, kernel_size, nonlinearity, se_ratio)
+
+    def forward(self, x):
+        b, c, h, w = x.shape
+        g, k, s = self.head, self.kernel_size, self.stride
+        ho, wo = h // s, w // s
+        cf = self.channel_branch(x).reshape(b * g, c // g, k, k)
+        sf = self.spatial_branch(x).reshape(b * g, k * k, ho, wo)
+        out = ddf(x.reshape(b * g, c // g, h, w), cf, sf,
+                  k, self.dilation, s, self.kernel_combine)
+        return out.reshape(b, c, ho, wo)
+
+
+class DDFUpPack(nn.Module):
+    """Upsampling pack: ``scale_factor**2`` (spatial, channel) branch pairs, one
+    ``ddf`` call per pair, outputs interleaved by pixel shuffle
+    (``ddf/ddf.py:225-272``).  The spatial filters may be predicted from a
+    separate guidance tensor ``joint_x``.
+
+    The reference's ``forward`` passes ``self.head`` in the ``kernel_combine``
+    position (``ddf/ddf.py:267-268``) and so trips the operator's own
+    assertion; here the arguments are in the operator's order.
+    """
+
+    def __init__(self, in_channels, kernel_size=3, scale_factor=2, dilation=1, head=1, se_ratio=0.2,
+                 nonlinearity='linear', dw_kernel_size=3, joint_channels=-1, kernel_combine='mul'):
+        super(DDFUpPack, self).__init__()
+        self.kernel_size = kernel_size
+        self.dilation = dilation
+        self.head = head
+        self.scale_factor = scale_factor
+        self.kernel_combine = kernel_combine
+
+        self.spatial_branch = nn.ModuleList()
+        self.channel_branch = nn.ModuleList()
+        own_guidance = joint_channels < 1
+        if own_guidance:
+            dw_kernel_size = max(dw_kernel_size, 3)
+        for _ in range(scale_factor ** 2):
+            spatial = build_spatial_branch(in_channels, kernel_size, head, nonlinearity, 1)
+            if own_guidance:
+                # a depthwise convolution first gives each sub-pixel branch its
+                # own view of the neighbourhood
+                spatial = nn.Sequential(
+                    nn.Conv2d(in_channels, in_channels, dw_kernel_size,
+                              padding=kernel_size // 2, groups=in_channels),
+                    spatial)
+            self.spatial_branch.append(spatial)
+            self.channel_branch.append(
+                build_channel_branch(in_channels, kernel_size, nonlinearity, se_ratio))
+
+    def forward(self, x, joint_x=None):
+        if joint_x is None:
+            joint_x = x
+        b, c, h, w = x.shape
+        g, k = self.head, self.kernel_size
+        grouped = x.reshape(b * g, c // g, h, w)
+        subpixels = []
+        for spatial, channel in zip(self.spatial_branch, self.channel_branch):
+            cf = channel(x).reshape(b * g, c // g, k, k)
+            sf = spatial(joint_x).reshape(b * g, k * k, h, w)
+            o = ddf(grouped, cf, sf, k, self.dilation, 1, self.kernel_combine)
+            subpixels.append(o.type_as(x).reshape(b, c, h, w))
+        # (b, c, r*r, h, w) -> (b, c*r*r, h, w) -> pixel shuffle
+        out = torch.stack(subpixels, dim=2).reshape(b, -1, h, w)
+        return F.pixel_shuffle(out, self.scale_factor)

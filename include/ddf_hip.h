@@ -1,0 +1,130 @@
+/*
+ * ddf_hip.h - C ABI of the Decoupled Dynamic Filter (DDF) operator for gfx950.
+ *
+ * The library (libddf_hip.so) holds hand-written HIP kernels for the DDF
+ * forward pass and its three gradients.  Every entry point takes plain device
+ * pointers, sizes and enums; nothing here depends on torch.  All tensors are
+ * dense NCHW ("contiguous") and live on the device that is current when the
+ * call is made.  Calls are asynchronous: they enqueue kernels on `stream`
+ * (a hipStream_t passed as void*, NULL = the default stream) and return
+ * without synchronising.  The library keeps no global state and is
+ * re-entrant; the caller owns every buffer.
+ *
+ * Operator (r = (k-1)/2, Ho = H / s, Wo = W / s with floor division,
+ * t = i*k + j, comb(a,b) = a*b for DDF_MUL and a+b for DDF_ADD; a term whose
+ * feature index falls outside the image is zero):
+ *
+ *   out[n,c,y,x] = sum_{i,j} X[n,c, y*s+(i-r)*d, x*s+(j-r)*d]
+ *                            * comb(CF[n,c,i,j], SF[n,t,y,x])
+ *
+ * Shapes: X (N,C,H,W); CF (N,C,k,k); SF (N,k*k,Ho,Wo); out (N,C,Ho,Wo).
+ *
+ * Reference interface replaced (theFoxofSky/ddfnet):
+ *   ddf/src/ddf_mul_ext.cpp:21-34, :36-55   forward / backward, 'mul'
+ *   ddf/src/ddf_add_ext.cpp:21-34, :36-55   forward / backward, 'add'
+ *   ddf/src/ddf_mul_faster_ext.cpp:13-26    tiled forward, 'mul'
+ *   ddf/src/ddf_add_faster_ext.cpp:13-26    tiled forward, 'add'
+ * The four pybind modules collapse into the two calls below; `combine`
+ * selects mul/add and `variant` selects the generic or the tiled kernels.
+ */
+#ifndef DDF_HIP_H
+#define DDF_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element type of every tensor of one call (no mixed types).  DDF_F16 reads
+ * and writes IEEE half and accumulates in fp32. */
+typedef enum { DDF_F16 = 0, DDF_F32 = 1, DDF_F64 = 2 } ddf_dtype_t;
+
+/* How the channel filter and the spatial filter are combined per tap. */
+typedef enum { DDF_MUL = 0, DDF_ADD = 1 } ddf_combine_t;
+
+/* Kernel family.  DDF_VARIANT_AUTO picks the tiled kernels when the shape is
+ * supported by them and the generic kernels otherwise.  DDF_VARIANT_GENERIC
+ * corresponds to the reference's version 'o', DDF_VARIANT_TILED to 'f'
+ * (ddf/ddf.py:77-84); asking for the tiled family on a shape it does not
+ * cover returns DDF_ERR_UNSUPPORTED. */
+typedef enum {
+    DDF_VARIANT_AUTO = 0,
+    DDF_VARIANT_GENERIC = 1,
+    DDF_VARIANT_TILED = 2
+} ddf_variant_t;
+
+/* Return codes.  0 is success; hip runtime failures are reported as
+ * DDF_ERR_HIP and the text is available from ddf_hip_last_error(). */
+typedef enum {
+    DDF_OK = 0,
+    DDF_ERR_BAD_ARG = 1,      /* null pointer, non-positive size, even k ... */
+    DDF_ERR_UNSUPPORTED = 2,  /* valid request no kernel here covers          */
+    DDF_ERR_WORKSPACE = 3,    /* workspace missing or too small               */
+    DDF_ERR_HIP = 4           /* hip runtime error at launch                  */
+} ddf_status_t;
+
+/* Bits of `need_mask` for ddf_hip_backward. */
+#define DDF_NEED_DX  1u
+#define DDF_NEED_DCF 2u
+#define DDF_NEED_DSF 4u
+#define DDF_NEED_ALL 7u
+
+/* Library version: major*10000 + minor*100 + patch. */
+int ddf_hip_version(void);
+
+/* Text for a status code (static storage). */
+const char *ddf_hip_status_string(int status);
+
+/* Text of the last failure on the calling thread (thread-local storage). */
+const char *ddf_hip_last_error(void);
+
+/*
+ * Forward pass.  Replaces `forward(features, channel_filter, spatial_filter,
+ * kernel_size, dilation, stride, output)` of ddf_{mul,add}{,_faster}_ext
+ * (ddf/src/ddf_mul_ext.cpp:21-34, ddf/src/ddf_mul_faster_ext.cpp:13-26).
+ * `output` is written in full, so it need not be zeroed.
+ */
+int ddf_hip_forward(const void *features, const void *channel_filter,
+                    const void *spatial_filter, void *output,
+                    int64_t N, int64_t C, int64_t H, int64_t W,
+                    int kernel_size, int dilation, int stride,
+                    int combine, int dtype, int variant, void *stream);
+
+/*
+ * Bytes of device scratch ddf_hip_backward needs for this problem (0 when
+ * none).  Same arguments as the backward call.
+ */
+size_t ddf_hip_backward_workspace_bytes(int64_t N, int64_t C, int64_t H,
+                                        int64_t W, int kernel_size,
+                                        int dilation, int stride, int combine,
+                                        int dtype, unsigned need_mask,
+                                        int variant);
+
+/*
+ * Backward pass: gradients with respect to features, channel_filter and
+ * spatial_filter.  Replaces `backward(top_grad, features, channel_filter,
+ * spatial_filter, kernel_size, dilation, stride, rtop_grad, rbottom_grad,
+ * rspatial_filter_grad, bottom_grad, channel_filter_grad,
+ * spatial_filter_grad)` of ddf_{mul,add}_ext
+ * (ddf/src/ddf_mul_ext.cpp:36-55).  The three NHWC scratch tensors of the
+ * reference have no counterpart: gradients are produced directly in NCHW.
+ * A gradient whose bit is clear in `need_mask` is not computed and its pointer
+ * may be NULL.  Requested gradients are written in full (no zeroing needed).
+ * `workspace` must hold at least ddf_hip_backward_workspace_bytes(...) bytes,
+ * 256-byte aligned; it may be NULL when that size is 0.
+ */
+int ddf_hip_backward(const void *grad_output, const void *features,
+                     const void *channel_filter, const void *spatial_filter,
+                     void *grad_features, void *grad_channel_filter,
+                     void *grad_spatial_filter, void *workspace,
+                     size_t workspace_bytes, int64_t N, int64_t C, int64_t H,
+                     int64_t W, int kernel_size, int dilation, int stride,
+                     int combine, int dtype, unsigned need_mask, int variant,
+                     void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DDF_HIP_H */

@@ -1,0 +1,319 @@
+"""GPU parity tests: the HIP kernels, reached through the public ``ddf``
+function and the C ABI, against the CPU oracle on identical seeded inputs.
+
+Tolerances (see ddf_testlib.TOL): fp64 1e-12, fp32 1e-5, fp16 1e-2 on
+max|got-want| / max|want|.  Shapes follow the reference's own test script
+(grad_check.py:33-299) and extend it with the edge cases it leaves out."""
+import ctypes
+import itertools
+
+import pytest
+import torch
+
+import oracle
+from ddf_testlib import (TOL, check_against_oracle, random_case, rel_err, run_ddf, to_dev)
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float64, torch.float32, torch.float16]
+VERSIONS = ['', 'o']
+
+
+def _ids(v):
+    return str(v).replace('torch.', '')
+
+
+# ---------------------------------------------------------------------------
+# shapes of the reference's test script
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize('version', ['o', 'f', ''])
+@pytest.mark.parametrize('d', [1, 2])
+def test_reference_forward_check(d, version):
+    """grad_check.py:33-73: 1x10x15x15 fp64, k=3, 'mul', versions 'o' and 'f'
+    against the loop form; the reference's bound is 1e-10 absolute."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(1, 10, 15, 15, generator=g, dtype=torch.float64)
+    cf = torch.randn(1, 10, 3, 3, generator=g, dtype=torch.float64)
+    sf = torch.randn(1, 9, 15, 15, generator=g, dtype=torch.float64)
+    want = oracle.loop_forward(x, cf, sf, 3, d, 1, 'mul')
+    from ddfnet_amd import ddf
+    got = ddf(x.cuda(), cf.cuda(), sf.cuda(), 3, d, 1, 'mul', version).cpu()
+    assert (got - want).abs().max().item() <= 1e-10
+
+
+@pytest.mark.parametrize('shape', [(96, 64, 56, 56), (96, 128, 28, 28), (96, 256, 14, 14),
+                                   (96, 512, 7, 7)], ids=_ids)
+def test_reference_o_equals_f(shape):
+    """grad_check.py:77-133: version 'o' and 'f' agree to 1e-10 in fp64 at the
+    four ResNet stage shapes (batch 96)."""
+    from ddfnet_amd import ddf
+    N, C, H, W = shape
+    g = torch.Generator(device='cuda').manual_seed(5)
+    x = torch.randn(N, C, H, W, generator=g, dtype=torch.float64, device='cuda')
+    cf = torch.randn(N, C, 3, 3, generator=g, dtype=torch.float64, device='cuda')
+    sf = torch.randn(N, 9, H, W, generator=g, dtype=torch.float64, device='cuda')
+    o = ddf(x, cf, sf, 3, 1, 1, 'mul', 'o')
+    f = ddf(x, cf, sf, 3, 1, 1, 'mul', 'f')
+    assert (o - f).abs().max().item() <= 1e-10
+
+
+GRADCHECK_SHAPES = {3: [(1, 70, 10, 10), (35, 1, 10, 10), (1, 1, 50, 50)],
+                    5: [(1, 70, 10, 10), (20, 1, 10, 10), (1, 1, 40, 40)]}
+
+
+@pytest.mark.parametrize('version', VERSIONS)
+@pytest.mark.parametrize('dtype', DTYPES, ids=_ids)
+@pytest.mark.parametrize('k', [3, 5])
+def test_reference_gradcheck_shapes_vs_oracle(k, dtype, version):
+    """grad_check.py:139-299: 3 shapes x d in {1,2} x s in {1,2} x {mul,add}
+    per kernel size.  The reference differentiated numerically on the GPU; here
+    every output and gradient is compared with the oracle, whose gradients are
+    themselves pinned by numerical differentiation on the CPU."""
+    for (N, C, H, W), d, s, combine in itertools.product(
+            GRADCHECK_SHAPES[k], (1, 2), (1, 2), ('mul', 'add')):
+        case = random_case(N, C, H, W, k, s, dtype, seed=N + C + H)
+        check_against_oracle(*case, k, d, s, combine, version, what=str((N, C, H, W)))
+
+
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('k,d,s', [(3, 1, 1), (3, 2, 2), (5, 1, 2)])
+def test_numerical_gradcheck_small(k, d, s, combine):
+    """torch.autograd.gradcheck on the device with the reference's settings
+    (atol=1e-5, eps=1e-3; grad_check.py:144)."""
+    from ddfnet_amd import ddf
+    x, cf, sf, _ = random_case(2, 3, 8, 6, k, s, torch.float64, seed=11)
+    x, cf, sf = (t.cuda().requires_grad_(True) for t in (x, cf, sf))
+    assert torch.autograd.gradcheck(ddf, (x, cf, sf, k, d, s, combine), atol=1e-5, eps=1e-3)
+
+
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+def test_config1_gradcheck_scale(combine):
+    """N=2, C=16, 14x14 fp64, k=3 d=1 s=1: outputs and all three gradients
+    against the oracle, then a fast-mode numerical gradcheck."""
+    from ddfnet_amd import ddf
+    case = random_case(2, 16, 14, 14, 3, 1, torch.float64, seed=0)
+    check_against_oracle(*case, 3, 1, 1, combine)
+    x, cf, sf = (t.cuda().requires_grad_(True) for t in case[:3])
+    assert torch.autograd.gradcheck(ddf, (x, cf, sf, 3, 1, 1, combine), atol=1e-5, eps=1e-3,
+                                    fast_mode=True)
+
+
+# ---------------------------------------------------------------------------
+# edge cases the reference's script leaves out
+# ---------------------------------------------------------------------------
+EDGE = [
+    # N, C, H, W, k, d, s
+    (2, 3, 9, 11, 3, 1, 2),     # odd sizes with stride 2: floor(H/s)
+    (1, 5, 2, 2, 3, 1, 1),      # image smaller than the window
+    (1, 5, 3, 4, 5, 2, 1),      # dilated window far larger than the image
+    (2, 4, 7, 7, 1, 1, 1),      # k = 1
+    (2, 4, 9, 9, 1, 1, 2),      # k = 1, strided
+    (1, 6, 12, 12, 7, 1, 1),    # k = 7
+    (1, 3, 13, 13, 3, 3, 3),    # dilation and stride 3
+    (3, 65, 14, 14, 3, 1, 1),   # C one past a wavefront
+    (2, 130, 7, 7, 3, 1, 1),    # 7x7 plane, C not a multiple of 64
+    (1, 2, 1, 1, 3, 1, 1),      # single pixel
+    (1, 1, 1, 64, 3, 1, 1),     # single row
+    (1, 1, 64, 1, 3, 1, 1),     # single column
+    (2, 3, 20, 30, 3, 1, 1),    # W not a multiple of anything nice
+    (1, 2, 5, 200, 5, 1, 2),    # wide and short
+    (1, 2, 31, 17, 3, 2, 1),    # primes
+    (1, 8, 3, 3, 3, 1, 4),      # stride larger than the window: Ho=Wo=0
+]
+
+
+@pytest.mark.parametrize('version', VERSIONS)
+@pytest.mark.parametrize('dtype', [torch.float64, torch.float32], ids=_ids)
+@pytest.mark.parametrize('case', EDGE, ids=_ids)
+def test_edge_cases(case, dtype, version):
+    N, C, H, W, k, d, s = case
+    for combine in ('mul', 'add'):
+        tensors = random_case(N, C, H, W, k, s, dtype, seed=7)
+        check_against_oracle(*tensors, k, d, s, combine, version, what=str(case))
+
+
+def test_empty_batch_and_channels():
+    from ddfnet_amd import ddf
+    for N, C in ((0, 4), (2, 0)):
+        x = torch.zeros(N, C, 8, 8, device='cuda', requires_grad=True)
+        cf = torch.zeros(N, C, 3, 3, device='cuda', requires_grad=True)
+        sf = torch.zeros(N, 9, 8, 8, device='cuda', requires_grad=True)
+        out = ddf(x, cf, sf, 3, 1, 1, 'mul')
+        assert out.shape == (N, C, 8, 8)
+        out.sum().backward()
+        assert x.grad.shape == x.shape and cf.grad.shape == cf.shape
+        assert sf.grad.shape == sf.shape
+        if sf.grad.numel():
+            assert (sf.grad == 0).all()
+
+
+# ---------------------------------------------------------------------------
+# benchmark configurations at full size
+# ---------------------------------------------------------------------------
+FULL = {
+    'C2': (64, 256, 14, 14, 3, 1, 1, 'mul', torch.float32),
+    'C3': (64, 64, 56, 56, 3, 1, 1, 'add', torch.float16),
+    'C4a': (32, 128, 56, 56, 3, 1, 2, 'mul', torch.float32),
+    'C4b': (32, 128, 56, 56, 5, 2, 1, 'mul', torch.float32),
+}
+
+
+@pytest.mark.parametrize('version', VERSIONS)
+@pytest.mark.parametrize('name', sorted(FULL))
+def test_full_size_configs(name, version):
+    """Standardised filters, seed 0, as the benchmark draws them."""
+    N, C, H, W, k, d, s, combine, dtype = FULL[name]
+    case = random_case(N, C, H, W, k, s, dtype, seed=0, standardize=True)
+    errs = check_against_oracle(*case, k, d, s, combine, version, what=name)
+    print(name, version, errs)
+
+
+@pytest.mark.parametrize('name', sorted(FULL))
+def test_full_size_invariants(name):
+    """Size-independent properties on the device results alone.  mul is
+    trilinear: <dX,X> = <dCF,CF> = <dSF,SF> = <dO,O>; add: <dX,X> = <dO,O> and
+    <dCF,CF> + <dSF,SF> = <dO,O>."""
+    N, C, H, W, k, d, s, combine, dtype = FULL[name]
+    x, cf, sf, go = random_case(N, C, H, W, k, s, dtype, seed=1, standardize=True)
+    out, dx, dcf, dsf = run_ddf(x, cf, sf, go, k, d, s, combine)
+    dot = lambda a, b: (a.double().cpu() * b.double().cpu()).sum().item()
+    tot = dot(go, out)
+    tol = 2e-2 if dtype == torch.float16 else 1e-4
+    scale = (go.double().abs() * out.double().cpu().abs()).sum().item()
+    assert abs(dot(dx, x) - tot) <= tol * scale
+    if combine == 'mul':
+        assert abs(dot(dcf, cf) - tot) <= tol * scale
+        assert abs(dot(dsf, sf) - tot) <= tol * scale
+    else:
+        assert abs(dot(dcf, cf) + dot(dsf, sf) - tot) <= tol * scale
+
+
+def test_closed_form_depthwise_conv_on_device():
+    """mul with SF == 1 is a per-sample depthwise convolution (reference
+    README.md:49-63), here against torch's own conv2d on the device."""
+    import torch.nn.functional as F
+    from ddfnet_amd import ddf
+    N, C, H, W, k = 4, 32, 28, 28, 3
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(N, C, H, W, generator=g).cuda()
+    cf = torch.randn(N, C, k, k, generator=g).cuda()
+    sf = torch.ones(N, k * k, H, W).cuda()
+    got = ddf(x, cf, sf, k, 1, 1, 'mul')
+    want = F.conv2d(x.view(1, N * C, H, W).double(), cf.view(N * C, 1, k, k).double(),
+                    padding=1, groups=N * C).view(N, C, H, W)
+    assert rel_err(got, want.cpu()) <= 1e-5
+
+
+# ---------------------------------------------------------------------------
+# API behaviour
+# ---------------------------------------------------------------------------
+def test_needs_input_grad_subsets():
+    x, cf, sf, go = random_case(2, 6, 10, 10, 3, 1, torch.float32, seed=4)
+    full = run_ddf(x, cf, sf, go, 3, 1, 1, 'mul')
+    for need in itertools.product((False, True), repeat=3):
+        if not any(need):
+            continue
+        part = run_ddf(x, cf, sf, go, 3, 1, 1, 'mul', need=need)
+        for g_full, g_part, n in zip(full[1:], part[1:], need):
+            if n:
+                assert torch.equal(g_full, g_part)
+            else:
+                assert g_part is None
+
+
+def test_mixed_dtypes_are_promoted():
+    """fp16 features with fp32 filters: the reference widens the fp16 operand
+    (ddf/ddf.py:37-42); result is fp32."""
+    from ddfnet_amd import ddf
+    x, cf, sf, _ = random_case(2, 4, 8, 8, 3, 1, torch.float32, seed=9)
+    got = ddf(x.half().cuda(), cf.cuda(), sf.cuda(), 3, 1, 1, 'mul')
+    assert got.dtype == torch.float32
+    want = oracle.forward(x.half(), cf, sf, 3, 1, 1, 'mul')
+    assert rel_err(got, want) <= 1e-5
+
+
+def test_non_contiguous_inputs_are_accepted():
+    from ddfnet_amd import ddf
+    x, cf, sf, _ = random_case(2, 4, 8, 10, 3, 1, torch.float32, seed=10)
+    xt = x.cuda().transpose(2, 3).contiguous().transpose(2, 3)  # same values, strided
+    assert not xt.is_contiguous()
+    got = ddf(xt, cf.cuda(), sf.cuda(), 3, 1, 1, 'add')
+    assert rel_err(got, oracle.forward(x, cf, sf, 3, 1, 1, 'add')) <= 1e-5
+
+
+def test_runs_on_the_current_stream():
+    from ddfnet_amd import ddf
+    x, cf, sf, _ = random_case(4, 16, 14, 14, 3, 1, torch.float32, seed=12)
+    want = oracle.forward(x, cf, sf, 3, 1, 1, 'mul')
+    side = torch.cuda.Stream()
+    xd, cfd, sfd = to_dev(x, cf, sf)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        got = ddf(xd, cfd, sfd, 3, 1, 1, 'mul')
+    side.synchronize()
+    assert rel_err(got, want) <= 1e-5
+
+
+def test_argument_errors():
+    from ddfnet_amd import ddf, OP_DICT
+    x, cf, sf, _ = to_dev(*random_case(1, 2, 6, 6, 3, 1, torch.float32))
+    with pytest.raises(AssertionError, match='input feature must be a CUDA tensor'):
+        ddf(x.cpu(), cf, sf, 3, 1, 1, 'mul')
+    with pytest.raises(AssertionError, match='does not match kernel size'):
+        ddf(x, cf, sf, 5, 1, 1, 'mul')
+    with pytest.raises(AssertionError, match='does not match feature size'):
+        ddf(x, cf[:, :1], sf, 3, 1, 1, 'mul')
+    with pytest.raises(AssertionError, match='with stride 2'):
+        ddf(x, cf, sf, 3, 1, 2, 'mul')
+    with pytest.raises(AssertionError, match='only support mul or add'):
+        ddf(x, cf, sf, 3, 1, 1, 'max')
+    with pytest.raises(RuntimeError, match='must be contiguous'):
+        OP_DICT['mul'].forward(x.transpose(2, 3), cf, sf, 3, 1, 1, torch.empty_like(x))
+    with pytest.raises(RuntimeError, match='not implemented on CPU'):
+        OP_DICT['mul'].forward(x.cpu(), cf, sf, 3, 1, 1, torch.empty_like(x))
+    assert OP_DICT['mul_faster'].backward is None
+
+
+def test_c_abi_directly():
+    """Raw ctypes calls with device pointers: status codes and the forward
+    result, without the autograd wrapper."""
+    from ddfnet_amd import _lib
+    lib = _lib.lib()
+    x, cf, sf, go = random_case(2, 8, 14, 14, 3, 1, torch.float32, seed=13)
+    xd, cfd, sfd, god = to_dev(x, cf, sf, go)
+    out = torch.empty_like(xd)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.ddf_hip_forward(p(xd), p(cfd), p(sfd), p(out), 2, 8, 14, 14, 3, 1, 1, 0, 1, 0, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert rel_err(out, oracle.forward(x, cf, sf)) <= 1e-5
+    # even kernel size -> DDF_ERR_BAD_ARG with a message
+    rc = lib.ddf_hip_forward(p(xd), p(cfd), p(sfd), p(out), 2, 8, 14, 14, 4, 1, 1, 0, 1, 0, stream)
+    assert rc == 1 and b'kernel_size' in lib.ddf_hip_last_error()
+    # null pointer
+    rc = lib.ddf_hip_forward(None, p(cfd), p(sfd), p(out), 2, 8, 14, 14, 3, 1, 1, 0, 1, 0, stream)
+    assert rc == 1
+    # backward with workspace handling
+    need = 7
+    nbytes = lib.ddf_hip_backward_workspace_bytes(2, 8, 14, 14, 3, 1, 1, 0, 1, need, 0)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device='cuda')
+    dx, dcf, dsf = torch.empty_like(xd), torch.empty_like(cfd), torch.empty_like(sfd)
+    rc = lib.ddf_hip_backward(p(god), p(xd), p(cfd), p(sfd), p(dx), p(dcf), p(dsf), p(ws), nbytes,
+                              2, 8, 14, 14, 3, 1, 1, 0, 1, need, 0, stream)
+    assert rc == 0, lib.ddf_hip_last_error()
+    torch.cuda.synchronize()
+    for g, w in zip((dx, dcf, dsf), oracle.backward(go, x, cf, sf)):
+        assert rel_err(g, w) <= 1e-5
+    if nbytes:
+        rc = lib.ddf_hip_backward(p(god), p(xd), p(cfd), p(sfd), p(dx), p(dcf), p(dsf), None, 0,
+                                  2, 8, 14, 14, 3, 1, 1, 0, 1, need, 0, stream)
+        assert rc == 3
+
+
+def test_results_are_deterministic():
+    x, cf, sf, go = random_case(8, 64, 14, 14, 3, 1, torch.float32, seed=14, standardize=True)
+    a = run_ddf(x, cf, sf, go, 3, 1, 1, 'mul')
+    b = run_ddf(x, cf, sf, go, 3, 1, 1, 'mul')
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)

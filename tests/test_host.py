@@ -1,0 +1,134 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header
+declares, the host wrapper mirrors the reference's argument contract, and the
+stock-PyTorch modules around the operator have the reference's structure.  No
+kernel is launched here."""
+import os
+import re
+
+import pytest
+import torch
+
+import ddfnet_amd
+from ddfnet_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, 'include', 'ddf_hip.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(ddf_hip_\w+)\s*\(', text)))
+
+
+def test_library_exports_every_declared_symbol():
+    assert ddfnet_amd.is_built(), 'run `python -m ddfnet_amd.build` first'
+    lib = _lib.lib()
+    names = header_functions()
+    assert len(names) >= 6
+    for name in names:
+        assert hasattr(lib, name), name
+    assert sorted(_lib.SYMBOLS) == names
+
+
+def test_version_and_status_strings():
+    lib = _lib.lib()
+    assert lib.ddf_hip_version() >= 100
+    assert lib.ddf_hip_status_string(0) == b'ok'
+    assert b'workspace' in lib.ddf_hip_status_string(3)
+
+
+def test_argument_validation_needs_no_gpu():
+    """Bad arguments are rejected before anything touches the device."""
+    lib = _lib.lib()
+    assert lib.ddf_hip_forward(None, None, None, None, 1, 1, 4, 4, 2, 1, 1, 0, 1, 0, None) == 1
+    assert b'kernel_size' in lib.ddf_hip_last_error()
+    assert lib.ddf_hip_forward(None, None, None, None, 1, 1, 4, 4, 3, 0, 1, 0, 1, 0, None) == 1
+    assert lib.ddf_hip_forward(None, None, None, None, 1, 1, 4, 4, 3, 1, 1, 2, 1, 0, None) == 1
+    assert lib.ddf_hip_forward(None, None, None, None, 1, 1, 4, 4, 3, 1, 1, 0, 9, 0, None) == 1
+    assert lib.ddf_hip_forward(None, None, None, None, -1, 1, 4, 4, 3, 1, 1, 0, 1, 0, None) == 1
+    # empty problem: success without touching any pointer
+    assert lib.ddf_hip_forward(None, None, None, None, 0, 8, 4, 4, 3, 1, 1, 0, 1, 0, None) == 0
+    assert lib.ddf_hip_backward_workspace_bytes(1, 1, 4, 4, 2, 1, 1, 0, 1, 7, 0) == 0
+
+
+def test_ddf_rejects_cpu_tensors_like_the_reference():
+    x = torch.randn(1, 2, 4, 4)
+    with pytest.raises(AssertionError, match='input feature must be a CUDA tensor'):
+        ddfnet_amd.ddf(x, torch.randn(1, 2, 3, 3), torch.randn(1, 9, 4, 4))
+    with pytest.raises(RuntimeError, match='not implemented on CPU'):
+        ddfnet_amd.OP_DICT['mul'].forward(x, x, x, 3, 1, 1, x)
+
+
+def test_public_surface_matches_reference_package():
+    import ddf as dropin
+    for name in ('ddf', 'DDFFunction', 'DDFPack', 'DDFUpPack', 'FilterNorm',
+                 'build_spatial_branch', 'build_channel_branch', 'OP_DICT'):
+        assert getattr(dropin, name) is getattr(ddfnet_amd, name)
+    assert sorted(dropin.OP_DICT) == ['add', 'add_faster', 'mul', 'mul_faster']
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, '_lib', None)
+    monkeypatch.setattr(_lib, 'LIB_PATH', str(tmp_path / 'libddf_hip.so'))
+    with pytest.raises(_lib.DDFHipError, match='no CPU or PyTorch fallback'):
+        _lib.lib()
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, 'ddfnet_amd')
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith(('.py', '.hip', '.h', '.cpp')):
+                src = open(os.path.join(dirpath, f)).read()
+                assert 'oracle' not in src, os.path.join(dirpath, f)
+
+
+# ------------------------------- modules ----------------------------------
+def test_filter_norm_spatial_closed_form():
+    from ddfnet_amd import FilterNorm
+    fn = FilterNorm(1, 3, 'spatial', 'relu')
+    x = torch.arange(1., 10.).view(1, 9, 1, 1).double()
+    got = fn(x).view(-1)
+    std = (60.0 / 8.0) ** 0.5  # unbiased
+    gain = (2.0 ** 0.5) / 3.0  # calculate_gain('relu') / kernel_size
+    want = (torch.arange(1., 10.).double() - 5.0) / (std + 1e-10) * gain
+    assert torch.allclose(got, want, atol=1e-12)
+
+
+def test_filter_norm_channel_learned_gain_and_mean():
+    from ddfnet_amd import FilterNorm
+    torch.manual_seed(0)
+    fn = FilterNorm(4, 3, 'channel', 'linear', running_std=True, running_mean=True)
+    assert fn.std.shape == (36,) and fn.mean.shape == (36,)
+    x = torch.randn(5, 36, 1, 1)
+    got = fn(x)
+    assert got.shape == (5, 36)
+    z = x.view(5, 4, 9)
+    z = (z - z.mean(2, keepdim=True)) / (z.std(2, keepdim=True) + 1e-10)
+    want = z.reshape(5, 36) * fn.std[None] + fn.mean[None]
+    assert torch.allclose(got, want, atol=1e-6)
+
+
+@pytest.mark.parametrize('c,want', [(64, 9429), (128, 35490), (256, 137532), (512, 536175)])
+def test_ddfpack_parameter_counts(c, want):
+    """Per-pack parameter counts at se_ratio 0.2 that add up to the README's
+    16.8 M for ddf_mul_resnet50."""
+    from ddfnet_amd import DDFPack
+    assert sum(p.numel() for p in DDFPack(c).parameters()) == want
+
+
+def test_ddfpack_state_dict_names():
+    from ddfnet_amd import DDFPack
+    keys = sorted(DDFPack(16, head=2).state_dict())
+    assert keys == ['channel_branch.1.bias', 'channel_branch.1.weight',
+                    'channel_branch.3.bias', 'channel_branch.3.weight',
+                    'channel_branch.4.std', 'spatial_branch.0.bias', 'spatial_branch.0.weight']
+
+
+def test_ddfuppack_structure():
+    from ddfnet_amd import DDFUpPack
+    up = DDFUpPack(8, scale_factor=2)
+    assert len(up.spatial_branch) == 4 and len(up.channel_branch) == 4
+    assert isinstance(up.spatial_branch[0][0], torch.nn.Conv2d)  # depthwise guidance conv
+    up2 = DDFUpPack(8, scale_factor=2, joint_channels=8)
+    assert isinstance(up2.spatial_branch[0][1], ddfnet_amd.FilterNorm)
