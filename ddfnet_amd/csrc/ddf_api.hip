@@ -164,14 +164,16 @@ int ddf_hip_backward(const void *grad_output, const void *features,
     const unsigned need = need_mask & DDF_NEED_ALL;
     if (need == 0) return DDF_OK;
     const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
-    if (N * C == 0) return DDF_OK;  // every gradient is empty
-    if (!grad_output && N * C * p.Ho * p.Wo != 0)
-        return fail(DDF_ERR_BAD_ARG, "null grad_output");
-    if (!features || !channel_filter || !spatial_filter)
-        if (N * C * H * W != 0) return fail(DDF_ERR_BAD_ARG, "null input tensor pointer");
-    if (((need & DDF_NEED_DX) && !grad_features && N * C * H * W != 0) ||
-        ((need & DDF_NEED_DCF) && !grad_channel_filter) ||
-        ((need & DDF_NEED_DSF) && !grad_spatial_filter && p.Ho * p.Wo != 0))
+    if (N == 0) return DDF_OK;  // every gradient is empty
+    // A pointer is only dereferenced when its tensor has elements.
+    const int64_t n_x = N * C * H * W, n_o = N * C * p.Ho * p.Wo;
+    const int64_t n_cf = N * C * p.kk, n_sf = N * p.kk * p.Ho * p.Wo;
+    if ((!grad_output && n_o) || (!features && n_x) || (!channel_filter && n_cf) ||
+        (!spatial_filter && n_sf))
+        return fail(DDF_ERR_BAD_ARG, "null input tensor pointer");
+    if (((need & DDF_NEED_DX) && !grad_features && n_x) ||
+        ((need & DDF_NEED_DCF) && !grad_channel_filter && n_cf) ||
+        ((need & DDF_NEED_DSF) && !grad_spatial_filter && n_sf))
         return fail(DDF_ERR_BAD_ARG, "null pointer for a requested gradient");
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
