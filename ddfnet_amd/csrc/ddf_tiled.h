@@ -1,12 +1,15 @@
-// Tiled DDF kernels for gfx950 (wave64): LDS-staged input strips, spatial-filter
-// taps held in registers and reused across the channels a workgroup walks,
-// wavefront butterfly reductions for the channel-filter gradient.
+// Filter-gradient kernel of the DDF operator for gfx950 (wave64).
 //
-// All kernels work on full-width row strips of one (n, channel-range): a strip
-// of an NCHW plane is one contiguous run in memory, so every global load and
-// store is a linear, coalesced access, and only the vertical halo is re-read.
-// The strip is staged in LDS with a zero border, which makes the tap loop free
-// of bounds tests.  Included by one translation unit per element type.
+// A block of four waves works on a full-width row strip of one sample and a
+// range of its channels.  A strip of an NCHW plane is one contiguous run in
+// memory, so the global side is a linear copy: 16-byte (or 8-byte) loads of
+// the X and dO strips into LDS, a few channels ahead of use.  X lands in a
+// zero-bordered tile, which makes the tap loop free of bounds tests.  The
+// spatial-filter taps of a lane's pixels are read once into registers and
+// reused for every channel the block walks; the channel-filter taps of the
+// current channel are wavefront-uniform (scalar loads).
+//
+// Included by one translation unit per element type.
 #pragma once
 
 #include "ddf_common.h"
@@ -15,25 +18,40 @@ namespace ddf {
 
 // Geometry of one launch, computed on the host (ddf_tiled_host.hip).
 struct TileGeom {
-    int C, H, W, Ho, Wo;   // problem (per sample)
-    int rows, cols;        // grid of work cells a strip is cut from
-    int TH, nstrips;       // cell rows per strip
-    int P, IH, tile;       // LDS tile: IH rows of pitch P elements; tile = IH * P
-    int src_rows, src_cols;  // extent of the tensor staged in LDS (X or dO)
-    int row0_off;          // source row of tile row 0, for strip 0 (adds strip*TH*row_step)
-    int row_step;          // source rows advanced per cell row
-    int col_off;           // tile column of source column 0
-    int cpb, csplit, CB;   // channels per block / number of channel splits / per LDS stage
-    int threads, nwaves;
-    int lw_shift, lrows;   // loader: row width 1<<lw_shift, rows per pass
-    unsigned cols_magic;   // ceil(2^32 / cols): q / cols for q < 65536; 0 when cols == 1
-    int nblocks;           // logical blocks = N * nstrips * csplit
+    int C, H, W, Ho, Wo;     // problem (per sample)
+    int rows, cols;          // grid of work cells a strip is cut from
+    int TH, nstrips;         // cell rows per strip
+    // staged source (X, or dO for the feature gradient): zero-bordered tile
+    int src_rows, src_cols;  // extent of the source plane
+    int P, IH, tile;         // tile: IH rows of pitch P; `tile` elements per channel
+    int row0_off, col_off;   // source row of tile row 0 in strip 0; tile column of source column 0
+    // result strip staged for the store (forward, feature gradient), or the
+    // dO strip of the filter gradients: linear tile
+    int lin_tile;            // elements per channel reserved in LDS
+    int cpb, csplit;         // channels per block; number of channel splits
+    int threads;
+    int vec;                 // elements per global access when alignment allows (1 = scalar)
+    unsigned src_magic;      // ceil(2^32 / src_cols): e / src_cols for e < 65536; 0 when src_cols == 1
+    unsigned cols_magic;     // same for q / cols
+    int nblocks;             // logical blocks = N * nstrips * csplit
     int lds_bytes;
 };
 
 namespace tiled {
 
 constexpr int kXcd = 8;
+// Channels staged in LDS per barrier round.
+constexpr int kCB = 8;
+// Channels whose channel-filter taps are fetched together (scalar loads).
+constexpr int kUC = 2;
+// Waves of a filter-gradient block, and channels each owns per stage.
+constexpr int kFilterWaves = 4;
+constexpr int kPerWave = kCB / kFilterWaves;
+
+template <typename T, int V>
+struct alignas(sizeof(T) * V) Vec {
+    T e[V];
+};
 
 // Workgroups are handed to the 8 XCDs round-robin by hardware.  Renumber them
 // so that consecutive logical blocks (same sample, neighbouring channel
@@ -46,6 +64,38 @@ __device__ __forceinline__ int logical_block(int nblocks) {
 // q / g.cols for q < 65536 by multiplication; cols == 1 has no 32-bit magic.
 __device__ __forceinline__ int row_of(int q, const TileGeom &g) {
     return g.cols_magic ? (int)__umulhi((unsigned)q, g.cols_magic) : q;
+}
+
+// f / d for 0 <= f < 2^22 and d >= 1, given rcp = 1.0f / d.
+__device__ __forceinline__ int div_small(int f, int d, float rcp) {
+    int q = (int)((float)f * rcp);
+    const int r = f - q * d;
+    q += (r >= d) ? 1 : 0;
+    q -= (r < 0) ? 1 : 0;
+    return q;
+}
+
+// Channel-filter taps of the block's channels: read once with coalesced vector
+// loads into LDS as accumulator-type values (tap_pitch<KK> per channel, 16-byte
+// aligned).  The per-channel reads are then wave-uniform LDS reads that never
+// wait on global memory; a scalar load per channel would be a cold miss to
+// HBM on the critical path of every channel.
+template <int KK>
+constexpr int tap_pitch() { return (KK + 3) / 4 * 4; }
+
+template <int KK, typename T, typename A>
+__device__ __forceinline__ void stage_taps(const T *__restrict__ cf, int64_t nc0, int nch,
+                                           A *taps, int threads) {
+    for (int i = threadIdx.x; i < nch * KK; i += threads) {
+        const int c = i / KK, t = i - c * KK;
+        taps[c * tap_pitch<KK>() + t] = ld(cf + nc0 * KK + i);
+    }
+}
+
+template <int KK, typename A>
+__device__ __forceinline__ void load_taps(const A *taps, int ci, A (&w)[KK]) {
+#pragma unroll
+    for (int t = 0; t < KK; ++t) w[t] = taps[ci * tap_pitch<KK>() + t];
 }
 
 template <int CTRL>
@@ -77,7 +127,7 @@ __device__ __forceinline__ A lane_xchg(A v) {
 // Sum each of N per-lane values over the 64 lanes of the wavefront.  At every
 // stage a lane keeps one half of its values and hands the other half to its
 // partner, so the work is ~3N instructions instead of 6N.  Returns the total
-// of the value whose index bfly_index() reports for this lane.
+// of the value whose index g_bfly_table<N> lists for this lane.
 template <int N, int STAGE, typename A>
 __device__ __forceinline__ A bfly_sum(const A (&v)[N], int lane) {
     if constexpr (STAGE == 6) {
@@ -98,20 +148,32 @@ __device__ __forceinline__ A bfly_sum(const A (&v)[N], int lane) {
     }
 }
 
-template <int N, int STAGE>
-__device__ __forceinline__ int bfly_index(const int (&id)[N], int lane) {
-    if constexpr (STAGE == 6) {
-        return id[0];
-    } else {
-        constexpr int h = N / 2, M = h + (N & 1);
-        int nid[M];
-        const bool up = (lane >> STAGE) & 1;
-#pragma unroll
+// Index of the value whose total bfly_sum() leaves in `lane`: the same
+// keep/send choices replayed on indices, evaluated at compile time.
+constexpr int bfly_index_of(int n, int lane) {
+    int id[kWave] = {};
+    for (int i = 0; i < n; ++i) id[i] = i;
+    int cnt = n;
+    for (int stage = 0; stage < 6; ++stage) {
+        const int h = cnt / 2;
+        const bool up = (lane >> stage) & 1;
+        int nid[kWave] = {};
         for (int j = 0; j < h; ++j) nid[j] = up ? id[j + h] : id[j];
-        if constexpr (N & 1) nid[h] = id[2 * h];
-        return bfly_index<M, STAGE + 1>(nid, lane);
+        if (cnt & 1) nid[h] = id[2 * h];
+        cnt = h + (cnt & 1);
+        for (int j = 0; j < cnt; ++j) id[j] = nid[j];
     }
+    return id[0];
 }
+template <int N>
+struct BflyTable {
+    int tap[kWave];
+    constexpr BflyTable() : tap{} {
+        for (int l = 0; l < kWave; ++l) tap[l] = bfly_index_of(N, l);
+    }
+};
+template <int N>
+__device__ const BflyTable<N> g_bfly_table{};
 
 // Lanes below this bound hold every index at least once after the reduction.
 template <int N>
@@ -121,214 +183,137 @@ constexpr int bfly_writers() {
     return w < kWave ? w : kWave;
 }
 
-// Stage CB source planes' strips in LDS.  Thread (lrow, lcol) copies source
-// element (row0 + r, lcol) for r = lrow, lrow + lrows, ...; cells outside the
-// source stay at the zero written once at kernel start.
-template <typename T>
-__device__ __forceinline__ void stage_strips(const TileGeom &g, T *lds, const T *src_plane0,
-                                             int64_t plane_stride, int ncb, int row0) {
-    const int lw = 1 << g.lw_shift;
-    const int lcol = threadIdx.x & (lw - 1);
-    const int lrow = threadIdx.x >> g.lw_shift;
-    if (lrow >= g.lrows) return;
-    for (int cl = 0; cl < ncb; ++cl) {
-        const T *src = src_plane0 + cl * plane_stride;
-        T *dst = lds + cl * g.tile + g.col_off;
-        for (int r = lrow; r < g.IH; r += g.lrows) {
-            const int sr = row0 + r;
-            if (sr < 0 || sr >= g.src_rows) continue;
-            for (int col = lcol; col < g.src_cols; col += lw)
-                dst[r * g.P + col] = src[(int64_t)sr * g.src_cols + col];
-        }
+// Block -> (sample, strip, channel range), shared by the three kernels.
+struct BlockWork {
+    int cs, strip, row_first, nrows, np, c_begin, c_end;
+    int64_t n;
+    __device__ __forceinline__ bool init(const TileGeom &g) {
+        const int b = logical_block(g.nblocks);
+        if (b >= g.nblocks) return false;
+        cs = b % g.csplit;
+        const int rest = b / g.csplit;
+        strip = rest % g.nstrips;
+        n = rest / g.nstrips;
+        row_first = strip * g.TH;
+        nrows = min(g.TH, g.rows - row_first);
+        np = nrows * g.cols;
+        c_begin = cs * g.cpb;
+        c_end = min(g.C, c_begin + g.cpb);
+        return true;
     }
-}
-
-// ---------------------------------------------------------------------------
-// Forward.  Work cell = output pixel; threads of the block split the strip's
-// pixels, every wave walks the same channels.
-// ---------------------------------------------------------------------------
-template <typename T, int K, int D, int S, bool MUL, int PS>
-__global__ __launch_bounds__(512) void k_forward(TileGeom g, const T *__restrict__ x,
-                                                 const T *__restrict__ cf,
-                                                 const T *__restrict__ sf,
-                                                 T *__restrict__ out) {
-    using A = typename Acc<T>::type;
-    constexpr int KK = K * K, R = (K - 1) / 2;
-    extern __shared__ __align__(16) unsigned char smem[];
-    T *lds = reinterpret_cast<T *>(smem);
-
-    const int b = logical_block(g.nblocks);
-    if (b >= g.nblocks) return;
-    const int cs = b % g.csplit;
-    const int strip = (b / g.csplit) % g.nstrips;
-    const int64_t n = b / (g.csplit * g.nstrips);
-    const int y0 = strip * g.TH;
-    const int np = min(g.TH, g.rows - y0) * g.cols;
-    const int c_begin = cs * g.cpb, c_end = min(g.C, c_begin + g.cpb);
-    const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
-
-    for (int i = threadIdx.x; i < g.CB * g.tile; i += g.threads) lds[i] = T(0.0f);
-
-    int lb[PS];
-    bool ok[PS];
-    A sfr[PS][KK];
-#pragma unroll
-    for (int m = 0; m < PS; ++m) {
-        const int q = threadIdx.x + m * g.threads;
-        ok[m] = q < np;
-        const int oy = row_of(q, g);
-        const int ox = q - oy * g.cols;
-        lb[m] = ok[m] ? (oy * S) * g.P + ox * S : 0;
-        const T *sfp = sf + (n * KK * g.Ho + y0) * g.Wo + q;
-#pragma unroll
-        for (int t = 0; t < KK; ++t) sfr[m][t] = ok[m] ? (A)ld(sfp + t * oplane) : A(0);
-    }
-    const int row0 = y0 * S + g.row0_off;
-    __syncthreads();
-
-    for (int c0 = c_begin; c0 < c_end; c0 += g.CB) {
-        const int ncb = min(g.CB, c_end - c0);
-        stage_strips(g, lds, x + (n * g.C + c0) * iplane, iplane, ncb, row0);
-        __syncthreads();
-        for (int cl = 0; cl < ncb; ++cl) {
-            const int64_t nc = n * g.C + c0 + cl;
-            A w[KK];
-#pragma unroll
-            for (int t = 0; t < KK; ++t) w[t] = ld(cf + nc * KK + t);
-            const T *tl = lds + cl * g.tile;
-#pragma unroll
-            for (int m = 0; m < PS; ++m) {
-                if (!ok[m]) continue;
-                A acc = 0;
-#pragma unroll
-                for (int i = 0; i < K; ++i)
-#pragma unroll
-                    for (int j = 0; j < K; ++j)
-                        acc += (A)ld(tl + lb[m] + i * D * g.P + j * D) *
-                               comb<MUL, A>(w[i * K + j], sfr[m][i * K + j]);
-                st(out + (nc * g.Ho + y0) * g.Wo + threadIdx.x + m * g.threads, acc);
-            }
-        }
-        __syncthreads();
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Gradient with respect to the features.  Work cell (qy, qx) = the S x S block
-// of input pixels (qy*S + pu, qx*S + pv).  Input pixel row u receives tap row
-// i only when u - (i-R)*D is a multiple of S; with e = (i-R)*D that fixes the
-// phase pu = e mod S and the output row qy + (pu - e)/S, both compile-time.
-// dO is staged in LDS, the spatial filter is gathered at the neighbour
-// positions once per cell and kept in registers.
-// ---------------------------------------------------------------------------
-template <int K, int D, int S>
-struct TapMap {
-    static constexpr int R = (K - 1) / 2;
-    static constexpr int e(int i) { return (i - R) * D; }
-    static constexpr int phase(int i) { return ((e(i) % S) + S) % S; }
-    static constexpr int dq(int i) { return (phase(i) - e(i)) / S; }
-    static constexpr int halo_lo = (R * D) / S;            // cells above / left
-    static constexpr int halo_hi = (R * D + S - 1) / S;    // cells below / right
 };
 
-template <typename T, int K, int D, int S, bool MUL, int PS>
-__global__ __launch_bounds__(512) void k_backward_features(
-    TileGeom g, const T *__restrict__ go, const T *__restrict__ cf,
-    const T *__restrict__ sf, T *__restrict__ dx) {
-    using A = typename Acc<T>::type;
-    using TM = TapMap<K, D, S>;
-    constexpr int KK = K * K;
-    extern __shared__ __align__(16) unsigned char smem[];
-    T *lds = reinterpret_cast<T *>(smem);
+// Moves the strips of up to kCB consecutive planes from global memory to LDS
+// by way of registers, V elements per access.  The strips of one stage are
+// numbered as one flat list of vectors (channel-major); a thread owns vectors
+// f = tid, tid + threads, ...  The first NS of them are prefetched: issue()
+// starts their loads without waiting, commit() writes them to LDS later and
+// moves any further vectors straight through.  Issuing stage s+1 before
+// computing on stage s overlaps the fetch with the arithmetic.
+//
+// The destination is either a zero-bordered tile (PADDED: row pitch P, column
+// offset col_off, first staged row at tile row row_shift) or a linear copy of
+// the run.  Requires src_cols >= V for PADDED (one row crossing per vector).
+template <typename T, int V, int NS, bool PADDED>
+struct Stager {
+    int nvec, run0, row_shift, dst_tile, src_cols, P, col_off, threads;
+    unsigned src_magic;
+    float rcp_nvec;
+    int cl[NS], eoff[NS], lo[NS], col[NS];
+    Vec<T, V> v[NS];
 
-    const int b = logical_block(g.nblocks);
-    if (b >= g.nblocks) return;
-    const int cs = b % g.csplit;
-    const int strip = (b / g.csplit) % g.nstrips;
-    const int64_t n = b / (g.csplit * g.nstrips);
-    const int qy0 = strip * g.TH;
-    const int np = min(g.TH, g.rows - qy0) * g.cols;
-    const int c_begin = cs * g.cpb, c_end = min(g.C, c_begin + g.cpb);
-    const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
-
-    for (int i = threadIdx.x; i < g.CB * g.tile; i += g.threads) lds[i] = T(0.0f);
-
-    int lb[PS], cy[PS], cx[PS];
-    bool ok[PS];
-    A sfg[PS][KK];
-#pragma unroll
-    for (int m = 0; m < PS; ++m) {
-        const int q = threadIdx.x + m * g.threads;
-        ok[m] = q < np;
-        const int ql = row_of(q, g);
-        cy[m] = qy0 + ql;
-        cx[m] = q - ql * g.cols;
-        lb[m] = ok[m] ? ql * g.P + cx[m] : 0;
-#pragma unroll
-        for (int i = 0; i < K; ++i)
-#pragma unroll
-            for (int j = 0; j < K; ++j) {
-                const int sy = cy[m] + TM::dq(i), sx = cx[m] + TM::dq(j);
-                const bool in = ok[m] && sy >= 0 && sy < g.Ho && sx >= 0 && sx < g.Wo;
-                sfg[m][i * K + j] =
-                    in ? (A)ld(sf + ((n * KK + i * K + j) * g.Ho + sy) * g.Wo + sx) : A(0);
-            }
-    }
-    const int row0 = qy0 + g.row0_off;
-    __syncthreads();
-
-    for (int c0 = c_begin; c0 < c_end; c0 += g.CB) {
-        const int ncb = min(g.CB, c_end - c0);
-        stage_strips(g, lds, go + (n * g.C + c0) * oplane, oplane, ncb, row0);
-        __syncthreads();
-        for (int cl = 0; cl < ncb; ++cl) {
-            const int64_t nc = n * g.C + c0 + cl;
-            A w[KK];
-#pragma unroll
-            for (int t = 0; t < KK; ++t) w[t] = ld(cf + nc * KK + t);
-            const T *tl = lds + cl * g.tile;
-#pragma unroll
-            for (int m = 0; m < PS; ++m) {
-                if (!ok[m]) continue;
-                A acc[S][S];
-#pragma unroll
-                for (int a = 0; a < S; ++a)
-#pragma unroll
-                    for (int c = 0; c < S; ++c) acc[a][c] = 0;
-#pragma unroll
-                for (int i = 0; i < K; ++i)
-#pragma unroll
-                    for (int j = 0; j < K; ++j) {
-                        const A gv = ld(tl + lb[m] + (TM::dq(i) + TM::halo_lo) * g.P +
-                                        TM::dq(j) + TM::halo_lo);
-                        acc[TM::phase(i)][TM::phase(j)] +=
-                            gv * comb<MUL, A>(w[i * K + j], sfg[m][i * K + j]);
-                    }
-                T *dst = dx + nc * iplane;
-#pragma unroll
-                for (int a = 0; a < S; ++a)
-#pragma unroll
-                    for (int c = 0; c < S; ++c) {
-                        const int u = cy[m] * S + a, v = cx[m] * S + c;
-                        if (u < g.H && v < g.W) st(dst + (int64_t)u * g.W + v, acc[a][c]);
-                    }
-            }
+    __device__ __forceinline__ void locate(int f, int &c, int &eo, int &l, int &cc) const {
+        c = div_small(f, nvec, rcp_nvec);
+        const int e = (f - c * nvec) * V;
+        eo = run0 + e;
+        if (PADDED) {
+            const int row = src_magic ? (int)__umulhi((unsigned)e, src_magic) : e;
+            cc = e - row * src_cols;
+            l = c * dst_tile + (row_shift + row) * P + col_off + cc;
+        } else {
+            cc = 0;
+            l = c * dst_tile + e;
         }
-        __syncthreads();
     }
+    // n_elems elements per channel starting at element run_start of each plane.
+    __device__ __forceinline__ void init(int n_elems, int run_start, int row_shift_, int dst_tile_,
+                                         int src_cols_, int P_, int col_off_, unsigned magic,
+                                         int threads_) {
+        nvec = n_elems / V;
+        run0 = run_start;
+        row_shift = row_shift_;
+        dst_tile = dst_tile_;
+        src_cols = src_cols_;
+        P = P_;
+        col_off = col_off_;
+        src_magic = magic;
+        threads = threads_;
+        rcp_nvec = 1.0f / (float)max(nvec, 1);
+#pragma unroll
+        for (int j = 0; j < NS; ++j)
+            locate(threadIdx.x + j * threads, cl[j], eoff[j], lo[j], col[j]);
+    }
+    __device__ __forceinline__ void put(T *lds, int l, int cc, const Vec<T, V> &val) const {
+        if (!PADDED) {
+            *reinterpret_cast<Vec<T, V> *>(lds + l) = val;
+        } else {
+#pragma unroll
+            for (int k = 0; k < V; ++k)
+                lds[l + k + ((cc + k >= src_cols) ? P - src_cols : 0)] = val.e[k];
+        }
+    }
+    __device__ __forceinline__ void issue(const T *__restrict__ src, int64_t plane, int ncb) {
+#pragma unroll
+        for (int j = 0; j < NS; ++j)
+            if (cl[j] < ncb)
+                v[j] = *reinterpret_cast<const Vec<T, V> *>(src + cl[j] * plane + eoff[j]);
+    }
+    // `src`, `plane`, `ncb` as given to the matching issue().
+    __device__ __forceinline__ void commit(T *lds, const T *__restrict__ src, int64_t plane,
+                                           int ncb) const {
+#pragma unroll
+        for (int j = 0; j < NS; ++j)
+            if (cl[j] < ncb) put(lds, lo[j], col[j], v[j]);
+        const int total = ncb * nvec;
+        for (int f = threadIdx.x + NS * threads; f < total; f += threads) {
+            int c, eo, l, cc;
+            locate(f, c, eo, l, cc);
+            put(lds, l, cc, *reinterpret_cast<const Vec<T, V> *>(src + c * plane + eo));
+        }
+    }
+};
+
+// Prefetch depth: 16-byte accesses keep 3 vectors in flight per thread,
+// 8-byte ones 4, scalar ones 8.
+template <typename T, int V>
+constexpr int stager_slots() {
+    return sizeof(T) * V >= 16 ? 3 : (V > 1 ? 4 : 8);
+}
+
+template <typename T>
+__device__ __forceinline__ void zero_tiles(const TileGeom &g, T *lds) {
+    for (int i = threadIdx.x; i < kCB * g.tile; i += g.threads) lds[i] = T(0.0f);
+}
+
+// First staged source row, clipped, and how many rows of the strip exist.
+__device__ __forceinline__ void clip_rows(const TileGeom &g, int row0, int &r_lo, int &n_rows) {
+    r_lo = max(row0, 0);
+    n_rows = max(min(row0 + g.IH, g.src_rows) - r_lo, 0);
 }
 
 // ---------------------------------------------------------------------------
 // Gradients with respect to both filters.  Work cell = output pixel, owned by
-// a lane (PS pixels per lane); the waves of a block take different channels.
-// Per channel a lane forms gx[t] = dO * X_t once and feeds it to both sums:
+// a lane (PS pixels per lane); the four waves of a block take different
+// channels.  Per channel a lane forms gx[t] = dO * X_t once and feeds it to
+// both sums:
 //   dSF[t, pixel] += gx[t] * CF[c, t]   (register accumulator, over channels)
 //   dCF[c, t]     += gx[t] * SF[t, pixel]  (butterfly over the wave's lanes)
 // Partial sums over channel splits (dSF) and strips (dCF) go to the workspace
 // and are added up by k_sum_partials; no atomics, so results are reproducible.
+// LDS: kCB zero-bordered X tiles, then kCB linear dO strips.
 // ---------------------------------------------------------------------------
-template <typename T, int K, int D, int S, bool MUL, int PS>
-__global__ __launch_bounds__(512) void k_backward_filters(
+template <typename T, int K, int D, int S, bool MUL, int PS, int V>
+__global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     TileGeom g, const T *__restrict__ go, const T *__restrict__ x,
     const T *__restrict__ cf, const T *__restrict__ sf, T *__restrict__ dcf,
     T *__restrict__ dsf, typename Acc<T>::type *__restrict__ ws_sf,
@@ -336,26 +321,17 @@ __global__ __launch_bounds__(512) void k_backward_filters(
     using A = typename Acc<T>::type;
     constexpr int KK = K * K;
     extern __shared__ __align__(16) unsigned char smem[];
-    T *lds = reinterpret_cast<T *>(smem);
+    T *lds_in = reinterpret_cast<T *>(smem);
+    T *lds_go = lds_in + kCB * g.tile;
+    A *taps = reinterpret_cast<A *>(lds_go + kCB * g.lin_tile);
 
-    const int b = logical_block(g.nblocks);
-    if (b >= g.nblocks) return;
-    const int cs = b % g.csplit;
-    const int strip = (b / g.csplit) % g.nstrips;
-    const int64_t n = b / (g.csplit * g.nstrips);
-    const int y0 = strip * g.TH;
-    const int np = min(g.TH, g.rows - y0) * g.cols;
-    const int c_begin = cs * g.cpb, c_end = min(g.C, c_begin + g.cpb);
+    BlockWork bw;
+    if (!bw.init(g)) return;
     const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
+    const int y0 = bw.row_first;
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const bool want_cf = need & DDF_NEED_DCF, want_sf = need & DDF_NEED_DSF;
-
-    for (int i = threadIdx.x; i < g.CB * g.tile; i += g.threads) lds[i] = T(0.0f);
-
-    int ids[KK];
-#pragma unroll
-    for (int t = 0; t < KK; ++t) ids[t] = t;
-    const int my_tap = bfly_index<KK, 0>(ids, lane);
+    const int my_tap = g_bfly_table<KK>.tap[lane];
 
     int lb[PS];
     bool ok[PS];
@@ -363,44 +339,68 @@ __global__ __launch_bounds__(512) void k_backward_filters(
 #pragma unroll
     for (int m = 0; m < PS; ++m) {
         const int q = lane + m * kWave;
-        ok[m] = q < np;
+        ok[m] = q < bw.np;
         const int oy = row_of(q, g);
         const int ox = q - oy * g.cols;
         lb[m] = ok[m] ? (oy * S) * g.P + ox * S : 0;
-        const T *sfp = sf + (n * KK * g.Ho + y0) * g.Wo + q;
+        const T *sfp = sf + (bw.n * KK * g.Ho + y0) * g.Wo + q;
 #pragma unroll
         for (int t = 0; t < KK; ++t) {
             sfr[m][t] = (MUL && ok[m]) ? (A)ld(sfp + t * oplane) : A(0);
             acc_sf[m][t] = 0;
         }
     }
-    const int row0 = y0 * S + g.row0_off;
+
+    int r_lo, n_rows;
+    clip_rows(g, y0 * S + g.row0_off, r_lo, n_rows);
+    Stager<T, V, stager_slots<T, V>(), true> stg;
+    stg.init(n_rows * g.src_cols, r_lo * g.src_cols, r_lo - (y0 * S + g.row0_off), g.tile,
+             g.src_cols, g.P, g.col_off, g.src_magic, g.threads);
+    Stager<T, V, (stager_slots<T, V>() + 1) / 2, false> stg_go;
+    stg_go.init(bw.np, y0 * g.Wo, 0, g.lin_tile, g.Wo, g.Wo, 0, 0u, g.threads);
+    const T *xs = x + (bw.n * g.C + bw.c_begin) * iplane;
+    const T *gs = go + (bw.n * g.C + bw.c_begin) * oplane;
+    {
+        const int ncb = min(kCB, bw.c_end - bw.c_begin);
+        stg.issue(xs, iplane, ncb);
+        stg_go.issue(gs, oplane, ncb);
+    }
+    if (MUL) stage_taps<KK>(cf, bw.n * g.C + bw.c_begin, bw.c_end - bw.c_begin, taps, g.threads);
+    zero_tiles(g, lds_in);
     __syncthreads();
 
-    for (int c0 = c_begin; c0 < c_end; c0 += g.CB) {
-        const int ncb = min(g.CB, c_end - c0);
-        stage_strips(g, lds, x + (n * g.C + c0) * iplane, iplane, ncb, row0);
+    for (int c0 = bw.c_begin; c0 < bw.c_end; c0 += kCB, xs += kCB * iplane, gs += kCB * oplane) {
+        const int ncb = min(kCB, bw.c_end - c0);
+        stg.commit(lds_in, xs, iplane, ncb);
+        stg_go.commit(lds_go, gs, oplane, ncb);
         __syncthreads();
-        for (int cl = wave; cl < ncb; cl += g.nwaves) {
-            const int64_t nc = n * g.C + c0 + cl;
-            A w[KK];
+        if (c0 + kCB < bw.c_end) {
+            const int nnext = min(kCB, bw.c_end - c0 - kCB);
+            stg.issue(xs + kCB * iplane, iplane, nnext);
+            stg_go.issue(gs + kCB * oplane, oplane, nnext);
+        }
 #pragma unroll
-            for (int t = 0; t < KK; ++t) w[t] = MUL ? (A)ld(cf + nc * KK + t) : A(1);
-            const T *tl = lds + cl * g.tile;
-            const T *gp = go + (nc * g.Ho + y0) * g.Wo + lane;
+        for (int u = 0; u < kPerWave; ++u) {
+            const int cl = wave + u * kFilterWaves;
+            if (cl >= ncb) break;
+            const int64_t nc = bw.n * g.C + c0 + cl;
+            A w[KK];
+            if (MUL) load_taps<KK>(taps, c0 - bw.c_begin + cl, w);
+            const T *tl = lds_in + cl * g.tile;
+            const T *gl = lds_go + cl * g.lin_tile + lane;
             A pcf[KK];
 #pragma unroll
             for (int t = 0; t < KK; ++t) pcf[t] = 0;
 #pragma unroll
             for (int m = 0; m < PS; ++m) {
                 if (!ok[m]) continue;
-                const A gv = ld(gp + m * kWave);
+                const A gval = ld(gl + m * kWave);
 #pragma unroll
                 for (int i = 0; i < K; ++i)
 #pragma unroll
                     for (int j = 0; j < K; ++j) {
                         const int t = i * K + j;
-                        const A gx = gv * (A)ld(tl + lb[m] + i * D * g.P + j * D);
+                        const A gx = gval * (A)ld(tl + lb[m] + i * D * g.P + j * D);
                         if (MUL) {
                             acc_sf[m][t] += gx * w[t];
                             pcf[t] += gx * sfr[m][t];
@@ -414,7 +414,7 @@ __global__ __launch_bounds__(512) void k_backward_filters(
                 const A tot = bfly_sum<KK, 0, A>(pcf, lane);
                 if (lane < bfly_writers<KK>()) {
                     if (g.nstrips == 1) st(dcf + nc * KK + my_tap, tot);
-                    else ws_cf[(nc * g.nstrips + strip) * KK + my_tap] = tot;
+                    else ws_cf[(nc * g.nstrips + bw.strip) * KK + my_tap] = tot;
                 }
             }
         }
@@ -422,20 +422,7 @@ __global__ __launch_bounds__(512) void k_backward_filters(
     }
 
     if (!want_sf) return;
-    if (g.nwaves == 1) {
-#pragma unroll
-        for (int m = 0; m < PS; ++m) {
-            if (!ok[m]) continue;
-            const int64_t pix = (int64_t)y0 * g.Wo + lane + m * kWave;
-#pragma unroll
-            for (int t = 0; t < KK; ++t) {
-                if (g.csplit == 1) st(dsf + (n * KK + t) * oplane + pix, acc_sf[m][t]);
-                else ws_sf[((n * g.csplit + cs) * KK + t) * oplane + pix] = acc_sf[m][t];
-            }
-        }
-        return;
-    }
-    // Add the waves' dSF accumulators: one slot at a time through LDS.
+    // Add the four waves' dSF accumulators: one pixel slot at a time through LDS.
     A *red = reinterpret_cast<A *>(smem);
 #pragma unroll
     for (int m = 0; m < PS; ++m) {
@@ -443,12 +430,13 @@ __global__ __launch_bounds__(512) void k_backward_filters(
         for (int t = 0; t < KK; ++t) red[(wave * KK + t) * kWave + lane] = acc_sf[m][t];
         __syncthreads();
         const int64_t pix = (int64_t)y0 * g.Wo + lane + m * kWave;
-        for (int t = wave; t < KK; t += g.nwaves) {
+        for (int t = wave; t < KK; t += kFilterWaves) {
             A tot = 0;
-            for (int wv = 0; wv < g.nwaves; ++wv) tot += red[(wv * KK + t) * kWave + lane];
+#pragma unroll
+            for (int wv = 0; wv < kFilterWaves; ++wv) tot += red[(wv * KK + t) * kWave + lane];
             if (ok[m]) {
-                if (g.csplit == 1) st(dsf + (n * KK + t) * oplane + pix, tot);
-                else ws_sf[((n * g.csplit + cs) * KK + t) * oplane + pix] = tot;
+                if (g.csplit == 1) st(dsf + (bw.n * KK + t) * oplane + pix, tot);
+                else ws_sf[((bw.n * g.csplit + bw.cs) * KK + t) * oplane + pix] = tot;
             }
         }
         __syncthreads();
@@ -472,7 +460,7 @@ __global__ __launch_bounds__(256) void k_sum_partials(
 }  // namespace tiled
 
 // Host-side geometry (ddf_tiled_host.hip).
-enum TiledKind { kKindForward = 0, kKindFeatures = 1, kKindFilters = 2 };
+enum TiledKind { kKindFilters = 2 };
 bool tiled_geometry(const Problem &p, int dtype, int kind, TileGeom *g, int *ps);
 bool tiled_shape_instantiated(int k, int d, int s);
 

@@ -4,6 +4,7 @@
 #include <cstdlib>
 
 #include "ddf_tiled.h"
+#include "ddf_wave.h"
 
 namespace ddf {
 
@@ -28,7 +29,8 @@ bool tiled_shape_instantiated(int k, int d, int s) {
 }
 
 // Fills *g and *ps for one kernel kind; false when the tiled family does not
-// cover the problem (the caller then uses the generic kernels).
+// cover the problem (the caller then uses the generic kernels).  *ps is the
+// number of pixels a lane owns in the filter-gradient kernel (1 otherwise).
 bool tiled_geometry(const Problem &p, int dtype, int kind, TileGeom *g, int *ps_out) {
     if (!tiled_shape_instantiated(p.k, p.d, p.s)) return false;
     if (p.N <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0) return false;
@@ -36,57 +38,70 @@ bool tiled_geometry(const Problem &p, int dtype, int kind, TileGeom *g, int *ps_
     const int esz = elem_size(dtype), asz = acc_size(dtype);
     const int K = p.k, D = p.d, S = p.s, R = p.r, KK = p.kk;
     const int H = (int)p.H, W = (int)p.W, Ho = (int)p.Ho, Wo = (int)p.Wo, C = (int)p.C;
+    const bool per_lane = (kind == kKindFilters);
 
     TileGeom t{};
     t.C = C; t.H = H; t.W = W; t.Ho = Ho; t.Wo = Wo;
-    int halo_lo = 0, halo_hi = 0;
-    if (kind == kKindFeatures) {
-        halo_lo = (R * D) / S;
-        halo_hi = (R * D + S - 1) / S;
-        t.rows = (H + S - 1) / S; t.cols = (W + S - 1) / S;
-        t.src_rows = Ho; t.src_cols = Wo;
-        t.P = t.cols + halo_lo + halo_hi;
-        t.col_off = halo_lo; t.row0_off = -halo_lo; t.row_step = 1;
-    } else {
+    int lin_cols;          // elements per row of the linear tile
+    int lin_rows_per_cell; // rows of it per cell row
+    {
         t.rows = Ho; t.cols = Wo;
         t.src_rows = H; t.src_cols = W;
         t.P = std::max((Wo - 1) * S + (K - 1) * D + 1, R * D + W);
-        t.col_off = R * D; t.row0_off = -R * D; t.row_step = S;
+        t.col_off = R * D; t.row0_off = -R * D;
+        lin_cols = Wo; lin_rows_per_cell = 1;     // the out strip, or the dO strip
     }
     auto tile_rows = [&](int th) {
-        return kind == kKindFeatures ? th + halo_lo + halo_hi : (th - 1) * S + (K - 1) * D + 1;
+        return (th - 1) * S + (K - 1) * D + 1;
     };
 
-    // Pixels (cells) one block pass can own.
-    const bool per_lane = (kind == kKindFilters);
-    const int max_ps = per_lane ? 4 : 2;
-    const int capacity = per_lane ? kWave * max_ps : kMaxThreads * max_ps;
-    if (t.cols > capacity || t.cols >= 65536) return false;
-    if (tile_rows(1) * t.P * esz > kLdsBudget) return false;
+    // Widest aligned global access: 16 bytes, else 8, else one element.  Every
+    // plane and every strip start must be a multiple of it, and a vector may
+    // cross at most one row end of the padded tile.
+    const int64_t plane_in = (int64_t)t.src_rows * t.src_cols;
+    const int64_t plane_lin = (int64_t)Ho * Wo;
+    auto vec_ok = [&](int v, int nstrips) {
+        if (v == 1) return true;
+        if (plane_in % v || plane_lin % v || t.src_cols < v) return false;
+        if (per_lane && ((int64_t)H * W) % v) return false;
+        return nstrips == 1 || (t.src_cols % v == 0 && lin_cols % v == 0);
+    };
+    const int forced_vec = env_int("DDF_TUNE_VEC", 0);
 
-    // Strip height and pixels per thread: minimise an instruction estimate per
-    // strip set.  Compute costs ~2*KK (3*KK for the filter gradients) per
-    // owned pixel slot, idle lanes included; staging costs ~4 per tile element;
-    // the filter-gradient kernel adds one butterfly (~3*KK) per wave pass.
+    // Cells one block pass can own.
+    const int max_ps = per_lane ? (KK > 9 ? 2 : 4) : 1;
+    const int min_ps = per_lane ? 2 : 1;
+    const int capacity = per_lane ? kWave * max_ps : kMaxThreads;
+    if (t.cols > capacity || t.cols >= 65536 || t.src_cols >= 65536) return false;
+
+    // Strip height (and pixels per lane): minimise an instruction estimate.
+    // Compute costs ~2*KK (3*KK for the filter gradients) per owned cell slot,
+    // idle lanes included; staging costs ~4 per tile element; the
+    // filter-gradient kernel adds one butterfly (~3*KK) per wave pass.
     const int c_comp = (per_lane ? 3 : 2) * KK, c_load = 4, c_red = 3 * KK;
     double best = 1e30;
     int best_th = 0, best_ps = 0;
     const int forced_th = env_int(per_lane ? "DDF_TUNE_TH_FILTERS" : "DDF_TUNE_TH", 0);
-    const int forced_ps = env_int(per_lane ? "DDF_TUNE_PS_FILTERS" : "DDF_TUNE_PS", 0);
+    const int forced_ps = env_int("DDF_TUNE_PS_FILTERS", 0);
+    auto threads_for = [&](int np) {
+        return per_lane ? kWave * tiled::kFilterWaves : round_up(np, kWave);
+    };
     for (int th = 1; th <= t.rows; ++th) {
         const int np = th * t.cols;
         if (np > capacity) break;
-        if (tile_rows(th) * t.P * esz > kLdsBudget) break;
         if (forced_th && th != std::min(forced_th, t.rows)) continue;
         const int nstrips = (t.rows + th - 1) / th;
-        for (int ps = 1; ps <= max_ps; ps *= 2) {
-            if (forced_ps && ps != forced_ps) continue;
-            const int lanes = per_lane ? kWave : kMaxThreads;
-            if (np > lanes * ps) continue;
-            const int slots = per_lane ? kWave * ps : round_up((np + ps - 1) / ps, kWave) * ps;
+        const int64_t lds = (int64_t)tiled::kCB * esz *
+                            (tile_rows(th) * t.P + round_up(th * lin_rows_per_cell * lin_cols, 8));
+        if (lds > kLdsBudget || tile_rows(th) * t.src_cols >= 65536) break;
+        for (int ps = min_ps; ps <= max_ps; ps *= 2) {
+            if (per_lane && forced_ps && ps != forced_ps) continue;
+            if (per_lane && np > kWave * ps) continue;
+            const int slots = per_lane ? kWave * ps : threads_for(np);
             double cost = (double)nstrips *
                           (slots * c_comp + (double)tile_rows(th) * t.P * c_load +
                            (per_lane ? c_red : 0));
+            if (!vec_ok(16 / esz, nstrips)) cost *= vec_ok(8 / esz, nstrips) ? 1.1 : 1.5;
             cost *= 1.0 + 0.02 * ps;  // mild preference for fewer registers
             if (cost < best) { best = cost; best_th = th; best_ps = ps; }
         }
@@ -96,68 +111,204 @@ bool tiled_geometry(const Problem &p, int dtype, int kind, TileGeom *g, int *ps_
     t.nstrips = (t.rows + t.TH - 1) / t.TH;
     t.IH = tile_rows(t.TH);
     t.tile = t.IH * t.P;
-    const int ps = best_ps;
-    const int np = t.TH * t.cols;
-
-    if (per_lane) {
-        t.nwaves = std::max(1, std::min(env_int("DDF_TUNE_WAVES_FILTERS", 4), C));
-        t.threads = kWave * t.nwaves;
-    } else {
-        t.threads = round_up((np + ps - 1) / ps, kWave);
-        t.nwaves = t.threads / kWave;
-    }
+    t.lin_tile = round_up(t.TH * lin_rows_per_cell * lin_cols, 8);
+    t.threads = threads_for(t.TH * t.cols);
+    t.vec = 1;
+    for (int bytes = 16; bytes >= 2 * esz && dtype != DDF_F64; bytes /= 2)
+        if (vec_ok(bytes / esz, t.nstrips)) { t.vec = bytes / esz; break; }
+    if (forced_vec) t.vec = std::min(t.vec, forced_vec);
 
     // Channels per block: enough blocks to fill 256 CUs several times over, but
     // long enough channel walks to amortise the spatial-filter registers.
     const int64_t base = p.N * t.nstrips;
     const int target = env_int(per_lane ? "DDF_TUNE_BLOCKS_FILTERS" : "DDF_TUNE_BLOCKS",
                                per_lane ? 1024 : 2048) * 256 / t.threads;
-    int min_cpb = per_lane ? 4 * t.nwaves : 8;
-    int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
-    int cpb = (int)std::max<int64_t>(min_cpb, (C + want_split - 1) / want_split);
+    const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
+    int cpb = (int)((C + want_split - 1) / want_split);
     const int forced_cpb = env_int(per_lane ? "DDF_TUNE_CPB_FILTERS" : "DDF_TUNE_CPB", 0);
     if (forced_cpb) cpb = forced_cpb;
-    if (per_lane) cpb = round_up(cpb, t.nwaves);
-    cpb = std::min(cpb, per_lane ? round_up(C, t.nwaves) : C);
+    cpb = std::min(round_up(std::max(cpb, 1), tiled::kCB), round_up(C, tiled::kCB));
+    cpb = std::min(cpb, 256);
     t.cpb = cpb;
     t.csplit = (C + cpb - 1) / cpb;
 
-    int cb = env_int("DDF_TUNE_CB", 8);
-    if (per_lane) cb = round_up(cb, t.nwaves);
-    cb = std::min(cb, cpb);
-    while (cb > 1 && cb * t.tile * esz > kLdsBudget) cb = per_lane ? cb - t.nwaves : cb - 1;
-    if (cb < 1 || cb * t.tile * esz > kLdsBudget) return false;
-    if (per_lane && cb % t.nwaves != 0 && cb != cpb) {
-        // fewer channels per stage than waves: shrink the block instead
-        t.nwaves = cb; t.threads = kWave * cb;
-    }
-    t.CB = cb;
-    t.lds_bytes = cb * t.tile * esz;
-    if (per_lane) t.lds_bytes = std::max(t.lds_bytes, t.nwaves * KK * kWave * asz);
+    // tiles, then the channel-filter taps of the block's channels (accumulator type)
+    t.lds_bytes = tiled::kCB * (t.tile + t.lin_tile) * esz + cpb * ((KK + 3) / 4 * 4) * asz;
+    if (per_lane)
+        t.lds_bytes = std::max(t.lds_bytes, tiled::kFilterWaves * KK * kWave * asz);
     if (t.lds_bytes > 64 * 1024) return false;
 
-    // Loader: rows of 2^lw_shift lanes, as many rows per pass as the block has.
-    int lw_shift = 0;
-    while ((1 << lw_shift) < t.src_cols && (2 << lw_shift) <= t.threads) ++lw_shift;
-    t.lw_shift = lw_shift;
-    t.lrows = t.threads >> lw_shift;
+    t.src_magic = t.src_cols == 1 ? 0u : (unsigned)((0x100000000ull + t.src_cols - 1) / t.src_cols);
     t.cols_magic = t.cols == 1 ? 0u : (unsigned)((0x100000000ull + t.cols - 1) / t.cols);
     const int64_t nblocks = base * t.csplit;
     if (nblocks > (1 << 30)) return false;
     t.nblocks = (int)nblocks;
     *g = t;
-    *ps_out = ps;
+    *ps_out = per_lane ? best_ps : 1;
+    return true;
+}
+
+// Geometry of the wavefront-per-strip kernels (forward, feature gradient).
+// *ps_out / *nv_out name the instantiation: cell slots per lane and source
+// vectors per lane per channel.
+bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom *g, int *ps_out,
+                   int *nv_out) {
+    if (!tiled_shape_instantiated(p.k, p.d, p.s)) return false;
+    if (p.N <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0) return false;
+    if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
+    const int esz = elem_size(dtype);
+    const int K = p.k, D = p.d, S = p.s, R = p.r;
+    const int H = (int)p.H, W = (int)p.W, Ho = (int)p.Ho, Wo = (int)p.Wo, C = (int)p.C;
+
+    WaveGeom t{};
+    t.C = C; t.H = H; t.W = W; t.Ho = Ho; t.Wo = Wo;
+    int halo_lo = 0, halo_hi = 0;
+    if (kind == kWaveFeatures) {
+        halo_lo = (R * D) / S;
+        halo_hi = (R * D + S - 1) / S;
+        t.rows = (H + S - 1) / S; t.cols = (W + S - 1) / S;
+        t.src_rows = Ho; t.src_cols = Wo;
+        t.P = t.cols + halo_lo + halo_hi;
+        t.col_off = halo_lo; t.row0_off = -halo_lo;
+        t.lin_cols = W; t.lin_rpc = S; t.lin_rows = H;
+    } else {
+        t.rows = Ho; t.cols = Wo;
+        t.src_rows = H; t.src_cols = W;
+        t.P = std::max((Wo - 1) * S + (K - 1) * D + 1, R * D + W);
+        t.col_off = R * D; t.row0_off = -R * D;
+        t.lin_cols = Wo; t.lin_rpc = 1; t.lin_rows = Ho;
+    }
+    auto tile_rows = [&](int th) {
+        return kind == kWaveFeatures ? th + halo_lo + halo_hi : (th - 1) * S + (K - 1) * D + 1;
+    };
+
+    // lanes: LW per cell row segment, 64 / LW cell rows per slot
+    int lw_shift = 0;
+    while ((1 << lw_shift) < std::min(t.cols, kWave)) ++lw_shift;
+    const int LW = 1 << lw_shift, RS = kWave / LW;
+    const int cseg = (t.cols + LW - 1) / LW;
+    if (cseg > kMaxSlots) return false;
+    t.lw_shift = lw_shift;
+
+    // Every strip's source run and result run must start and end on a vector
+    // boundary for V-element accesses.
+    const int64_t plane_in = (int64_t)t.src_rows * t.src_cols;
+    const int64_t plane_lin = (int64_t)t.lin_rows * t.lin_cols;
+    auto vec_ok = [&](int v, int th) {
+        if (v == 1) return true;
+        if (plane_in % v || plane_lin % v || t.src_cols < v) return false;
+        for (int first = 0; first < t.rows; first += th) {
+            const int nrows = std::min(th, t.rows - first);
+            const int row0 = (kind == kWaveFeatures ? first : first * S) + t.row0_off;
+            const int r_lo = std::max(row0, 0);
+            const int n_rows = std::max(std::min(row0 + tile_rows(th), t.src_rows) - r_lo, 0);
+            if (((int64_t)r_lo * t.src_cols) % v || ((int64_t)n_rows * t.src_cols) % v) return false;
+            const int l0 = first * t.lin_rpc;
+            const int ln = std::min(nrows * t.lin_rpc, t.lin_rows - l0);
+            if (((int64_t)l0 * t.lin_cols) % v || ((int64_t)ln * t.lin_cols) % v) return false;
+        }
+        return true;
+    };
+    const int forced_vec = env_int("DDF_TUNE_VEC", 0);
+    const int forced_ps = env_int("DDF_TUNE_PS", 0);
+
+    // Candidates: 4 or 8 slots per lane.  Cost ~ slots walked (idle lanes
+    // included) plus the halo rows re-staged per strip.
+    double best = 1e30;
+    int best_ps = 0, best_th = 0, best_v = 0, best_nv = 0;
+    for (int ps = 4; ps <= kMaxSlots; ps *= 2) {
+        if (forced_ps && ps != forced_ps) continue;
+        if (ps < cseg) continue;
+        int th = (ps / cseg) * RS;
+        th = std::min(th, t.rows);
+        const int forced_th = env_int("DDF_TUNE_TH", 0);
+        if (forced_th) th = std::min(th, forced_th);
+        const int nstrips = (t.rows + th - 1) / th;
+        int v = 1;
+        if (dtype != DDF_F64 && vec_ok(4, th)) v = 4;
+        if (forced_vec) v = std::min(v, forced_vec);
+        if (max_vec) v = std::min(v, max_vec);
+        const int staged = std::min(tile_rows(th), t.src_rows) * t.src_cols;
+        const int need_nv = (staged + v * kWave - 1) / (v * kWave);
+        int nv = 0;
+        for (int cand : {1, 2, 4, 8})
+            if (cand >= need_nv) { nv = cand; break; }
+        // instantiated: V=4 with (ps 4: nv 1, 2, 4; ps 8: nv 4); V=1 with (ps 4: nv 4, 8)
+        if (nv == 0) continue;
+        if (v == 4) {
+            if (nv == 8) continue;
+            if (ps == 8) nv = 4;
+        } else {
+            if (ps == 8) continue;
+            nv = std::max(nv, 4);
+        }
+        const int64_t lds = (int64_t)esz * (2 * round_up(tile_rows(th) * t.P, 8) + 2 * wave::kSpare +
+                                            round_up(th * t.lin_rpc * t.lin_cols, 8)) + 4096;
+        if (lds > 64 * 1024) continue;
+        const int slots_used = ((th + RS - 1) / RS) * cseg;
+        double cost = (double)nstrips * (slots_used * kWave * 2.0 * p.kk +
+                                         (double)tile_rows(th) * t.P * 3.0 + 150.0);
+        if (v == 1) cost *= 1.3;
+        if (ps == 8) cost *= 1.05;  // register pressure
+        if (cost < best) { best = cost; best_ps = ps; best_th = th; best_v = v; best_nv = nv; }
+    }
+    if (best_ps == 0) return false;
+    t.TH = best_th;
+    t.nstrips = (t.rows + t.TH - 1) / t.TH;
+    t.nslots = ((t.TH + RS - 1) / RS) * cseg;
+    for (int m = 0; m < kMaxSlots; ++m) {
+        t.slot_row[m] = m < t.nslots ? (m / cseg) * RS : 0;
+        t.slot_col[m] = m < t.nslots ? (m % cseg) * LW : 0;
+    }
+    t.IH = tile_rows(t.TH);
+    {
+        // farthest element any lane (idle ones included) reads: last slot row,
+        // last lane column, last tap
+        const int step = kind == kWaveFeatures ? 1 : S;
+        const int last_row = (t.slot_row[t.nslots - 1] + RS - 1) * step;
+        const int last_col = (t.slot_col[t.nslots - 1] + LW - 1) * step;
+        const int reach = kind == kWaveFeatures ? halo_lo + halo_hi : (K - 1) * D;
+        const int extent = (last_row + reach) * t.P + last_col + reach + 1;
+        t.tile = round_up(std::max(t.IH * t.P, extent), 8);
+    }
+    t.lin_tile = round_up(t.TH * t.lin_rpc * t.lin_cols, 8);
+    t.vec = best_v;
+    t.nv = best_nv;
+
+    // Channels per wave: enough waves to fill the machine several times over,
+    // long enough walks to amortise the spatial-filter registers.
+    const int64_t base = p.N * t.nstrips;
+    const int target = env_int("DDF_TUNE_WAVES", 4096);
+    const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
+    int cpw = (int)((C + want_split - 1) / want_split);
+    cpw = std::max(cpw, std::min(C, env_int("DDF_TUNE_MIN_CPW", 4)));
+    cpw = std::min(cpw, std::max(1, wave::kTapLoads * kWave / p.kk));  // taps staged in one go
+    const int forced_cpw = env_int("DDF_TUNE_CPW", 0);
+    if (forced_cpw) cpw = std::min(forced_cpw, C);
+    t.cpw = cpw;
+    t.csplit = (C + cpw - 1) / cpw;
+    // tiles, then the channel-filter taps of the wave's channels (accumulator type)
+    t.lds_bytes = (t.tile + t.lin_tile + 2 * wave::kSpare) * esz +
+                  cpw * ((p.kk + 3) / 4 * 4) * acc_size(dtype);
+    if (t.lds_bytes > 64 * 1024) return false;
+    t.src_magic = t.src_cols == 1 ? 0u : (unsigned)((0x100000000ull + t.src_cols - 1) / t.src_cols);
+    const int64_t nblocks = base * t.csplit;
+    if (nblocks > (1 << 30)) return false;
+    t.nblocks = (int)nblocks;
+    *g = t;
+    *ps_out = best_ps;
+    *nv_out = best_nv;
     return true;
 }
 
 bool tiled_forward_supported(const Problem &p, int dtype) {
-    TileGeom g; int ps;
-    return tiled_geometry(p, dtype, kKindForward, &g, &ps);
+    WaveGeom g; int ps, nv;
+    return wave_geometry(p, dtype, kWaveForward, 0, &g, &ps, &nv);
 }
 
 bool tiled_backward_supported(const Problem &p, int dtype) {
-    TileGeom g; int ps;
-    return tiled_geometry(p, dtype, kKindFeatures, &g, &ps) &&
+    WaveGeom w; TileGeom g; int ps, nv;
+    return wave_geometry(p, dtype, kWaveFeatures, 0, &w, &ps, &nv) &&
            tiled_geometry(p, dtype, kKindFilters, &g, &ps);
 }
 

@@ -1,7 +1,12 @@
 // Launch code of the tiled kernels, instantiated once per element type.
 #pragma once
 
+#include <initializer_list>
+
+#include <type_traits>
+
 #include "ddf_tiled.h"
+#include "ddf_wave.h"
 
 namespace ddf {
 namespace tiled {
@@ -25,29 +30,77 @@ inline unsigned padded_grid(int nblocks) { return (unsigned)((nblocks + kXcd - 1
         }                                                                  \
     } while (0)
 
-template <typename T, int K, int D, int S, int PS>
-hipError_t launch_forward(const Problem &p, const TileGeom &g, const T *x, const T *cf,
-                          const T *sf, T *out, hipStream_t st) {
-    const dim3 grid(padded_grid(g.nblocks)), block(g.threads);
-    if (p.mul)
-        hipLaunchKernelGGL((k_forward<T, K, D, S, true, PS>), grid, block, g.lds_bytes, st, g, x,
-                           cf, sf, out);
-    else
-        hipLaunchKernelGGL((k_forward<T, K, D, S, false, PS>), grid, block, g.lds_bytes, st, g,
-                           x, cf, sf, out);
+// Elements per global access: the geometry's choice, unless a pointer is not
+// aligned to it.
+template <typename T>
+inline int usable_vec(const TileGeom &g, std::initializer_list<const void *> ptrs) {
+    int v = g.vec;
+    for (const void *p : ptrs)
+        while (v > 1 && (reinterpret_cast<uintptr_t>(p) % (v * sizeof(T))) != 0) v /= 2;
+    return v;
+}
+
+// The wide access (16 bytes), the narrow one (8 bytes) or single elements.
+template <typename T> constexpr int wide_vec() { return sizeof(T) == 8 ? 1 : 16 / sizeof(T); }
+template <typename T> constexpr int narrow_vec() { return sizeof(T) == 8 ? 1 : 8 / sizeof(T); }
+
+#define DDF_DISPATCH_VEC(T, v, ...)                                                  \
+    do {                                                                             \
+        if (sizeof(T) != 8 && (v) == wide_vec<T>()) { constexpr int VV_ = wide_vec<T>(); __VA_ARGS__; } \
+        else if (sizeof(T) != 8 && (v) == narrow_vec<T>()) { constexpr int VV_ = narrow_vec<T>(); __VA_ARGS__; } \
+        else { constexpr int VV_ = 1; __VA_ARGS__; }                                 \
+    } while (0)
+
+// Largest power-of-two vector <= v to which every pointer is aligned.
+template <typename T>
+inline bool aligned_for(int v, std::initializer_list<const void *> ptrs) {
+    for (const void *p : ptrs)
+        if (reinterpret_cast<uintptr_t>(p) % (v * sizeof(T)) != 0) return false;
+    return true;
+}
+
+// Instantiated (PS, NV, V) of the wave kernels: V=4 with (4,1) (4,2) (4,4)
+// (8,4); V=1 with (4,4) (4,8).
+#define DDF_DISPATCH_WAVE(ps, nv, v, ...)                                              \
+    do {                                                                               \
+        if ((v) == 4 && (ps) == 4 && (nv) == 1) { constexpr int PS_ = 4, NV_ = 1, VV_ = 4; __VA_ARGS__; } \
+        else if ((v) == 4 && (ps) == 4 && (nv) == 2) { constexpr int PS_ = 4, NV_ = 2, VV_ = 4; __VA_ARGS__; } \
+        else if ((v) == 4 && (ps) == 4 && (nv) == 4) { constexpr int PS_ = 4, NV_ = 4, VV_ = 4; __VA_ARGS__; } \
+        else if ((v) == 4 && (ps) == 8 && (nv) == 4) { constexpr int PS_ = 8, NV_ = 4, VV_ = 4; __VA_ARGS__; } \
+        else if ((v) == 1 && (ps) == 4 && (nv) == 4) { constexpr int PS_ = 4, NV_ = 4, VV_ = 1; __VA_ARGS__; } \
+        else if ((v) == 1 && (ps) == 4 && (nv) == 8) { constexpr int PS_ = 4, NV_ = 8, VV_ = 1; __VA_ARGS__; } \
+        else return hipErrorNotSupported;                                              \
+    } while (0)
+
+template <typename T, int K, int D, int S>
+hipError_t launch_forward(const Problem &p, const WaveGeom &g, int ps, int nv, const T *x,
+                          const T *cf, const T *sf, T *out, hipStream_t st) {
+    const dim3 grid(padded_grid(g.nblocks)), block(kWave);
+    DDF_DISPATCH_WAVE(ps, nv, g.vec, {
+        if constexpr (sizeof(T) == 8 && VV_ != 1) return hipErrorNotSupported;
+        else if (p.mul)
+            hipLaunchKernelGGL((wave::k_forward<T, K, D, S, true, PS_, NV_, VV_>), grid, block,
+                               g.lds_bytes, st, g, x, cf, sf, out);
+        else
+            hipLaunchKernelGGL((wave::k_forward<T, K, D, S, false, PS_, NV_, VV_>), grid, block,
+                               g.lds_bytes, st, g, x, cf, sf, out);
+    });
     return hipGetLastError();
 }
 
-template <typename T, int K, int D, int S, int PS>
-hipError_t launch_features(const Problem &p, const TileGeom &g, const T *go, const T *cf,
-                           const T *sf, T *dx, hipStream_t st) {
-    const dim3 grid(padded_grid(g.nblocks)), block(g.threads);
-    if (p.mul)
-        hipLaunchKernelGGL((k_backward_features<T, K, D, S, true, PS>), grid, block, g.lds_bytes,
-                           st, g, go, cf, sf, dx);
-    else
-        hipLaunchKernelGGL((k_backward_features<T, K, D, S, false, PS>), grid, block,
-                           g.lds_bytes, st, g, go, cf, sf, dx);
+template <typename T, int K, int D, int S>
+hipError_t launch_features(const Problem &p, const WaveGeom &g, int ps, int nv, const T *go,
+                           const T *cf, const T *sf, T *dx, hipStream_t st) {
+    const dim3 grid(padded_grid(g.nblocks)), block(kWave);
+    DDF_DISPATCH_WAVE(ps, nv, g.vec, {
+        if constexpr (sizeof(T) == 8 && VV_ != 1) return hipErrorNotSupported;
+        else if (p.mul)
+            hipLaunchKernelGGL((wave::k_backward_features<T, K, D, S, true, PS_, NV_, VV_>), grid,
+                               block, g.lds_bytes, st, g, go, cf, sf, dx);
+        else
+            hipLaunchKernelGGL((wave::k_backward_features<T, K, D, S, false, PS_, NV_, VV_>), grid,
+                               block, g.lds_bytes, st, g, go, cf, sf, dx);
+    });
     return hipGetLastError();
 }
 
@@ -57,27 +110,38 @@ hipError_t launch_filters(const Problem &p, const TileGeom &g, const T *go, cons
                           typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                           unsigned need, hipStream_t st) {
     const dim3 grid(padded_grid(g.nblocks)), block(g.threads);
-    if (p.mul)
-        hipLaunchKernelGGL((k_backward_filters<T, K, D, S, true, PS>), grid, block, g.lds_bytes,
-                           st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
-    else
-        hipLaunchKernelGGL((k_backward_filters<T, K, D, S, false, PS>), grid, block, g.lds_bytes,
-                           st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
+    const int v = usable_vec<T>(g, {go, x});
+    DDF_DISPATCH_VEC(T, v, {
+        if (p.mul)
+            hipLaunchKernelGGL((k_backward_filters<T, K, D, S, true, PS, VV_>), grid, block,
+                               g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
+        else
+            hipLaunchKernelGGL((k_backward_filters<T, K, D, S, false, PS, VV_>), grid, block,
+                               g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
+    });
     return hipGetLastError();
 }
 
 }  // namespace tiled
 
+// A misaligned pointer sends the problem down the scalar-access geometry
+// (same kernels, one element per access).
+template <typename T>
+bool wave_plan(const Problem &p, int kind, std::initializer_list<const void *> ptrs, WaveGeom *g,
+               int *ps, int *nv) {
+    const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
+    if (!wave_geometry(p, dtype, kind, 0, g, ps, nv)) return false;
+    if (g->vec > 1 && !tiled::aligned_for<T>(g->vec, ptrs))
+        return wave_geometry(p, dtype, kind, 1, g, ps, nv);
+    return true;
+}
+
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf, T *out,
                          hipStream_t st) {
-    TileGeom g; int ps;
-    const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
-    if (!tiled_geometry(p, dtype, kKindForward, &g, &ps)) return hipErrorNotSupported;
-    DDF_DISPATCH_KDS(p, do {
-        if (ps == 1) return tiled::launch_forward<T, KK_, DD_, SS_, 1>(p, g, x, cf, sf, out, st);
-        return tiled::launch_forward<T, KK_, DD_, SS_, 2>(p, g, x, cf, sf, out, st);
-    } while (0));
+    WaveGeom g; int ps, nv;
+    if (!wave_plan<T>(p, kWaveForward, {x, out}, &g, &ps, &nv)) return hipErrorNotSupported;
+    DDF_DISPATCH_KDS(p, return tiled::launch_forward<T, KK_, DD_, SS_>(p, g, ps, nv, x, cf, sf, out, st));
     return hipErrorNotSupported;
 }
 
@@ -88,13 +152,9 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
     hipError_t err = hipSuccess;
     if (need & DDF_NEED_DX) {
-        TileGeom g; int ps;
-        if (!tiled_geometry(p, dtype, kKindFeatures, &g, &ps)) return hipErrorNotSupported;
-        DDF_DISPATCH_KDS(p, do {
-            err = ps == 1
-                ? tiled::launch_features<T, KK_, DD_, SS_, 1>(p, g, go, cf, sf, dx, st)
-                : tiled::launch_features<T, KK_, DD_, SS_, 2>(p, g, go, cf, sf, dx, st);
-        } while (0));
+        WaveGeom g; int ps, nv;
+        if (!wave_plan<T>(p, kWaveFeatures, {go, dx}, &g, &ps, &nv)) return hipErrorNotSupported;
+        DDF_DISPATCH_KDS(p, err = tiled::launch_features<T, KK_, DD_, SS_>(p, g, ps, nv, go, cf, sf, dx, st));
         if (err != hipSuccess) return err;
     }
     const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
@@ -111,10 +171,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
         }
         if ((fneed & DDF_NEED_DCF) && g.nstrips > 1) ws_cf = reinterpret_cast<A *>(wp);
         DDF_DISPATCH_KDS(p, do {
-            if (ps == 1)
-                err = tiled::launch_filters<T, KK_, DD_, SS_, 1>(p, g, go, x, cf, sf, dcf, dsf,
-                                                                 ws_sf, ws_cf, fneed, st);
-            else if (ps == 2)
+            if (ps == 2)
                 err = tiled::launch_filters<T, KK_, DD_, SS_, 2>(p, g, go, x, cf, sf, dcf, dsf,
                                                                  ws_sf, ws_cf, fneed, st);
             else

@@ -1,0 +1,475 @@
+// Wavefront-per-strip DDF kernels for gfx950: forward and feature gradient.
+//
+// One 64-lane wavefront (a workgroup of its own) owns a full-width row strip of
+// one sample and walks a range of its channels.  Lanes are laid out 2-D over
+// the strip's work cells - LW = 2^k >= cols lanes per cell row, 64/LW cell rows
+// per pass ("slot"), PS slots per lane - so that LDS addresses are linear in
+// the lane id (no bank conflicts) and no division is needed to find a cell.
+//
+// Per channel the wave
+//   1. copies the source strip (X, or dO for the feature gradient) from global
+//      memory with 16-byte loads, a few channels ahead of use, and scatters it
+//      into a zero-bordered LDS tile (the border makes the tap loop free of
+//      bounds tests),
+//   2. runs the tap loop for its PS cells out of LDS, with the spatial-filter
+//      taps of those cells held in registers for the whole channel walk and
+//      the channel-filter taps of the current channel in scalar registers,
+//   3. writes the results to a linear LDS copy of the result strip and stores
+//      that with 16-byte accesses.
+// The global side is therefore a plain linear copy in both directions, and a
+// wave never waits for another wave: there is no workgroup barrier at all.
+#pragma once
+
+#include <type_traits>
+
+#include "ddf_common.h"
+
+namespace ddf {
+
+constexpr int kMaxSlots = 8;
+
+struct WaveGeom {
+    int C, H, W, Ho, Wo;      // problem (per sample)
+    int rows, cols;           // grid of work cells a strip is cut from
+    int lw_shift;             // lanes per cell row segment = 1 << lw_shift
+    int TH, nstrips;          // cell rows per strip
+    int nslots;               // slots in use (<= PS of the kernel launched)
+    // staged source plane (X, or dO for the feature gradient) and its zero-bordered tile
+    int src_rows, src_cols;
+    int P, IH, tile;          // tile: IH rows of pitch P elements, `tile` elements reserved
+    int row0_off, col_off;    // source row of tile row 0 in strip 0; tile column of source column 0
+    // result strip (out, or dX): `lin_cols` elements per row, `lin_rpc` rows per cell row
+    int lin_cols, lin_rpc, lin_rows, lin_tile;
+    int cpw, csplit;          // channels per wave; number of channel ranges
+    int vec, nv;              // elements per global access; vectors per lane per channel strip
+    unsigned src_magic;       // ceil(2^32 / src_cols); 0 when src_cols == 1
+    int nblocks;              // = N * nstrips * csplit
+    int lds_bytes;
+    int slot_row[kMaxSlots];  // cell row (within the strip) of lane row 0 in slot m
+    int slot_col[kMaxSlots];  // cell column of lane column 0 in slot m
+};
+
+namespace wave {
+
+constexpr int kXcd = 8;
+// Spare LDS elements behind each tile: idle lanes write there instead of branching.
+constexpr int kSpare = 8;
+
+template <typename T, int V>
+struct alignas(sizeof(T) * V) Vec {
+    T e[V];
+};
+
+// Compiler-level ordering point between LDS writes and the reads of other
+// lanes of the same wavefront.  The LDS unit executes one wave's instructions
+// in order, so no hardware wait is needed.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroups are handed to the 8 XCDs round-robin by hardware.  Renumber them
+// so that consecutive logical blocks (same sample, neighbouring channel
+// ranges: same spatial filter) share an XCD and its L2.
+__device__ __forceinline__ int logical_block(int nblocks) {
+    const int per = (nblocks + kXcd - 1) / kXcd;
+    return (int)(blockIdx.x % kXcd) * per + (int)(blockIdx.x / kXcd);
+}
+
+struct WaveWork {
+    int cs, strip, row_first, nrows, c_begin, c_end;
+    int64_t n;
+    __device__ __forceinline__ bool init(const WaveGeom &g) {
+        const int b = logical_block(g.nblocks);
+        if (b >= g.nblocks) return false;
+        cs = b % g.csplit;
+        const int rest = b / g.csplit;
+        strip = rest % g.nstrips;
+        n = rest / g.nstrips;
+        row_first = strip * g.TH;
+        nrows = min(g.TH, g.rows - row_first);
+        c_begin = cs * g.cpw;
+        c_end = min(g.C, c_begin + g.cpw);
+        return true;
+    }
+};
+
+// Channel-filter taps of the wave's channels.  Read once, with one coalesced
+// vector load, into LDS as accumulator-type values (kTapPitch<KK> per channel,
+// 16-byte aligned); the per-channel reads are then wave-uniform LDS reads that
+// never wait on global memory.  (A scalar load per channel would be a cold
+// miss to HBM on the critical path of every channel.)
+template <int KK>
+constexpr int tap_pitch() { return (KK + 3) / 4 * 4; }
+
+// Loads of at most kTapLoads * 64 tap values start here, before anything
+// waits; put() writes them to LDS later.  The host keeps cpw * KK within that.
+constexpr int kTapLoads = 4;
+template <int KK, typename T, typename A>
+struct TapStager {
+    T v[kTapLoads];
+    __device__ __forceinline__ void issue(const T *__restrict__ cf, int64_t nc0, int nch,
+                                          int lane) {
+        const T *src = cf + nc0 * KK;
+#pragma unroll
+        for (int r = 0; r < kTapLoads; ++r) {
+            const int i = lane + r * kWave;
+            v[r] = src[min(i, nch * KK - 1)];      // clamped: no branch
+        }
+    }
+    __device__ __forceinline__ void put(A *taps, int nch, int lane) const {
+#pragma unroll
+        for (int r = 0; r < kTapLoads; ++r) {
+            const int i = lane + r * kWave;
+            const int c = i / KK, t = i - c * KK;
+            if (i < nch * KK) taps[c * tap_pitch<KK>() + t] = ld(&v[r]);
+        }
+    }
+};
+
+template <int KK, typename A>
+__device__ __forceinline__ void load_taps(const A *taps, int ci, A (&w)[KK]) {
+#pragma unroll
+    for (int t = 0; t < KK; ++t) w[t] = taps[ci * tap_pitch<KK>() + t];
+}
+
+// Channels in flight per wave for a given number of vectors per channel.
+template <int NV>
+constexpr int stages() { return NV <= 1 ? 4 : (NV <= 2 ? 2 : 1); }
+
+// Source strip -> zero-bordered LDS tile, through registers.  The strip of one
+// channel is a run of n_in contiguous elements; lane l owns vectors
+// f = l, l + 64, ... of it.  Their tile offsets are computed once.
+template <typename T, int V, int NV>
+struct Stager {
+    static constexpr int NST = stages<NV>();
+    int goff[NV];        // element offset of the vector inside a source plane
+    int lo[NV][V];       // tile offset of each element
+    Vec<T, V> v[NST][NV];
+
+    // Lanes without a vector load plane element 0 and write to the spare cell
+    // behind the tile, so that neither issue() nor commit() branches: the
+    // compiler then counts outstanding loads exactly and a commit waits only
+    // for its own stage.
+    __device__ __forceinline__ void init(const WaveGeom &g, int row0, int lane) {
+        const int r_lo = max(row0, 0);
+        const int n_rows = max(min(row0 + g.IH, g.src_rows) - r_lo, 0);
+        const int nvec = n_rows * g.src_cols / V;
+        const int row_shift = r_lo - row0;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int f = lane + j * kWave;
+            const int e = f * V;
+            int row = g.src_magic ? (int)__umulhi((unsigned)e, g.src_magic) : e;
+            int col = e - row * g.src_cols;
+            const bool used = f < nvec;
+            goff[j] = used ? r_lo * g.src_cols + e : 0;
+#pragma unroll
+            for (int k = 0; k < V; ++k) {
+                lo[j][k] = used ? (row_shift + row) * g.P + g.col_off + col : g.tile + k;
+                if (++col >= g.src_cols) { col = 0; ++row; }
+            }
+        }
+    }
+    template <int ST>
+    __device__ __forceinline__ void issue(const T *__restrict__ plane) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+            v[ST][j] = *reinterpret_cast<const Vec<T, V> *>(plane + goff[j]);
+    }
+    template <int ST>
+    __device__ __forceinline__ void commit(T *lds) const {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+#pragma unroll
+            for (int k = 0; k < V; ++k) lds[lo[j][k]] = v[ST][j].e[k];
+    }
+};
+
+// Linear LDS strip -> global memory, V elements per access.
+template <typename T, int V>
+__device__ __forceinline__ void store_strip(const T *lds, T *__restrict__ dst, int n_elems,
+                                            int lane) {
+    const int nvec = n_elems / V;
+    for (int f = lane; f < nvec; f += kWave)
+        *reinterpret_cast<Vec<T, V> *>(dst + f * V) =
+            *reinterpret_cast<const Vec<T, V> *>(lds + f * V);
+}
+
+template <typename T>
+__device__ __forceinline__ void zero_tile(T *lds, int n, int lane) {
+    // `n` is a multiple of 8 elements and the tile is 16-byte aligned
+    constexpr int W16 = 16 / sizeof(T);
+    Vec<T, W16> z;
+#pragma unroll
+    for (int k = 0; k < W16; ++k) z.e[k] = T(0.0f);
+    for (int i = lane * W16; i < n; i += kWave * W16) *reinterpret_cast<Vec<T, W16> *>(lds + i) = z;
+}
+
+// ---------------------------------------------------------------------------
+// Forward: work cell = output pixel.
+// ---------------------------------------------------------------------------
+template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V>
+__global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restrict__ x,
+                                                   const T *__restrict__ cf,
+                                                   const T *__restrict__ sf,
+                                                   T *__restrict__ out) {
+    using A = typename Acc<T>::type;
+    constexpr int KK = K * K;
+    using Stg = Stager<T, V, NV>;
+    constexpr int NST = Stg::NST;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *lds_in = reinterpret_cast<T *>(smem);
+    T *lds_out = lds_in + g.tile + kSpare;
+    A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kSpare);
+
+    WaveWork ww;
+    if (!ww.init(g)) return;
+    const int lane = threadIdx.x;
+    const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
+    const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
+    const int y0 = ww.row_first;
+    // every load of the prologue is issued before the first wait: the wave pays
+    // one trip to memory, not one per tensor
+    TapStager<KK, T, A> tst;
+    tst.issue(cf, ww.n * g.C + ww.c_begin, ww.c_end - ww.c_begin, lane);
+    const int n_out = ww.nrows * g.Wo;
+
+    // per slot: is the cell real, where its taps start in the tile, where its
+    // result goes in the linear strip; its spatial-filter taps in registers
+    bool ok[PS];
+    int lb[PS], ob[PS];
+    A sfr[PS][KK];
+#pragma unroll
+    for (int m = 0; m < PS; ++m) {
+        const int row = g.slot_row[m] + lr, col = g.slot_col[m] + lc;
+        ok[m] = m < g.nslots && row < ww.nrows && col < g.cols;
+        // idle lanes keep their lane-linear tile address (inside the LDS
+        // allocation): a shared dummy address would collide with the banks of
+        // the working lanes and double the time of every tap read
+        lb[m] = (row * S) * g.P + col * S;
+        ob[m] = ok[m] ? row * g.Wo + col : 0;
+        // idle lanes read pixel 0 of the strip: no branch around the loads
+        const T *sfp = sf + (ww.n * KK * g.Ho + y0) * g.Wo + ob[m];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) sfr[m][t] = ld(sfp + t * oplane);
+    }
+
+    Stg stg;
+    stg.init(g, y0 * S + g.row0_off, lane);
+    const T *xs = x + (ww.n * g.C + ww.c_begin) * iplane;
+    T *os = out + (ww.n * g.C + ww.c_begin) * oplane + (int64_t)y0 * g.Wo;
+    const int nch = ww.c_end - ww.c_begin;
+    // start the first NST channels' loads (clamped to the last channel, so that
+    // they are unconditional), then clear the tile under them
+    stg.template issue<0>(xs);
+    if constexpr (NST > 1) stg.template issue<1>(xs + (int64_t)min(1, nch - 1) * iplane);
+    if constexpr (NST > 2) stg.template issue<2>(xs + (int64_t)min(2, nch - 1) * iplane);
+    if constexpr (NST > 3) stg.template issue<3>(xs + (int64_t)min(3, nch - 1) * iplane);
+    zero_tile(lds_in, g.tile, lane);
+    tst.put(taps, nch, lane);
+    wave_sync();
+
+    auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        stg.template commit<ST>(lds_in);
+        stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch - 1) * iplane);
+        wave_sync();
+        A w[KK];
+        load_taps<KK>(taps, ci, w);
+#pragma unroll
+        for (int m = 0; m < PS; ++m) {
+            if (m >= g.nslots) break;
+            A acc = 0;
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j)
+                    acc += (A)ld(lds_in + lb[m] + i * D * g.P + j * D) *
+                           comb<MUL, A>(w[i * K + j], sfr[m][i * K + j]);
+            if (ok[m]) st(lds_out + ob[m], acc);
+        }
+        wave_sync();
+        store_strip<T, V>(lds_out, os + (int64_t)ci * oplane, n_out, lane);
+        wave_sync();
+    };
+
+    auto group = [&](int c) __attribute__((always_inline)) {
+        channel(std::integral_constant<int, 0>{}, c);
+        if constexpr (NST > 1) channel(std::integral_constant<int, 1>{}, c + 1);
+        if constexpr (NST > 2) channel(std::integral_constant<int, 2>{}, c + 2);
+        if constexpr (NST > 3) channel(std::integral_constant<int, 3>{}, c + 3);
+    };
+    // The first group is peeled off the loop: the loop is then entered only in
+    // its steady state (NST loads and NST stores in flight), and the wait the
+    // compiler places before a commit covers that stage's load alone instead
+    // of draining the younger loads and stores as well.
+    const int nfull = nch / NST * NST;
+    if (nfull > 0) {
+        group(0);
+        for (int c = NST; c < nfull; c += NST) group(c);
+    }
+    if constexpr (NST > 1) {
+        // the last nch % NST channels already sit in stages 0, 1, ...
+        if (nfull < nch) channel(std::integral_constant<int, 0>{}, nfull);
+        if constexpr (NST > 2) {
+            if (nfull + 1 < nch) channel(std::integral_constant<int, 1>{}, nfull + 1);
+            if (nfull + 2 < nch) channel(std::integral_constant<int, 2>{}, nfull + 2);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Gradient with respect to the features.  Work cell (qy, qx) = the S x S block
+// of input pixels (qy*S + pu, qx*S + pv).  Input pixel row u receives tap row
+// i only when u - (i-R)*D is a multiple of S; with e = (i-R)*D that fixes the
+// phase pu = e mod S and the output row qy + (pu - e)/S, both compile-time.
+// dO is staged in the zero-bordered tile, the spatial filter is gathered at
+// the neighbour positions once per cell and kept in registers, and the S*S
+// results of a cell go to the linear copy of the dX strip.
+// ---------------------------------------------------------------------------
+template <int K, int D, int S>
+struct TapMap {
+    static constexpr int R = (K - 1) / 2;
+    static constexpr int e(int i) { return (i - R) * D; }
+    static constexpr int phase(int i) { return ((e(i) % S) + S) % S; }
+    static constexpr int dq(int i) { return (phase(i) - e(i)) / S; }
+    static constexpr int halo_lo = (R * D) / S;            // cells above / left
+    static constexpr int halo_hi = (R * D + S - 1) / S;    // cells below / right
+};
+
+template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V>
+__global__ __launch_bounds__(kWave) void k_backward_features(
+    WaveGeom g, const T *__restrict__ go, const T *__restrict__ cf,
+    const T *__restrict__ sf, T *__restrict__ dx) {
+    using A = typename Acc<T>::type;
+    using TM = TapMap<K, D, S>;
+    constexpr int KK = K * K;
+    using Stg = Stager<T, V, NV>;
+    constexpr int NST = Stg::NST;
+    extern __shared__ __align__(16) unsigned char smem[];
+    T *lds_in = reinterpret_cast<T *>(smem);
+    T *lds_out = lds_in + g.tile + kSpare;
+    A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kSpare);
+
+    WaveWork ww;
+    if (!ww.init(g)) return;
+    const int lane = threadIdx.x;
+    const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
+    const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
+    const int qy0 = ww.row_first;
+    TapStager<KK, T, A> tst;
+    tst.issue(cf, ww.n * g.C + ww.c_begin, ww.c_end - ww.c_begin, lane);
+    const int u0 = qy0 * S;                                     // first dX row of the strip
+    const int n_out = min(ww.nrows * S, g.H - u0) * g.W;        // its element count
+
+    bool ok[PS];
+    int lb[PS], ob[PS], cu[PS], cv[PS];
+    A sfg[PS][KK];
+#pragma unroll
+    for (int m = 0; m < PS; ++m) {
+        const int ql = g.slot_row[m] + lr, cx = g.slot_col[m] + lc;
+        const int cy = qy0 + ql;
+        ok[m] = m < g.nslots && ql < ww.nrows && cx < g.cols;
+        lb[m] = ql * g.P + cx;   // idle lanes keep a lane-linear (bank-conflict-free) address
+        ob[m] = ok[m] ? (ql * S) * g.W + cx * S : 0;
+        // idle cells get coordinates outside the image: none of their results is kept
+        cu[m] = ok[m] ? cy * S : g.H;
+        cv[m] = cx * S;
+#pragma unroll
+        for (int i = 0; i < K; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                const int sy = cy + TM::dq(i), sx = cx + TM::dq(j);
+                const bool in = ok[m] && sy >= 0 && sy < g.Ho && sx >= 0 && sx < g.Wo;
+                // out-of-range neighbours read element 0 and are zeroed: no branch
+                const A val = ld(sf + (ww.n * KK + i * K + j) * oplane +
+                                 (in ? (int64_t)sy * g.Wo + sx : 0));
+                sfg[m][i * K + j] = in ? val : A(0);
+            }
+    }
+
+    Stg stg;
+    stg.init(g, qy0 + g.row0_off, lane);
+    const T *gs = go + (ww.n * g.C + ww.c_begin) * oplane;
+    T *ds = dx + (ww.n * g.C + ww.c_begin) * iplane + (int64_t)u0 * g.W;
+    const int nch = ww.c_end - ww.c_begin;
+    stg.template issue<0>(gs);
+    if constexpr (NST > 1) stg.template issue<1>(gs + (int64_t)min(1, nch - 1) * oplane);
+    if constexpr (NST > 2) stg.template issue<2>(gs + (int64_t)min(2, nch - 1) * oplane);
+    if constexpr (NST > 3) stg.template issue<3>(gs + (int64_t)min(3, nch - 1) * oplane);
+    zero_tile(lds_in, g.tile, lane);
+    tst.put(taps, nch, lane);
+    wave_sync();
+
+    auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        stg.template commit<ST>(lds_in);
+        stg.template issue<ST>(gs + (int64_t)min(ci + NST, nch - 1) * oplane);
+        wave_sync();
+        A w[KK];
+        load_taps<KK>(taps, ci, w);
+#pragma unroll
+        for (int m = 0; m < PS; ++m) {
+            if (m >= g.nslots) break;
+            A acc[S][S];
+#pragma unroll
+            for (int a = 0; a < S; ++a)
+#pragma unroll
+                for (int c = 0; c < S; ++c) acc[a][c] = 0;
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const A gv = ld(lds_in + lb[m] + (TM::dq(i) + TM::halo_lo) * g.P + TM::dq(j) +
+                                    TM::halo_lo);
+                    acc[TM::phase(i)][TM::phase(j)] +=
+                        gv * comb<MUL, A>(w[i * K + j], sfg[m][i * K + j]);
+                }
+#pragma unroll
+            for (int a = 0; a < S; ++a)
+#pragma unroll
+                for (int c = 0; c < S; ++c) {
+                    if (cu[m] + a < g.H && cv[m] + c < g.W)
+                        st(lds_out + ob[m] + a * g.W + c, acc[a][c]);
+                }
+        }
+        wave_sync();
+        store_strip<T, V>(lds_out, ds + (int64_t)ci * iplane, n_out, lane);
+        wave_sync();
+    };
+
+    auto group = [&](int c) __attribute__((always_inline)) {
+        channel(std::integral_constant<int, 0>{}, c);
+        if constexpr (NST > 1) channel(std::integral_constant<int, 1>{}, c + 1);
+        if constexpr (NST > 2) channel(std::integral_constant<int, 2>{}, c + 2);
+        if constexpr (NST > 3) channel(std::integral_constant<int, 3>{}, c + 3);
+    };
+    // The first group is peeled off the loop: the loop is then entered only in
+    // its steady state (NST loads and NST stores in flight), and the wait the
+    // compiler places before a commit covers that stage's load alone instead
+    // of draining the younger loads and stores as well.
+    const int nfull = nch / NST * NST;
+    if (nfull > 0) {
+        group(0);
+        for (int c = NST; c < nfull; c += NST) group(c);
+    }
+    if constexpr (NST > 1) {
+        if (nfull < nch) channel(std::integral_constant<int, 0>{}, nfull);
+        if constexpr (NST > 2) {
+            if (nfull + 1 < nch) channel(std::integral_constant<int, 1>{}, nfull + 1);
+            if (nfull + 2 < nch) channel(std::integral_constant<int, 2>{}, nfull + 2);
+        }
+    }
+}
+
+}  // namespace wave
+
+enum WaveKind { kWaveForward = 0, kWaveFeatures = 1 };
+// Host-side geometry (ddf_tiled_host.hip).  *ps and *nv select the kernel.
+// max_vec > 0 caps the elements per global access (1 = scalar accesses).
+bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom *g, int *ps,
+                   int *nv);
+
+}  // namespace ddf
