@@ -12,13 +12,17 @@ bracketed by device synchronisation.  Inputs and outputs rotate over enough
 distinct buffer sets to exceed the 256 MB last-level cache, so the figure is an
 HBM figure.  ``value`` = algorithmic bytes of forward+backward / time per step.
 
-After the timed region the same K steps are replayed with an event pair around
-every library call (forward / feature gradient / filter gradients) to obtain the
-per-kernel durations the ``roofline`` object reports for the dominant kernel.
+After the timed region each library call of a step (forward / feature gradient
+/ filter gradients) is timed on its own: K back-to-back launches between one
+event pair, same buffers.  The ``roofline`` object reports the slowest of them.
+
+``--model`` additionally times ddf_mul_resnet50 inference (fp16, batch 128,
+224x224, random weights) and reports images/s with the DDF share of the time.
 
 Prints ONE JSON line on stdout; everything else goes to stderr.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -44,6 +48,7 @@ WORKLOADS = {
 }
 DEFAULT_WORKLOAD = 'r50_stage3_mul_fp32'
 DTYPE_NAME = {torch.float32: 'f32', torch.float16: 'f16', torch.float64: 'f64'}
+PHASES = ('fwd', 'dx', 'dfilters')
 
 
 def log(*a):
@@ -76,7 +81,7 @@ def algorithmic_bytes(N, C, H, W, k, s, esz):
     return {
         'fwd': esz * (X + O + CF + SF),
         'bwd': esz * (2 * X + O + 2 * CF + 2 * SF),
-        # per kernel of the backward pass
+        # per library call of the backward pass
         'dx': esz * (O + CF + SF + X),
         'dfilters': esz * (O + X + CF + SF + CF + SF),
     }
@@ -85,7 +90,7 @@ def algorithmic_bytes(N, C, H, W, k, s, esz):
 class Workset(object):
     """One rotating set of device buffers for a workload."""
 
-    def __init__(self, host, like=None):
+    def __init__(self, host):
         x, cf, sf, go = host
         self.x, self.cf, self.sf, self.go = (t.cuda() for t in (x, cf, sf, go))
         self.out = torch.empty_like(self.go)
@@ -98,7 +103,59 @@ class Workset(object):
                    (self.x, self.cf, self.sf, self.go, self.out, self.dx, self.dcf, self.dsf))
 
 
-def run_workload(name, steps, warmup, lib, verbose=True):
+class Launcher(object):
+    """Pre-built argument lists for the C ABI, so that the timed loops spend
+    their host time in ``ddf_hip_forward`` / ``ddf_hip_backward`` and not in
+    building ctypes objects."""
+
+    def __init__(self, lib, sets, shape, k, d, s, combine, dtype, ws):
+        N, C, H, W = shape
+        self.clib = lib.lib()
+        self.check = lib.check
+        p = lambda t: ctypes.c_void_p(t.data_ptr())
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        tail = (N, C, H, W, k, d, s, lib.COMBINE[combine], lib.DTYPE[dtype])
+        ws_bytes = ws.numel() if ws is not None else 0
+        self.fwd_args = [(p(b.x), p(b.cf), p(b.sf), p(b.out)) + tail + (0, stream) for b in sets]
+        self.bwd_args = {
+            need: [(p(b.go), p(b.x), p(b.cf), p(b.sf), p(b.dx), p(b.dcf), p(b.dsf),
+                    p(ws) if ws is not None else None, ws_bytes) + tail + (need, 0, stream)
+                   for b in sets]
+            for need in (lib.NEED_DX, lib.NEED_DCF | lib.NEED_DSF, 7)}
+        self.n = len(sets)
+
+    def fwd(self, i):
+        rc = self.clib.ddf_hip_forward(*self.fwd_args[i % self.n])
+        if rc:
+            self.check(rc)
+
+    def bwd(self, i, need=7):
+        rc = self.clib.ddf_hip_backward(*self.bwd_args[need][i % self.n])
+        if rc:
+            self.check(rc)
+
+    def phase(self, name, i):
+        if name == 'fwd':
+            self.fwd(i)
+        elif name == 'dx':
+            self.bwd(i, 1)
+        else:
+            self.bwd(i, 6)
+
+
+def timed(fn, count):
+    """Milliseconds per call of fn(i), i < count, between two stream events."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(count):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / count
+
+
+def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
     N, C, H, W, k, d, s, combine, dtype = WORKLOADS[name]
     esz = torch.empty(0, dtype=dtype).element_size()
     host = make_inputs(N, C, H, W, k, s, dtype)
@@ -107,50 +164,33 @@ def run_workload(name, steps, warmup, lib, verbose=True):
     free, _ = torch.cuda.mem_get_info()
     nsets = int(min(nsets, max(2, (free // 2) // first.nbytes())))
     sets = [first] + [Workset(host) for _ in range(nsets - 1)]
-    need_all = lib.NEED_DX | lib.NEED_DCF | lib.NEED_DSF
-    ws_bytes = lib.backward_workspace_bytes((N, C, H, W), k, d, s, combine, dtype, need_all)
-    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device='cuda')
-
-    def fwd(b):
-        lib.forward(b.x, b.cf, b.sf, b.out, k, d, s, combine)
-
-    def bwd(b, need=need_all):
-        lib.backward(b.go, b.x, b.cf, b.sf, b.dx, b.dcf, b.dsf, k, d, s, combine, need, ws)
+    ws_bytes = lib.backward_workspace_bytes((N, C, H, W), k, d, s, combine, dtype, 7)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda') if ws_bytes else None
+    run = Launcher(lib, sets, (N, C, H, W), k, d, s, combine, dtype, ws)
 
     def step(i):
-        b = sets[i % nsets]
-        fwd(b)
-        bwd(b)
+        run.fwd(i)
+        run.bwd(i)
 
     for i in range(warmup):
         step(i)
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for i in range(steps):
-        step(i)
-    stop.record()
-    torch.cuda.synchronize()
-    ms_per_step = start.elapsed_time(stop) / steps
+    ms_per_step = timed(step, steps)
 
-    # replay with an event pair around every library call
-    phases = {'fwd': lambda b: fwd(b),
-              'dx': lambda b: bwd(b, lib.NEED_DX),
-              'dfilters': lambda b: bwd(b, lib.NEED_DCF | lib.NEED_DSF)}
-    evs = {p: [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-               for _ in range(steps)] for p in phases}
-    for i in range(steps):
-        b = sets[i % nsets]
-        for p, fn in phases.items():
-            e0, e1 = evs[p][i]
-            e0.record()
-            fn(b)
-            e1.record()
-    torch.cuda.synchronize()
+    # each library call on its own: back-to-back launches, same buffers
     phase_ms = {}
-    for p in phases:
-        ts = sorted(e0.elapsed_time(e1) for e0, e1 in evs[p])
-        phase_ms[p] = {'mean': sum(ts) / len(ts), 'median': ts[len(ts) // 2], 'min': ts[0]}
+    for ph in PHASES:
+        for i in range(min(warmup, 10)):
+            run.phase(ph, i)
+        phase_ms[ph] = timed(lambda i, ph=ph: run.phase(ph, i), steps)
+
+    if copy_probe:
+        # a plain device copy of known size: the yardstick the hardware
+        # fetch/write counters are scaled by
+        a = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device='cuda')
+        b = torch.empty_like(a)
+        for _ in range(4):
+            b.copy_(a)
+        torch.cuda.synchronize()
 
     ab = algorithmic_bytes(N, C, H, W, k, s, esz)
     total = ab['fwd'] + ab['bwd']
@@ -161,27 +201,28 @@ def run_workload(name, steps, warmup, lib, verbose=True):
         'gbps': total / (ms_per_step * 1e-3) / 1e9,
         'images_per_s': N / (ms_per_step * 1e-3),
         'bytes': ab, 'phase_ms': phase_ms, 'buffer_sets': nsets,
-        'phase_gbps': {p: ab[p] / (phase_ms[p]['mean'] * 1e-3) / 1e9 for p in phases},
+        'phase_gbps': {p: ab[p] / (phase_ms[p] * 1e-3) / 1e9 for p in PHASES},
     }
     if verbose:
         log('[%s] %.1f us/step  fwd+bwd %.0f GB/s (%.1f%% of HBM peak), %d buffer sets' % (
             name, ms_per_step * 1e3, res['gbps'], 100 * res['gbps'] / HBM_PEAK_GBPS, nsets))
-        for p in phases:
-            log('    %-9s %7.1f us (median %.1f, min %.1f)  %6.0f GB/s  %.1f%%' % (
-                p, phase_ms[p]['mean'] * 1e3, phase_ms[p]['median'] * 1e3, phase_ms[p]['min'] * 1e3,
-                res['phase_gbps'][p], 100 * res['phase_gbps'][p] / HBM_PEAK_GBPS))
-    del sets, first
+        for p in PHASES:
+            log('    %-9s %7.1f us  %6.0f GB/s  %.1f%%' % (
+                p, phase_ms[p] * 1e3, res['phase_gbps'][p],
+                100 * res['phase_gbps'][p] / HBM_PEAK_GBPS))
+    del sets, first, run
     torch.cuda.empty_cache()
     return res
 
 
-def cpu_baseline(name, budget_s=15.0):
+def cpu_baseline(name, budget_s=12.0):
     """The CPU oracle (a port of the reference's formulation; the reference has
     no CPU path of its own) timed on this host: fp32, forward + backward, on a
-    batch slice sized to finish within the budget."""
+    the whole batch of the workload,
+    repeated until the time budget is used."""
     import oracle
     N, C, H, W, k, d, s, combine, dtype = WORKLOADS[name]
-    n_sub = min(N, 8)
+    n_sub = N
     x, cf, sf, go = (t.float() for t in make_inputs(n_sub, C, H, W, k, s, dtype))
     threads = oracle.num_threads()
 
@@ -196,17 +237,34 @@ def cpu_baseline(name, budget_s=15.0):
         once()
         reps += 1
         el = time.perf_counter() - t0
-        if el > budget_s or reps >= 200:
+        if el > budget_s:
             break
     per = el / reps
     ab = algorithmic_bytes(n_sub, C, H, W, k, s, 4)
     return {
-        'value': (ab['fwd'] + ab['bwd']) / per / 1e9, 'unit': 'GB/s', 'cores': threads,
-        'kind': 'port',
-        'sample': '%d of %d samples of %s in fp32, forward+backward, %d repetitions, '
-                  '%.2f s each, C oracle with OpenMP' % (n_sub, N, name, reps, per),
-        'images_per_s': n_sub / per,
+        'value': round((ab['fwd'] + ab['bwd']) / per / 1e9, 3), 'unit': 'GB/s',
+        'cores': threads, 'kind': 'port',
+        'sample': 'all %d samples of %s in fp32, forward+backward, %d repetitions in %.1f s '
+                  '(%.4f s each), C oracle with OpenMP' % (N, name, reps, el, per),
+        'images_per_s': round(n_sub / per, 1),
     }
+
+
+def model_inference(batch=128, steps=10, warmup=3):
+    """ddf_mul_resnet50 inference, fp16, random weights, synthetic input."""
+    from ddfnet_amd import ddf_resnet
+    torch.manual_seed(0)
+    model = ddf_resnet.ddf_mul_resnet50().cuda().half().eval()
+    x = torch.randn(batch, 3, 224, 224, device='cuda', dtype=torch.float16)
+    with torch.no_grad():
+        for _ in range(warmup):
+            model(x)
+        ms = timed(lambda i: model(x), steps)
+        layers = ddf_resnet.time_ddf_layers(model, x)
+    ddf_ms = sum(l['ms'] for l in layers)
+    return {'model': 'ddf_mul_resnet50', 'batch': batch, 'dtype': 'f16',
+            'images_per_s': round(batch / (ms * 1e-3), 1), 'ms_per_batch': round(ms, 3),
+            'ddf_ms_per_batch': round(ddf_ms, 3), 'ddf_layers': layers}
 
 
 def main():
@@ -215,8 +273,11 @@ def main():
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--workload', default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
-    ap.add_argument('--all', action='store_true', help='also time the other workloads (stderr)')
+    ap.add_argument('--all', action='store_true', help='also time the other workloads')
+    ap.add_argument('--model', action='store_true', help='also time ddf_mul_resnet50 inference')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--copy-probe', action='store_true',
+                    help='also run a plain 256 MiB device copy (calibrates hardware counters)')
     args = ap.parse_args()
     if args.gpus != 1:
         log('bench.py measures one GPU: the operator shards over the batch with no exchange, '
@@ -232,11 +293,11 @@ def main():
         for name in WORKLOADS:
             if name != args.workload:
                 extra[name] = run_workload(name, args.steps, args.warmup, lib)
-    res = run_workload(args.workload, args.steps, args.warmup, lib)
+    res = run_workload(args.workload, args.steps, args.warmup, lib, copy_probe=args.copy_probe)
 
-    dominant = max(res['phase_ms'], key=lambda p: res['phase_ms'][p]['mean'])
+    dominant = max(PHASES, key=lambda p: res['phase_ms'][p])
     dom_bytes = res['bytes'][dominant]
-    dom_s = res['phase_ms'][dominant]['mean'] * 1e-3
+    dom_s = res['phase_ms'][dominant] * 1e-3
     achieved = dom_bytes / dom_s / 1e9
     line = {
         'metric': 'ddf_fwd_bwd_hbm_gbps', 'value': round(res['gbps'], 2), 'unit': 'GB/s',
@@ -255,17 +316,23 @@ def main():
                      'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': None,
                      'bytes_per_launch': dom_bytes,
                      'avg_launch_us': round(dom_s * 1e6, 3)},
-        'phases_us': {p: round(v['mean'] * 1e3, 3) for p, v in res['phase_ms'].items()},
+        'phases_us': {p: round(res['phase_ms'][p] * 1e3, 3) for p in PHASES},
     }
     if extra:
         line['other_workloads'] = {
             n: {'gbps': round(r['gbps'], 1), 'us_per_step': round(r['ms_per_step'] * 1e3, 2),
-                'images_per_s': round(r['images_per_s'], 1)} for n, r in extra.items()}
+                'images_per_s': round(r['images_per_s'], 1),
+                'phases_us': {p: round(r['phase_ms'][p] * 1e3, 2) for p in PHASES}}
+            for n, r in extra.items()}
+    if args.model:
+        line['model_inference'] = model_inference()
+        mi = line['model_inference']
+        log('[model] %s bs%d %s: %.1f images/s (%.2f ms/batch, DDF layers %.2f ms)' % (
+            mi['model'], mi['batch'], mi['dtype'], mi['images_per_s'], mi['ms_per_batch'],
+            mi['ddf_ms_per_batch']))
     if not args.no_cpu:
         line['cpu_baseline'] = cpu_baseline(args.workload)
         cb = line['cpu_baseline']
-        cb['value'] = round(cb['value'], 3)
-        cb['images_per_s'] = round(cb['images_per_s'], 1)
         log('[cpu] %s: %.2f GB/s on %d threads' % (cb['sample'], cb['value'], cb['cores']))
     print(json.dumps(line), flush=True)
 

@@ -1,0 +1,120 @@
+"""Callers of the operator on the GPU: DDFPack, DDFUpPack and a DDF-ResNet,
+against the same modules evaluated on the CPU in fp64 with the oracle standing
+in for the HIP operator (same weights, same inputs)."""
+import copy
+
+import pytest
+import torch
+
+import oracle
+import ddfnet_amd
+from ddfnet_amd import modules as ddf_modules
+
+pytestmark = pytest.mark.gpu
+
+
+class _OracleOp(object):
+    """``ddf`` replacement for CPU fp64 modules: the differentiable unfold form."""
+
+    def __call__(self, x, cf, sf, k=3, d=1, s=1, combine='mul', version=''):
+        return oracle.unfold_forward(x, cf, sf, k, d, s, combine)
+
+
+def cpu_reference(module, monkeypatch, *inputs):
+    ref = copy.deepcopy(module).cpu().double()
+    monkeypatch.setattr(ddf_modules, 'ddf', _OracleOp())
+    ins = [t.detach().cpu().double().requires_grad_(True) for t in inputs]
+    out = ref(*ins)
+    monkeypatch.undo()
+    return ref, ins, out
+
+
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('stride,head', [(1, 1), (2, 1), (1, 4)])
+def test_ddfpack_matches_cpu_reference(stride, head, combine, monkeypatch):
+    torch.manual_seed(0)
+    pack = ddfnet_amd.DDFPack(16, kernel_size=3, stride=stride, head=head,
+                              kernel_combine=combine).cuda()
+    x = torch.randn(2, 16, 12, 12, device='cuda', requires_grad=True)
+    out = pack(x)
+    assert out.shape == (2, 16, 12 // stride, 12 // stride)
+    go = torch.randn_like(out)
+    out.backward(go)
+    ref, (xr,), out_r = cpu_reference(pack, monkeypatch, x)
+    out_r.backward(go.cpu().double())
+    assert torch.allclose(out.detach().cpu().double(), out_r.detach(), rtol=1e-4, atol=1e-5)
+    assert torch.allclose(x.grad.cpu().double(), xr.grad, rtol=1e-3, atol=1e-4)
+    for (name, p), (_, pr) in zip(pack.named_parameters(), ref.named_parameters()):
+        assert torch.allclose(p.grad.cpu().double(), pr.grad, rtol=1e-3, atol=1e-4), name
+
+
+def test_ddfuppack_matches_cpu_reference(monkeypatch):
+    torch.manual_seed(1)
+    up = ddfnet_amd.DDFUpPack(8, kernel_size=3, scale_factor=2).cuda()
+    x = torch.randn(2, 8, 10, 10, device='cuda')
+    out = up(x)
+    assert out.shape == (2, 8, 20, 20)
+    _, _, out_r = cpu_reference(up, monkeypatch, x)
+    assert torch.allclose(out.detach().cpu().double(), out_r.detach(), rtol=1e-4, atol=1e-5)
+
+
+def test_ddfuppack_with_joint_guidance(monkeypatch):
+    torch.manual_seed(2)
+    up = ddfnet_amd.DDFUpPack(8, kernel_size=3, scale_factor=2, joint_channels=8).cuda()
+    x = torch.randn(1, 8, 6, 6, device='cuda')
+    joint = torch.randn(1, 8, 6, 6, device='cuda')
+    out = up(x, joint)
+    _, _, out_r = cpu_reference(up, monkeypatch, x, joint)
+    assert torch.allclose(out.detach().cpu().double(), out_r.detach(), rtol=1e-4, atol=1e-5)
+
+
+def test_ddfpack_fp16_keeps_dtype():
+    pack = ddfnet_amd.DDFPack(32).cuda().half()
+    x = torch.randn(2, 32, 14, 14, device='cuda', dtype=torch.float16)
+    out = pack(x)
+    assert out.dtype == torch.float16 and torch.isfinite(out).all()
+
+
+def test_ddfpack_under_autocast():
+    """fp16 activations meet fp32 parameters inside the filter branches; the
+    operator promotes its operands to one dtype."""
+    pack = ddfnet_amd.DDFPack(32).cuda()
+    x = torch.randn(2, 32, 14, 14, device='cuda')
+    with torch.autocast('cuda', dtype=torch.float16):
+        out = pack(x)
+    want = pack(x)
+    assert torch.isfinite(out).all()
+    assert (out.float() - want).abs().max() / want.abs().max() < 2e-2
+
+
+def test_resnet50_forward_matches_cpu_reference(monkeypatch):
+    """ddf_mul_resnet50 at a reduced resolution (64x64, batch 2): 16 DDF layers
+    at four plane sizes and both strides, fp32 against the CPU fp64 model."""
+    from ddfnet_amd import ddf_resnet
+    torch.manual_seed(3)
+    model = ddf_resnet.ddf_mul_resnet50(num_classes=10).cuda().eval()
+    x = torch.randn(2, 3, 64, 64, device='cuda')
+    with torch.no_grad():
+        out = model(x)
+        assert out.shape == (2, 10)
+        ref = copy.deepcopy(model).cpu().double()
+        monkeypatch.setattr(ddf_modules, 'ddf', _OracleOp())
+        out_r = ref(x.cpu().double())
+    scale = out_r.abs().max().item()
+    assert (out.cpu().double() - out_r).abs().max().item() <= 1e-3 * scale
+
+
+def test_resnet50_fp16_inference_and_layer_timing():
+    from ddfnet_amd import ddf_resnet
+    torch.manual_seed(4)
+    model = ddf_resnet.ddf_mul_resnet50().cuda().half().eval()
+    x = torch.randn(4, 3, 224, 224, device='cuda', dtype=torch.float16)
+    with torch.no_grad():
+        out = model(x)
+    assert out.shape == (4, 1000) and torch.isfinite(out).all()
+    layers = ddf_resnet.time_ddf_layers(model, x, iters=2)
+    shapes = [(l['shape'][1], l['shape'][2], l['stride']) for l in layers]
+    # the 16 DDF call shapes of ResNet-50 at 224x224
+    want = ([(64, 56, 1)] * 3 + [(128, 56, 2)] + [(128, 28, 1)] * 3 + [(256, 28, 2)] +
+            [(256, 14, 1)] * 5 + [(512, 14, 2)] + [(512, 7, 1)] * 2)
+    assert shapes == want
