@@ -3,15 +3,12 @@
 #include <algorithm>
 #include <cstdlib>
 
-#include "ddf_tiled.h"
 #include "ddf_wave.h"
 
 namespace ddf {
 
 namespace {
 
-constexpr int kLdsBudget = 48 * 1024;   // bytes per workgroup; leaves room for >= 3 per CU
-constexpr int kMaxThreads = 512;
 
 int env_int(const char *name, int fallback) {
     const char *v = std::getenv(name);
@@ -26,126 +23,6 @@ int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 bool tiled_shape_instantiated(int k, int d, int s) {
     return (k == 3 || k == 5) && (d == 1 || d == 2) && (s == 1 || s == 2);
-}
-
-// Fills *g and *ps for one kernel kind; false when the tiled family does not
-// cover the problem (the caller then uses the generic kernels).  *ps is the
-// number of pixels a lane owns in the filter-gradient kernel (1 otherwise).
-bool tiled_geometry(const Problem &p, int dtype, int kind, TileGeom *g, int *ps_out) {
-    if (!tiled_shape_instantiated(p.k, p.d, p.s)) return false;
-    if (p.N <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0) return false;
-    if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
-    const int esz = elem_size(dtype), asz = acc_size(dtype);
-    const int K = p.k, D = p.d, S = p.s, R = p.r, KK = p.kk;
-    const int H = (int)p.H, W = (int)p.W, Ho = (int)p.Ho, Wo = (int)p.Wo, C = (int)p.C;
-    const bool per_lane = (kind == kKindFilters);
-
-    TileGeom t{};
-    t.C = C; t.H = H; t.W = W; t.Ho = Ho; t.Wo = Wo;
-    int lin_cols;          // elements per row of the linear tile
-    int lin_rows_per_cell; // rows of it per cell row
-    {
-        t.rows = Ho; t.cols = Wo;
-        t.src_rows = H; t.src_cols = W;
-        t.P = std::max((Wo - 1) * S + (K - 1) * D + 1, R * D + W);
-        t.col_off = R * D; t.row0_off = -R * D;
-        lin_cols = Wo; lin_rows_per_cell = 1;     // the out strip, or the dO strip
-    }
-    auto tile_rows = [&](int th) {
-        return (th - 1) * S + (K - 1) * D + 1;
-    };
-
-    // Widest aligned global access: 16 bytes, else 8, else one element.  Every
-    // plane and every strip start must be a multiple of it, and a vector may
-    // cross at most one row end of the padded tile.
-    const int64_t plane_in = (int64_t)t.src_rows * t.src_cols;
-    const int64_t plane_lin = (int64_t)Ho * Wo;
-    auto vec_ok = [&](int v, int nstrips) {
-        if (v == 1) return true;
-        if (plane_in % v || plane_lin % v || t.src_cols < v) return false;
-        if (per_lane && ((int64_t)H * W) % v) return false;
-        return nstrips == 1 || (t.src_cols % v == 0 && lin_cols % v == 0);
-    };
-    const int forced_vec = env_int("DDF_TUNE_VEC", 0);
-
-    // Cells one block pass can own.
-    const int max_ps = per_lane ? (KK > 9 ? 2 : 4) : 1;
-    const int min_ps = per_lane ? 2 : 1;
-    const int capacity = per_lane ? kWave * max_ps : kMaxThreads;
-    if (t.cols > capacity || t.cols >= 65536 || t.src_cols >= 65536) return false;
-
-    // Strip height (and pixels per lane): minimise an instruction estimate.
-    // Compute costs ~2*KK (3*KK for the filter gradients) per owned cell slot,
-    // idle lanes included; staging costs ~4 per tile element; the
-    // filter-gradient kernel adds one butterfly (~3*KK) per wave pass.
-    const int c_comp = (per_lane ? 3 : 2) * KK, c_load = 4, c_red = 3 * KK;
-    double best = 1e30;
-    int best_th = 0, best_ps = 0;
-    const int forced_th = env_int(per_lane ? "DDF_TUNE_TH_FILTERS" : "DDF_TUNE_TH", 0);
-    const int forced_ps = env_int("DDF_TUNE_PS_FILTERS", 0);
-    auto threads_for = [&](int np) {
-        return per_lane ? kWave * tiled::kFilterWaves : round_up(np, kWave);
-    };
-    for (int th = 1; th <= t.rows; ++th) {
-        const int np = th * t.cols;
-        if (np > capacity) break;
-        if (forced_th && th != std::min(forced_th, t.rows)) continue;
-        const int nstrips = (t.rows + th - 1) / th;
-        const int64_t lds = (int64_t)tiled::kCB * esz *
-                            (tile_rows(th) * t.P + round_up(th * lin_rows_per_cell * lin_cols, 8));
-        if (lds > kLdsBudget || tile_rows(th) * t.src_cols >= 65536) break;
-        for (int ps = min_ps; ps <= max_ps; ps *= 2) {
-            if (per_lane && forced_ps && ps != forced_ps) continue;
-            if (per_lane && np > kWave * ps) continue;
-            const int slots = per_lane ? kWave * ps : threads_for(np);
-            double cost = (double)nstrips *
-                          (slots * c_comp + (double)tile_rows(th) * t.P * c_load +
-                           (per_lane ? c_red : 0));
-            if (!vec_ok(16 / esz, nstrips)) cost *= vec_ok(8 / esz, nstrips) ? 1.1 : 1.5;
-            cost *= 1.0 + 0.02 * ps;  // mild preference for fewer registers
-            if (cost < best) { best = cost; best_th = th; best_ps = ps; }
-        }
-    }
-    if (best_th == 0) return false;
-    t.TH = best_th;
-    t.nstrips = (t.rows + t.TH - 1) / t.TH;
-    t.IH = tile_rows(t.TH);
-    t.tile = t.IH * t.P;
-    t.lin_tile = round_up(t.TH * lin_rows_per_cell * lin_cols, 8);
-    t.threads = threads_for(t.TH * t.cols);
-    t.vec = 1;
-    for (int bytes = 16; bytes >= 2 * esz && dtype != DDF_F64; bytes /= 2)
-        if (vec_ok(bytes / esz, t.nstrips)) { t.vec = bytes / esz; break; }
-    if (forced_vec) t.vec = std::min(t.vec, forced_vec);
-
-    // Channels per block: enough blocks to fill 256 CUs several times over, but
-    // long enough channel walks to amortise the spatial-filter registers.
-    const int64_t base = p.N * t.nstrips;
-    const int target = env_int(per_lane ? "DDF_TUNE_BLOCKS_FILTERS" : "DDF_TUNE_BLOCKS",
-                               per_lane ? 1024 : 2048) * 256 / t.threads;
-    const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
-    int cpb = (int)((C + want_split - 1) / want_split);
-    const int forced_cpb = env_int(per_lane ? "DDF_TUNE_CPB_FILTERS" : "DDF_TUNE_CPB", 0);
-    if (forced_cpb) cpb = forced_cpb;
-    cpb = std::min(round_up(std::max(cpb, 1), tiled::kCB), round_up(C, tiled::kCB));
-    cpb = std::min(cpb, 256);
-    t.cpb = cpb;
-    t.csplit = (C + cpb - 1) / cpb;
-
-    // tiles, then the channel-filter taps of the block's channels (accumulator type)
-    t.lds_bytes = tiled::kCB * (t.tile + t.lin_tile) * esz + cpb * ((KK + 3) / 4 * 4) * asz;
-    if (per_lane)
-        t.lds_bytes = std::max(t.lds_bytes, tiled::kFilterWaves * KK * kWave * asz);
-    if (t.lds_bytes > 64 * 1024) return false;
-
-    t.src_magic = t.src_cols == 1 ? 0u : (unsigned)((0x100000000ull + t.src_cols - 1) / t.src_cols);
-    t.cols_magic = t.cols == 1 ? 0u : (unsigned)((0x100000000ull + t.cols - 1) / t.cols);
-    const int64_t nblocks = base * t.csplit;
-    if (nblocks > (1 << 30)) return false;
-    t.nblocks = (int)nblocks;
-    *g = t;
-    *ps_out = per_lane ? best_ps : 1;
-    return true;
 }
 
 // Geometry of the wavefront-per-strip kernels (forward, feature gradient).
@@ -216,32 +93,41 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     // included) plus the halo rows re-staged per strip.
     double best = 1e30;
     int best_ps = 0, best_th = 0, best_v = 0, best_nv = 0;
-    for (int ps = 4; ps <= kMaxSlots; ps *= 2) {
-        if (forced_ps && ps != forced_ps) continue;
+    // slots per lane: 4 or 8; the filter-gradient kernel keeps two register
+    // sets per slot and is built for 4 (k=3) or 2 (k=5) only
+    const bool filters = kind == kWaveFilters;
+    const int ps_lo = filters ? (p.kk > 9 ? 2 : 4) : 4;
+    const int ps_hi = filters ? ps_lo : kMaxSlots;
+    for (int ps = ps_lo; ps <= ps_hi; ps *= 2) {
+        if (forced_ps && !filters && ps != forced_ps) continue;
         if (ps < cseg) continue;
-        int th = (ps / cseg) * RS;
-        th = std::min(th, t.rows);
+        // cell rows per strip: as many slot rows as the lane's slots allow,
+        // fewer when the source strip would not fit the staging registers
         const int forced_th = env_int("DDF_TUNE_TH", 0);
-        if (forced_th) th = std::min(th, forced_th);
-        const int nstrips = (t.rows + th - 1) / th;
-        int v = 1;
-        if (dtype != DDF_F64 && vec_ok(4, th)) v = 4;
-        if (forced_vec) v = std::min(v, forced_vec);
-        if (max_vec) v = std::min(v, max_vec);
-        const int staged = std::min(tile_rows(th), t.src_rows) * t.src_cols;
-        const int need_nv = (staged + v * kWave - 1) / (v * kWave);
-        int nv = 0;
-        for (int cand : {1, 2, 4, 8})
-            if (cand >= need_nv) { nv = cand; break; }
-        // instantiated: V=4 with (ps 4: nv 1, 2, 4; ps 8: nv 4); V=1 with (ps 4: nv 4, 8)
-        if (nv == 0) continue;
-        if (v == 4) {
-            if (nv == 8) continue;
-            if (ps == 8) nv = 4;
-        } else {
-            if (ps == 8) continue;
-            nv = std::max(nv, 4);
+        int th = 0, v = 1, nv = 0;
+        for (int srows = ps / cseg; srows >= 1 && nv == 0; --srows) {
+            th = std::min(srows * RS, t.rows);
+            if (forced_th) th = std::min(th, forced_th);
+            v = (dtype != DDF_F64 && vec_ok(4, th)) ? 4 : 1;
+            if (forced_vec) v = std::min(v, forced_vec);
+            if (max_vec) v = std::min(v, max_vec);
+            const int staged = std::min(tile_rows(th), t.src_rows) * t.src_cols;
+            const int need_nv = (staged + v * kWave - 1) / (v * kWave);
+            for (int cand : {1, 2, 4, 8})
+                if (cand >= need_nv) { nv = cand; break; }
+            // instantiated: V=4 with (ps 2|4: nv 1, 2, 4; ps 8: nv 4); V=1 with (ps 4: nv 4, 8; ps 2: nv 4)
+            if (nv == 0) continue;   // more than 8 vectors per lane: try fewer rows
+            if (v == 4) {
+                if (nv == 8) nv = 0;
+                else if (ps == 8) nv = 4;
+            } else {
+                if (ps == 8) nv = 0;
+                else nv = std::max(nv, 4);
+                if (ps == 2 && nv == 8) nv = 0;
+            }
         }
+        if (nv == 0) continue;
+        const int nstrips = (t.rows + th - 1) / th;
         const int64_t lds = (int64_t)esz * (2 * round_up(tile_rows(th) * t.P, 8) + 2 * wave::kSpare +
                                             round_up(th * t.lin_rpc * t.lin_cols, 8)) + 4096;
         if (lds > 64 * 1024) continue;
@@ -277,19 +163,25 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
 
     // Channels per wave: enough waves to fill the machine several times over,
     // long enough walks to amortise the spatial-filter registers.
+    const int waves_per_block = filters ? wave::kFilterWaves : 1;
     const int64_t base = p.N * t.nstrips;
-    const int target = env_int("DDF_TUNE_WAVES", 4096);
+    const int target = env_int(filters ? "DDF_TUNE_WAVES_FILTERS" : "DDF_TUNE_WAVES",
+                               filters ? 2048 : 4096);
     const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
     int cpw = (int)((C + want_split - 1) / want_split);
     cpw = std::max(cpw, std::min(C, env_int("DDF_TUNE_MIN_CPW", 4)));
-    cpw = std::min(cpw, std::max(1, wave::kTapLoads * kWave / p.kk));  // taps staged in one go
-    const int forced_cpw = env_int("DDF_TUNE_CPW", 0);
+    const int forced_cpw = env_int(filters ? "DDF_TUNE_CPW_FILTERS" : "DDF_TUNE_CPW", 0);
     if (forced_cpw) cpw = std::min(forced_cpw, C);
+    cpw = std::max(1, std::min(cpw, wave::kTapLoads * kWave / p.kk));  // taps staged in one go
     t.cpw = cpw;
-    t.csplit = (C + cpw - 1) / cpw;
-    // tiles, then the channel-filter taps of the wave's channels (accumulator type)
-    t.lds_bytes = (t.tile + t.lin_tile + 2 * wave::kSpare) * esz +
-                  cpw * ((p.kk + 3) / 4 * 4) * acc_size(dtype);
+    t.cpb = cpw * waves_per_block;
+    t.csplit = (C + t.cpb - 1) / t.cpb;
+    // per wave: tiles, then the channel-filter taps of its channels (accumulator type)
+    t.lds_wave_bytes = round_up((t.tile + t.lin_tile + 2 * wave::kSpare) * esz +
+                                cpw * ((p.kk + 3) / 4 * 4) * acc_size(dtype), 16);
+    t.lds_bytes = t.lds_wave_bytes * waves_per_block;
+    if (filters)  // the cross-wave sum of the dSF accumulators reuses the block's LDS
+        t.lds_bytes = std::max(t.lds_bytes, waves_per_block * p.kk * kWave * acc_size(dtype));
     if (t.lds_bytes > 64 * 1024) return false;
     t.src_magic = t.src_cols == 1 ? 0u : (unsigned)((0x100000000ull + t.src_cols - 1) / t.src_cols);
     const int64_t nblocks = base * t.csplit;
@@ -307,17 +199,19 @@ bool tiled_forward_supported(const Problem &p, int dtype) {
 }
 
 bool tiled_backward_supported(const Problem &p, int dtype) {
-    WaveGeom w; TileGeom g; int ps, nv;
+    WaveGeom w; int ps, nv;
     return wave_geometry(p, dtype, kWaveFeatures, 0, &w, &ps, &nv) &&
-           tiled_geometry(p, dtype, kKindFilters, &g, &ps);
+           wave_geometry(p, dtype, kWaveFilters, 0, &w, &ps, &nv);
 }
 
 // Workspace layout: [dSF partials over channel splits][dCF partials over strips],
 // each in the accumulator type and starting on a 256-byte boundary.
 size_t tiled_backward_workspace(const Problem &p, int dtype, unsigned need) {
     if (!(need & (DDF_NEED_DCF | DDF_NEED_DSF))) return 0;
-    TileGeom g; int ps;
-    if (!tiled_geometry(p, dtype, kKindFilters, &g, &ps)) return 0;
+    // csplit and nstrips do not depend on the access width, so the scalar
+    // fallback for misaligned pointers needs the same workspace
+    WaveGeom g; int ps, nv;
+    if (!wave_geometry(p, dtype, kWaveFilters, 0, &g, &ps, &nv)) return 0;
     const size_t asz = acc_size(dtype);
     size_t bytes = 0;
     if ((need & DDF_NEED_DSF) && g.csplit > 1)

@@ -5,13 +5,14 @@
 
 #include <type_traits>
 
-#include "ddf_tiled.h"
 #include "ddf_wave.h"
 
 namespace ddf {
 namespace tiled {
 
-inline unsigned padded_grid(int nblocks) { return (unsigned)((nblocks + kXcd - 1) / kXcd * kXcd); }
+inline unsigned padded_grid(int nblocks) {
+    return (unsigned)((nblocks + wave::kXcd - 1) / wave::kXcd * wave::kXcd);
+}
 
 // Expands BODY for the (K, D, S) of the problem; BODY sees constexpr KK_, DD_, SS_.
 #define DDF_DISPATCH_KDS(p, ...)                                           \
@@ -28,27 +29,6 @@ inline unsigned padded_grid(int nblocks) { return (unsigned)((nblocks + kXcd - 1
             case 522: { constexpr int KK_ = 5, DD_ = 2, SS_ = 2; __VA_ARGS__; } break; \
             default: return hipErrorNotSupported;                          \
         }                                                                  \
-    } while (0)
-
-// Elements per global access: the geometry's choice, unless a pointer is not
-// aligned to it.
-template <typename T>
-inline int usable_vec(const TileGeom &g, std::initializer_list<const void *> ptrs) {
-    int v = g.vec;
-    for (const void *p : ptrs)
-        while (v > 1 && (reinterpret_cast<uintptr_t>(p) % (v * sizeof(T))) != 0) v /= 2;
-    return v;
-}
-
-// The wide access (16 bytes), the narrow one (8 bytes) or single elements.
-template <typename T> constexpr int wide_vec() { return sizeof(T) == 8 ? 1 : 16 / sizeof(T); }
-template <typename T> constexpr int narrow_vec() { return sizeof(T) == 8 ? 1 : 8 / sizeof(T); }
-
-#define DDF_DISPATCH_VEC(T, v, ...)                                                  \
-    do {                                                                             \
-        if (sizeof(T) != 8 && (v) == wide_vec<T>()) { constexpr int VV_ = wide_vec<T>(); __VA_ARGS__; } \
-        else if (sizeof(T) != 8 && (v) == narrow_vec<T>()) { constexpr int VV_ = narrow_vec<T>(); __VA_ARGS__; } \
-        else { constexpr int VV_ = 1; __VA_ARGS__; }                                 \
     } while (0)
 
 // Largest power-of-two vector <= v to which every pointer is aligned.
@@ -104,22 +84,43 @@ hipError_t launch_features(const Problem &p, const WaveGeom &g, int ps, int nv, 
     return hipGetLastError();
 }
 
-template <typename T, int K, int D, int S, int PS>
-hipError_t launch_filters(const Problem &p, const TileGeom &g, const T *go, const T *x,
-                          const T *cf, const T *sf, T *dcf, T *dsf,
+// Filter gradients: 4 pixel slots per lane for k=3, 2 for k=5 (two register
+// sets per slot); V=4 with NV 1, 2, 4 and V=1 with NV 4 (and 8 for k=3).
+template <typename T, int K, int D, int S, int NV, int V>
+hipError_t launch_filters_nv(const Problem &p, const WaveGeom &g, const T *go, const T *x,
+                             const T *cf, const T *sf, T *dcf, T *dsf,
+                             typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
+                             unsigned need, hipStream_t st) {
+    constexpr int PS = K == 3 ? 4 : 2;
+    const dim3 grid(padded_grid(g.nblocks)), block(kWave * wave::kFilterWaves);
+    if (p.mul)
+        hipLaunchKernelGGL((wave::k_backward_filters<T, K, D, S, true, PS, NV, V>), grid, block,
+                           g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
+    else
+        hipLaunchKernelGGL((wave::k_backward_filters<T, K, D, S, false, PS, NV, V>), grid, block,
+                           g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
+    return hipGetLastError();
+}
+
+template <typename T, int K, int D, int S>
+hipError_t launch_filters(const Problem &p, const WaveGeom &g, int ps, int nv, const T *go,
+                          const T *x, const T *cf, const T *sf, T *dcf, T *dsf,
                           typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                           unsigned need, hipStream_t st) {
-    const dim3 grid(padded_grid(g.nblocks)), block(g.threads);
-    const int v = usable_vec<T>(g, {go, x});
-    DDF_DISPATCH_VEC(T, v, {
-        if (p.mul)
-            hipLaunchKernelGGL((k_backward_filters<T, K, D, S, true, PS, VV_>), grid, block,
-                               g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
-        else
-            hipLaunchKernelGGL((k_backward_filters<T, K, D, S, false, PS, VV_>), grid, block,
-                               g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
-    });
-    return hipGetLastError();
+    if (ps != (K == 3 ? 4 : 2)) return hipErrorNotSupported;
+#define DDF_FILTERS_CASE(NV_, V_)                                                             \
+    if (g.vec == V_ && nv == NV_)                                                             \
+        return launch_filters_nv<T, K, D, S, NV_, V_>(p, g, go, x, cf, sf, dcf, dsf, ws_sf,   \
+                                                      ws_cf, need, st);
+    if constexpr (sizeof(T) != 8) {
+        DDF_FILTERS_CASE(1, 4)
+        DDF_FILTERS_CASE(2, 4)
+        DDF_FILTERS_CASE(4, 4)
+    }
+    DDF_FILTERS_CASE(4, 1)
+    if constexpr (K == 3) { DDF_FILTERS_CASE(8, 1) }
+#undef DDF_FILTERS_CASE
+    return hipErrorNotSupported;
 }
 
 }  // namespace tiled
@@ -131,8 +132,13 @@ bool wave_plan(const Problem &p, int kind, std::initializer_list<const void *> p
                int *ps, int *nv) {
     const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
     if (!wave_geometry(p, dtype, kind, 0, g, ps, nv)) return false;
-    if (g->vec > 1 && !tiled::aligned_for<T>(g->vec, ptrs))
-        return wave_geometry(p, dtype, kind, 1, g, ps, nv);
+    if (g->vec > 1 && !tiled::aligned_for<T>(g->vec, ptrs)) {
+        // the workspace was sized for the aligned plan: the scalar plan must cut
+        // the problem the same way
+        const int th = g->TH, csplit = g->csplit;
+        if (!wave_geometry(p, dtype, kind, 1, g, ps, nv)) return false;
+        return g->TH == th && g->csplit == csplit;
+    }
     return true;
 }
 
@@ -140,7 +146,8 @@ template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf, T *out,
                          hipStream_t st) {
     WaveGeom g; int ps, nv;
-    if (!wave_plan<T>(p, kWaveForward, {x, out}, &g, &ps, &nv)) return hipErrorNotSupported;
+    if (!wave_plan<T>(p, kWaveForward, {x, out}, &g, &ps, &nv))
+        return generic_forward<T>(p, x, cf, sf, out, st);   // e.g. pointers not 16-byte aligned
     DDF_DISPATCH_KDS(p, return tiled::launch_forward<T, KK_, DD_, SS_>(p, g, ps, nv, x, cf, sf, out, st));
     return hipErrorNotSupported;
 }
@@ -153,14 +160,18 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     hipError_t err = hipSuccess;
     if (need & DDF_NEED_DX) {
         WaveGeom g; int ps, nv;
-        if (!wave_plan<T>(p, kWaveFeatures, {go, dx}, &g, &ps, &nv)) return hipErrorNotSupported;
-        DDF_DISPATCH_KDS(p, err = tiled::launch_features<T, KK_, DD_, SS_>(p, g, ps, nv, go, cf, sf, dx, st));
+        if (!wave_plan<T>(p, kWaveFeatures, {go, dx}, &g, &ps, &nv)) {
+            err = generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, DDF_NEED_DX, st);
+        } else {
+            DDF_DISPATCH_KDS(p, err = tiled::launch_features<T, KK_, DD_, SS_>(p, g, ps, nv, go, cf, sf, dx, st));
+        }
         if (err != hipSuccess) return err;
     }
     const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
     if (fneed) {
-        TileGeom g; int ps;
-        if (!tiled_geometry(p, dtype, kKindFilters, &g, &ps)) return hipErrorNotSupported;
+        WaveGeom g; int ps, nv;
+        if (!wave_plan<T>(p, kWaveFilters, {go, x}, &g, &ps, &nv))
+            return generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, fneed, st);
         // carve the workspace exactly as tiled_backward_workspace() sized it
         unsigned char *wp = static_cast<unsigned char *>(ws);
         A *ws_sf = nullptr, *ws_cf = nullptr;
@@ -170,26 +181,20 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
             wp += ((size_t)n_sf * g.csplit * sizeof(A) + 255) / 256 * 256;
         }
         if ((fneed & DDF_NEED_DCF) && g.nstrips > 1) ws_cf = reinterpret_cast<A *>(wp);
-        DDF_DISPATCH_KDS(p, do {
-            if (ps == 2)
-                err = tiled::launch_filters<T, KK_, DD_, SS_, 2>(p, g, go, x, cf, sf, dcf, dsf,
-                                                                 ws_sf, ws_cf, fneed, st);
-            else
-                err = tiled::launch_filters<T, KK_, DD_, SS_, 4>(p, g, go, x, cf, sf, dcf, dsf,
-                                                                 ws_sf, ws_cf, fneed, st);
-        } while (0));
+        DDF_DISPATCH_KDS(p, err = tiled::launch_filters<T, KK_, DD_, SS_>(
+                                p, g, ps, nv, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, fneed, st));
         if (err != hipSuccess) return err;
         if (ws_sf) {
             // dSF[n, t, pix] = sum over channel splits
             const int64_t inner = p.kk * p.Ho * p.Wo, total = p.N * inner;
-            hipLaunchKernelGGL((tiled::k_sum_partials<T>), dim3((unsigned)cdiv(total, 256)),
+            hipLaunchKernelGGL((wave::k_sum_partials<T>), dim3((unsigned)cdiv(total, 256)),
                                dim3(256), 0, st, ws_sf, dsf, p.N, g.csplit, inner);
             if ((err = hipGetLastError()) != hipSuccess) return err;
         }
         if (ws_cf) {
             // dCF[nc, t] = sum over strips
             const int64_t total = p.N * p.C * p.kk;
-            hipLaunchKernelGGL((tiled::k_sum_partials<T>), dim3((unsigned)cdiv(total, 256)),
+            hipLaunchKernelGGL((wave::k_sum_partials<T>), dim3((unsigned)cdiv(total, 256)),
                                dim3(256), 0, st, ws_cf, dcf, p.N * p.C, g.nstrips,
                                (int64_t)p.kk);
             if ((err = hipGetLastError()) != hipSuccess) return err;

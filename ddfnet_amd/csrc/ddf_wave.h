@@ -40,7 +40,9 @@ struct WaveGeom {
     int row0_off, col_off;    // source row of tile row 0 in strip 0; tile column of source column 0
     // result strip (out, or dX): `lin_cols` elements per row, `lin_rpc` rows per cell row
     int lin_cols, lin_rpc, lin_rows, lin_tile;
-    int cpw, csplit;          // channels per wave; number of channel ranges
+    int cpw, csplit;          // channels per wave; number of channel ranges (of cpw * waves per block)
+    int cpb;                  // channels per block (= cpw for the one-wave kernels)
+    int lds_wave_bytes;       // LDS of one wave (filter-gradient blocks hold four)
     int vec, nv;              // elements per global access; vectors per lane per channel strip
     unsigned src_magic;       // ceil(2^32 / src_cols); 0 when src_cols == 1
     int nblocks;              // = N * nstrips * csplit
@@ -89,8 +91,8 @@ struct WaveWork {
         n = rest / g.nstrips;
         row_first = strip * g.TH;
         nrows = min(g.TH, g.rows - row_first);
-        c_begin = cs * g.cpw;
-        c_end = min(g.C, c_begin + g.cpw);
+        c_begin = cs * g.cpb;
+        c_end = min(g.C, c_begin + g.cpb);
         return true;
     }
 };
@@ -225,7 +227,7 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
     A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kSpare);
 
     WaveWork ww;
-    if (!ww.init(g)) return;
+    if (!ww.init(g) || ww.c_end <= ww.c_begin) return;
     const int lane = threadIdx.x;
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
     const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
@@ -354,7 +356,7 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
     A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kSpare);
 
     WaveWork ww;
-    if (!ww.init(g)) return;
+    if (!ww.init(g) || ww.c_end <= ww.c_begin) return;
     const int lane = threadIdx.x;
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
     const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
@@ -464,9 +466,311 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
     }
 }
 
+// Linear strip (dO of the filter gradients) -> linear LDS copy, through
+// registers, V elements per access; lane l owns vectors l, l + 64, ...
+template <typename T, int V, int NG, int NST>
+struct LinStager {
+    int off[NG];                 // element offset inside the strip (clamped to 0 when unused)
+    bool used[NG];
+    Vec<T, V> v[NST][NG];
+    __device__ __forceinline__ void init(int n_elems, int lane) {
+#pragma unroll
+        for (int j = 0; j < NG; ++j) {
+            const int f = lane + j * kWave;
+            used[j] = f < n_elems / V;
+            off[j] = used[j] ? f * V : 0;
+        }
+    }
+    template <int ST>
+    __device__ __forceinline__ void issue(const T *__restrict__ strip) {
+#pragma unroll
+        for (int j = 0; j < NG; ++j)
+            v[ST][j] = *reinterpret_cast<const Vec<T, V> *>(strip + off[j]);
+    }
+    template <int ST>
+    __device__ __forceinline__ void commit(T *lds) const {
+#pragma unroll
+        for (int j = 0; j < NG; ++j)
+            if (used[j]) *reinterpret_cast<Vec<T, V> *>(lds + off[j]) = v[ST][j];
+    }
+};
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int CTRL>
+__device__ __forceinline__ double dpp_move(double v) {
+    const long long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), CTRL, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, 0xf, 0xf, false);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+
+// Value held by the partner lane of butterfly stage STAGE.  Stages 0, 1, 3
+// are swaps (lane^1, lane^2, lane^8); stage 2 rotates the 16-lane row by 4, so
+// a lane receives from the quad next to its own: after stage 3 the two
+// rotations have covered all four quads of the row.  Stages 4, 5 cross rows.
+template <int STAGE, typename A>
+__device__ __forceinline__ A lane_xchg(A v) {
+    if constexpr (STAGE == 0) return dpp_move<0xB1>(v);        // quad_perm [1,0,3,2]
+    else if constexpr (STAGE == 1) return dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (STAGE == 2) return dpp_move<0x124>(v);  // row_ror:4
+    else if constexpr (STAGE == 3) return dpp_move<0x128>(v);  // row_ror:8
+    else if constexpr (STAGE == 4) return __shfl_xor(v, 16, kWave);
+    else return __shfl_xor(v, 32, kWave);
+}
+
+// Sum each of N per-lane values over the 64 lanes of the wavefront.  At every
+// stage a lane keeps one half of its values and hands the other half to its
+// partner, so the work is ~3N instructions instead of 6N.  Returns the total
+// of the value whose index g_bfly_table<N> lists for this lane.
+template <int N, int STAGE, typename A>
+__device__ __forceinline__ A bfly_sum(const A (&v)[N], int lane) {
+    if constexpr (STAGE == 6) {
+        static_assert(N == 1, "at most 64 values");
+        return v[0];
+    } else {
+        constexpr int h = N / 2, M = h + (N & 1);
+        A nv[M];
+        const bool up = (lane >> STAGE) & 1;
+#pragma unroll
+        for (int j = 0; j < h; ++j) {
+            const A keep = up ? v[j + h] : v[j];
+            const A send = up ? v[j] : v[j + h];
+            nv[j] = keep + lane_xchg<STAGE>(send);
+        }
+        if constexpr (N & 1) nv[h] = v[2 * h] + lane_xchg<STAGE>(v[2 * h]);
+        return bfly_sum<M, STAGE + 1, A>(nv, lane);
+    }
+}
+
+// Index of the value whose total bfly_sum() leaves in `lane`: the same
+// keep/send choices replayed on indices, evaluated at compile time.
+constexpr int bfly_index_of(int n, int lane) {
+    int id[kWave] = {};
+    for (int i = 0; i < n; ++i) id[i] = i;
+    int cnt = n;
+    for (int stage = 0; stage < 6; ++stage) {
+        const int h = cnt / 2;
+        const bool up = (lane >> stage) & 1;
+        int nid[kWave] = {};
+        for (int j = 0; j < h; ++j) nid[j] = up ? id[j + h] : id[j];
+        if (cnt & 1) nid[h] = id[2 * h];
+        cnt = h + (cnt & 1);
+        for (int j = 0; j < cnt; ++j) id[j] = nid[j];
+    }
+    return id[0];
+}
+template <int N>
+struct BflyTable {
+    int tap[kWave];
+    constexpr BflyTable() : tap{} {
+        for (int l = 0; l < kWave; ++l) tap[l] = bfly_index_of(N, l);
+    }
+};
+template <int N>
+__device__ const BflyTable<N> g_bfly_table{};
+
+// Lanes below this bound hold every index at least once after the reduction.
+template <int N>
+constexpr int bfly_writers() {
+    int w = 1;
+    while (w < N) w *= 2;
+    return w < kWave ? w : kWave;
+}
+
+// ---------------------------------------------------------------------------
+// Gradients with respect to both filters.  Work cell = output pixel.  The
+// kFilterWaves waves of a block work on the same strip of the same sample and
+// take consecutive channel ranges of g.cpw channels each; in the channel walk
+// they are as independent as the waves of the other two kernels (private LDS
+// tiles, no barrier).  Per channel a lane forms gx[t] = dO * X_t once and
+// feeds it to both sums:
+//   dSF[t, pixel] += gx[t] * CF[c, t]      (register accumulator, over channels)
+//   dCF[c, t]     += gx[t] * SF[t, pixel]  (butterfly over the wave's lanes)
+// After the walk the waves add their dSF accumulators through LDS (the only
+// barriers of the kernel).  Partial sums over channel splits (dSF) and strips
+// (dCF) go to the workspace and are added up by k_sum_partials: no atomics, so
+// results are reproducible.
+// ---------------------------------------------------------------------------
+constexpr int kFilterWaves = 4;
+
+template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V>
+__global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
+    WaveGeom g, const T *__restrict__ go, const T *__restrict__ x,
+    const T *__restrict__ cf, const T *__restrict__ sf, T *__restrict__ dcf,
+    T *__restrict__ dsf, typename Acc<T>::type *__restrict__ ws_sf,
+    typename Acc<T>::type *__restrict__ ws_cf, unsigned need) {
+    using A = typename Acc<T>::type;
+    constexpr int KK = K * K;
+    using Stg = Stager<T, V, NV>;
+    constexpr int NST = Stg::NST;
+    constexpr int NG = (PS + V - 1) / V;
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    // private LDS of this wave: X tile, dO strip, taps
+    T *lds_in = reinterpret_cast<T *>(smem + (size_t)wave * g.lds_wave_bytes);
+    T *lds_go = lds_in + g.tile + kSpare;
+    A *taps = reinterpret_cast<A *>(lds_go + g.lin_tile + kSpare);
+
+    WaveWork ww;
+    if (!ww.init(g)) return;   // whole block leaves together
+    const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
+    const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
+    const int y0 = ww.row_first;
+    const bool want_cf = need & DDF_NEED_DCF, want_sf = need & DDF_NEED_DSF;
+    const int my_tap = g_bfly_table<KK>.tap[lane];
+    // this wave's channels inside the block's range
+    const int c_begin = min(ww.c_begin + wave * g.cpw, ww.c_end);
+    const int nch = min(g.cpw, ww.c_end - c_begin);
+    const int nch1 = max(nch, 1);   // a wave without channels still issues (harmless) loads
+
+    TapStager<KK, T, A> tst;
+    if (MUL) tst.issue(cf, ww.n * g.C + min(c_begin, g.C - 1), nch1, lane);
+
+    bool ok[PS];
+    int lb[PS], ob[PS];
+    A sfr[PS][KK], acc_sf[PS][KK];
+#pragma unroll
+    for (int m = 0; m < PS; ++m) {
+        const int row = g.slot_row[m] + lr, col = g.slot_col[m] + lc;
+        ok[m] = m < g.nslots && row < ww.nrows && col < g.cols;
+        lb[m] = (row * S) * g.P + col * S;     // lane-linear: no bank conflicts, idle lanes included
+        ob[m] = ok[m] ? row * g.Wo + col : 0;
+        const T *sfp = sf + (ww.n * KK * g.Ho + y0) * g.Wo + ob[m];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            sfr[m][t] = MUL ? (A)ld(sfp + t * oplane) : A(0);
+            acc_sf[m][t] = 0;
+        }
+    }
+
+    Stg stg;
+    stg.init(g, y0 * S + g.row0_off, lane);
+    LinStager<T, V, NG, NST> sgo;
+    sgo.init(ww.nrows * g.Wo, lane);
+    const int c_first = min(c_begin, g.C - 1);
+    const T *xs = x + (ww.n * g.C + c_first) * iplane;
+    const T *gs = go + (ww.n * g.C + c_first) * oplane + (int64_t)y0 * g.Wo;
+    stg.template issue<0>(xs);
+    sgo.template issue<0>(gs);
+    if constexpr (NST > 1) {
+        stg.template issue<1>(xs + (int64_t)min(1, nch1 - 1) * iplane);
+        sgo.template issue<1>(gs + (int64_t)min(1, nch1 - 1) * oplane);
+    }
+    if constexpr (NST > 2) {
+        stg.template issue<2>(xs + (int64_t)min(2, nch1 - 1) * iplane);
+        sgo.template issue<2>(gs + (int64_t)min(2, nch1 - 1) * oplane);
+        stg.template issue<3>(xs + (int64_t)min(3, nch1 - 1) * iplane);
+        sgo.template issue<3>(gs + (int64_t)min(3, nch1 - 1) * oplane);
+    }
+    zero_tile(lds_in, g.tile, lane);
+    if (MUL) tst.put(taps, nch, lane);
+    wave_sync();
+
+    auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        stg.template commit<ST>(lds_in);
+        sgo.template commit<ST>(lds_go);
+        stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch1 - 1) * iplane);
+        sgo.template issue<ST>(gs + (int64_t)min(ci + NST, nch1 - 1) * oplane);
+        wave_sync();
+        A w[KK];
+        if (MUL) load_taps<KK>(taps, ci, w);
+        A pcf[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) pcf[t] = 0;
+#pragma unroll
+        for (int m = 0; m < PS; ++m) {
+            if (m >= g.nslots) break;
+            // idle lanes read dO element 0 and are zeroed: they add nothing
+            const A gval = ok[m] ? (A)ld(lds_go + ob[m]) : A(0);
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const int t = i * K + j;
+                    const A gx = gval * (A)ld(lds_in + lb[m] + i * D * g.P + j * D);
+                    if (MUL) {
+                        acc_sf[m][t] += gx * w[t];
+                        pcf[t] += gx * sfr[m][t];
+                    } else {
+                        acc_sf[m][t] += gx;
+                        pcf[t] += gx;
+                    }
+                }
+        }
+        if (want_cf) {
+            const A tot = bfly_sum<KK, 0, A>(pcf, lane);
+            if (lane < bfly_writers<KK>()) {
+                const int64_t nc = ww.n * g.C + c_begin + ci;
+                if (g.nstrips == 1) st(dcf + nc * KK + my_tap, tot);
+                else ws_cf[(nc * g.nstrips + ww.strip) * KK + my_tap] = tot;
+            }
+        }
+        wave_sync();
+    };
+    auto group = [&](int c) __attribute__((always_inline)) {
+        channel(std::integral_constant<int, 0>{}, c);
+        if constexpr (NST > 1) channel(std::integral_constant<int, 1>{}, c + 1);
+        if constexpr (NST > 2) channel(std::integral_constant<int, 2>{}, c + 2);
+        if constexpr (NST > 3) channel(std::integral_constant<int, 3>{}, c + 3);
+    };
+    const int nfull = nch > 0 ? nch / NST * NST : 0;
+    if (nfull > 0) {
+        group(0);
+        for (int c = NST; c < nfull; c += NST) group(c);
+    }
+    if constexpr (NST > 1) {
+        if (nfull < nch) channel(std::integral_constant<int, 0>{}, nfull);
+        if constexpr (NST > 2) {
+            if (nfull + 1 < nch) channel(std::integral_constant<int, 1>{}, nfull + 1);
+            if (nfull + 2 < nch) channel(std::integral_constant<int, 2>{}, nfull + 2);
+        }
+    }
+
+    if (!want_sf) return;
+    // Add the waves' dSF accumulators: one pixel slot at a time through LDS.
+    __syncthreads();
+    A *red = reinterpret_cast<A *>(smem);
+#pragma unroll
+    for (int m = 0; m < PS; ++m) {
+        if (m >= g.nslots) break;
+#pragma unroll
+        for (int t = 0; t < KK; ++t) red[(wave * KK + t) * kWave + lane] = acc_sf[m][t];
+        __syncthreads();
+        const int64_t pix = (int64_t)y0 * g.Wo + ob[m];
+        for (int t = wave; t < KK; t += kFilterWaves) {
+            A tot = 0;
+#pragma unroll
+            for (int wv = 0; wv < kFilterWaves; ++wv) tot += red[(wv * KK + t) * kWave + lane];
+            if (ok[m]) {
+                if (g.csplit == 1) st(dsf + (ww.n * KK + t) * oplane + pix, tot);
+                else ws_sf[((ww.n * g.csplit + ww.cs) * KK + t) * oplane + pix] = tot;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// out[o, i] = sum_p part[o, p, i] for o < outer, p < parts, i < inner.
+template <typename T>
+__global__ __launch_bounds__(256) void k_sum_partials(
+    const typename Acc<T>::type *__restrict__ part, T *__restrict__ out, int64_t outer,
+    int parts, int64_t inner) {
+    using A = typename Acc<T>::type;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= outer * inner) return;
+    const int64_t o = idx / inner, i = idx - o * inner;
+    A tot = 0;
+    for (int p = 0; p < parts; ++p) tot += part[(o * parts + p) * inner + i];
+    st(out + idx, tot);
+}
+
 }  // namespace wave
 
-enum WaveKind { kWaveForward = 0, kWaveFeatures = 1 };
+enum WaveKind { kWaveForward = 0, kWaveFeatures = 1, kWaveFilters = 2 };
 // Host-side geometry (ddf_tiled_host.hip).  *ps and *nv select the kernel.
 // max_vec > 0 caps the elements per global access (1 = scalar accesses).
 bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom *g, int *ps,
