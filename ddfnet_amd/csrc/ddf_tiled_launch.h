@@ -146,7 +146,7 @@ template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf, T *out,
                          hipStream_t st) {
     WaveGeom g; int ps, nv;
-    if (!wave_plan<T>(p, kWaveForward, {x, out}, &g, &ps, &nv))
+    if (!wave_plan<T>(p, kWaveForward, {x, sf, out}, &g, &ps, &nv))
         return generic_forward<T>(p, x, cf, sf, out, st);   // e.g. pointers not 16-byte aligned
     DDF_DISPATCH_KDS(p, return tiled::launch_forward<T, KK_, DD_, SS_>(p, g, ps, nv, x, cf, sf, out, st));
     return hipErrorNotSupported;
@@ -160,7 +160,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     hipError_t err = hipSuccess;
     if (need & DDF_NEED_DX) {
         WaveGeom g; int ps, nv;
-        if (!wave_plan<T>(p, kWaveFeatures, {go, dx}, &g, &ps, &nv)) {
+        if (!wave_plan<T>(p, kWaveFeatures, {go, sf, dx}, &g, &ps, &nv)) {
             err = generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, DDF_NEED_DX, st);
         } else {
             DDF_DISPATCH_KDS(p, err = tiled::launch_features<T, KK_, DD_, SS_>(p, g, ps, nv, go, cf, sf, dx, st));
@@ -170,7 +170,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
     if (fneed) {
         WaveGeom g; int ps, nv;
-        if (!wave_plan<T>(p, kWaveFilters, {go, x}, &g, &ps, &nv))
+        if (!wave_plan<T>(p, kWaveFilters, {go, x, sf}, &g, &ps, &nv))
             return generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, fneed, st);
         // carve the workspace exactly as tiled_backward_workspace() sized it
         unsigned char *wp = static_cast<unsigned char *>(ws);

@@ -24,6 +24,11 @@
 
 #include "ddf_common.h"
 
+// Hook for a timing harness; expands to nothing in the library.
+#ifndef DDF_STAMP
+#define DDF_STAMP(slot)
+#endif
+
 namespace ddf {
 
 constexpr int kMaxSlots = 8;
@@ -61,6 +66,16 @@ template <typename T, int V>
 struct alignas(sizeof(T) * V) Vec {
     T e[V];
 };
+
+// Register image of V elements that are only moved, never computed on.
+template <int BYTES> struct RawBytes;
+template <> struct RawBytes<2> { using type = uint16_t; };
+template <> struct RawBytes<4> { using type = uint32_t; };
+template <> struct RawBytes<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct RawBytes<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <> struct RawBytes<32> { typedef uint32_t type __attribute__((ext_vector_type(8))); };
+template <typename T, int V>
+using Raw = typename RawBytes<sizeof(T) * V>::type;
 
 // Compiler-level ordering point between LDS writes and the reads of other
 // lanes of the same wavefront.  The LDS unit executes one wave's instructions
@@ -195,8 +210,8 @@ __device__ __forceinline__ void store_strip(const T *lds, T *__restrict__ dst, i
                                             int lane) {
     const int nvec = n_elems / V;
     for (int f = lane; f < nvec; f += kWave)
-        *reinterpret_cast<Vec<T, V> *>(dst + f * V) =
-            *reinterpret_cast<const Vec<T, V> *>(lds + f * V);
+        *reinterpret_cast<Raw<T, V> *>(dst + f * V) =
+            *reinterpret_cast<const Raw<T, V> *>(lds + f * V);
 }
 
 template <typename T>
@@ -208,6 +223,48 @@ __device__ __forceinline__ void zero_tile(T *lds, int n, int lane) {
     for (int k = 0; k < W16; ++k) z.e[k] = T(0.0f);
     for (int i = lane * W16; i < n; i += kWave * W16) *reinterpret_cast<Vec<T, W16> *>(lds + i) = z;
 }
+
+// Spatial-filter taps of a lane's cells.  A lane-per-cell gather would cost
+// KK * PS four-byte load instructions per wave, and at a few channels per wave
+// those loads, not the feature maps, fill the memory pipeline.  Instead the
+// strip of every tap plane is read as a linear run with V-element accesses (NG
+// per lane and tap), passed through a linear LDS buffer and picked up per cell.
+template <typename T, int V, int NG, int KK>
+struct FilterStager {
+    int off[NG];   // element offset inside the strip; lanes past its end repeat vector 0
+    Raw<T, V> v[KK][NG];
+    __device__ __forceinline__ void init(int n_elems, int lane) {
+#pragma unroll
+        for (int j = 0; j < NG; ++j) {
+            const int f = lane + j * kWave;
+            off[j] = f < n_elems / V ? f * V : 0;
+        }
+    }
+    // tap t of the strip starts at strip0 + t * plane
+    template <int TT = 0>
+    __device__ __forceinline__ void issue(const T *__restrict__ strip0, int64_t plane) {
+        if constexpr (TT < KK) {
+#pragma unroll
+            for (int j = 0; j < NG; ++j)
+                v[TT][j] = *reinterpret_cast<const Raw<T, V> *>(strip0 + TT * plane + off[j]);
+            issue<TT + 1>(strip0, plane);
+        }
+    }
+    // lds: at least n_elems elements; idx[m]: element of the lane's cell m
+    template <int TT = 0, int PS, typename A>
+    __device__ __forceinline__ void collect(T *lds, const int (&idx)[PS], A (&sfr)[PS][KK]) const {
+        if constexpr (TT < KK) {
+#pragma unroll
+            for (int j = 0; j < NG; ++j)
+                *reinterpret_cast<Raw<T, V> *>(lds + off[j]) = v[TT][j];
+            wave_sync();
+#pragma unroll
+            for (int m = 0; m < PS; ++m) sfr[m][TT] = ld(lds + idx[m]);
+            wave_sync();
+            collect<TT + 1>(lds, idx, sfr);
+        }
+    }
+};
 
 // ---------------------------------------------------------------------------
 // Forward: work cell = output pixel.
@@ -226,6 +283,7 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
     T *lds_out = lds_in + g.tile + kSpare;
     A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kSpare);
 
+    DDF_STAMP(0);
     WaveWork ww;
     if (!ww.init(g) || ww.c_end <= ww.c_begin) return;
     const int lane = threadIdx.x;
@@ -251,12 +309,11 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
         // allocation): a shared dummy address would collide with the banks of
         // the working lanes and double the time of every tap read
         lb[m] = (row * S) * g.P + col * S;
-        ob[m] = ok[m] ? row * g.Wo + col : 0;
-        // idle lanes read pixel 0 of the strip: no branch around the loads
-        const T *sfp = sf + (ww.n * KK * g.Ho + y0) * g.Wo + ob[m];
-#pragma unroll
-        for (int t = 0; t < KK; ++t) sfr[m][t] = ld(sfp + t * oplane);
+        ob[m] = ok[m] ? row * g.Wo + col : 0;   // idle lanes pick up pixel 0 (unused)
     }
+    FilterStager<T, V, (PS + V - 1) / V, KK> fst;
+    fst.init(n_out, lane);
+    fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
 
     Stg stg;
     stg.init(g, y0 * S + g.row0_off, lane);
@@ -269,17 +326,21 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
     if constexpr (NST > 1) stg.template issue<1>(xs + (int64_t)min(1, nch - 1) * iplane);
     if constexpr (NST > 2) stg.template issue<2>(xs + (int64_t)min(2, nch - 1) * iplane);
     if constexpr (NST > 3) stg.template issue<3>(xs + (int64_t)min(3, nch - 1) * iplane);
+    DDF_STAMP(1);
     zero_tile(lds_in, g.tile, lane);
     tst.put(taps, nch, lane);
-    wave_sync();
+    fst.collect(lds_out, ob, sfr);
+    DDF_STAMP(2);
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         stg.template commit<ST>(lds_in);
+        DDF_STAMP(3 + 4 * ci);
         stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch - 1) * iplane);
         wave_sync();
         A w[KK];
         load_taps<KK>(taps, ci, w);
+        DDF_STAMP(4 + 4 * ci);
 #pragma unroll
         for (int m = 0; m < PS; ++m) {
             if (m >= g.nslots) break;
@@ -293,8 +354,10 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
             if (ok[m]) st(lds_out + ob[m], acc);
         }
         wave_sync();
+        DDF_STAMP(5 + 4 * ci);
         store_strip<T, V>(lds_out, os + (int64_t)ci * oplane, n_out, lane);
         wave_sync();
+        DDF_STAMP(6 + 4 * ci);
     };
 
     auto group = [&](int c) __attribute__((always_inline)) {
@@ -341,6 +404,46 @@ struct TapMap {
     static constexpr int halo_hi = (R * D + S - 1) / S;    // cells below / right
 };
 
+// Spatial-filter taps at the neighbour positions of a lane's cells.  Each tap
+// plane has the shape of dO, so its strip is brought in exactly like a dO strip
+// (same vector offsets, same zero-bordered tile: neighbours outside the image
+// read as zero) and every cell picks its neighbour out of the tile.
+template <typename T, int V, int NV, int K, int D, int S>
+struct NeighbourFilterStager {
+    static constexpr int KK = K * K;
+    using TM = TapMap<K, D, S>;
+    Vec<T, V> v[KK][NV];
+    template <int TT = 0>
+    __device__ __forceinline__ void issue(const T *__restrict__ sf_n, int64_t plane,
+                                          const int (&goff)[NV]) {
+        if constexpr (TT < KK) {
+#pragma unroll
+            for (int j = 0; j < NV; ++j)
+                v[TT][j] = *reinterpret_cast<const Vec<T, V> *>(sf_n + TT * plane + goff[j]);
+            issue<TT + 1>(sf_n, plane, goff);
+        }
+    }
+    template <int TT = 0, int PS, typename A>
+    __device__ __forceinline__ void collect(T *tile, const int (&lo)[NV][V],
+                                            const int (&lb)[PS], int P,
+                                            A (&sfg)[PS][KK]) const {
+        if constexpr (TT < KK) {
+            constexpr int i = TT / K, j = TT % K;
+#pragma unroll
+            for (int q = 0; q < NV; ++q)
+#pragma unroll
+                for (int k = 0; k < V; ++k) tile[lo[q][k]] = v[TT][q].e[k];
+            wave_sync();
+#pragma unroll
+            for (int m = 0; m < PS; ++m)
+                sfg[m][TT] = ld(tile + lb[m] + (TM::dq(i) + TM::halo_lo) * P + TM::dq(j) +
+                                TM::halo_lo);
+            wave_sync();
+            collect<TT + 1>(tile, lo, lb, P, sfg);
+        }
+    }
+};
+
 template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V>
 __global__ __launch_bounds__(kWave) void k_backward_features(
     WaveGeom g, const T *__restrict__ go, const T *__restrict__ cf,
@@ -379,21 +482,32 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
         // idle cells get coordinates outside the image: none of their results is kept
         cu[m] = ok[m] ? cy * S : g.H;
         cv[m] = cx * S;
-#pragma unroll
-        for (int i = 0; i < K; ++i)
-#pragma unroll
-            for (int j = 0; j < K; ++j) {
-                const int sy = cy + TM::dq(i), sx = cx + TM::dq(j);
-                const bool in = ok[m] && sy >= 0 && sy < g.Ho && sx >= 0 && sx < g.Wo;
-                // out-of-range neighbours read element 0 and are zeroed: no branch
-                const A val = ld(sf + (ww.n * KK + i * K + j) * oplane +
-                                 (in ? (int64_t)sy * g.Wo + sx : 0));
-                sfg[m][i * K + j] = in ? val : A(0);
-            }
     }
-
     Stg stg;
     stg.init(g, qy0 + g.row0_off, lane);
+    // Few vectors per plane: bring the filter in through the tile.  Otherwise
+    // (scalar accesses, or more registers than the taps themselves) gather it.
+    constexpr bool kStageFilter = V > 1 && NV * V <= 8;
+    NeighbourFilterStager<T, V, kStageFilter ? NV : 1, K, D, S> nfs;
+    if constexpr (kStageFilter) {
+        nfs.issue(sf + ww.n * KK * oplane, oplane, stg.goff);
+    } else {
+#pragma unroll
+        for (int m = 0; m < PS; ++m) {
+            const int cy = qy0 + g.slot_row[m] + lr, cx = g.slot_col[m] + lc;
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const int sy = cy + TM::dq(i), sx = cx + TM::dq(j);
+                    const bool in = ok[m] && sy >= 0 && sy < g.Ho && sx >= 0 && sx < g.Wo;
+                    // out-of-range neighbours read element 0 and are zeroed: no branch
+                    const A val = ld(sf + (ww.n * KK + i * K + j) * oplane +
+                                     (in ? (int64_t)sy * g.Wo + sx : 0));
+                    sfg[m][i * K + j] = in ? val : A(0);
+                }
+        }
+    }
     const T *gs = go + (ww.n * g.C + ww.c_begin) * oplane;
     T *ds = dx + (ww.n * g.C + ww.c_begin) * iplane + (int64_t)u0 * g.W;
     const int nch = ww.c_end - ww.c_begin;
@@ -404,6 +518,7 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
     zero_tile(lds_in, g.tile, lane);
     tst.put(taps, nch, lane);
     wave_sync();
+    if constexpr (kStageFilter) nfs.collect(lds_in, stg.lo, lb, g.P, sfg);
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
@@ -470,28 +585,26 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
 // registers, V elements per access; lane l owns vectors l, l + 64, ...
 template <typename T, int V, int NG, int NST>
 struct LinStager {
-    int off[NG];                 // element offset inside the strip (clamped to 0 when unused)
-    bool used[NG];
-    Vec<T, V> v[NST][NG];
+    int off[NG];   // element offset inside the strip; lanes past its end repeat vector 0
+    Raw<T, V> v[NST][NG];
     __device__ __forceinline__ void init(int n_elems, int lane) {
 #pragma unroll
         for (int j = 0; j < NG; ++j) {
             const int f = lane + j * kWave;
-            used[j] = f < n_elems / V;
-            off[j] = used[j] ? f * V : 0;
+            off[j] = f < n_elems / V ? f * V : 0;
         }
     }
     template <int ST>
     __device__ __forceinline__ void issue(const T *__restrict__ strip) {
 #pragma unroll
         for (int j = 0; j < NG; ++j)
-            v[ST][j] = *reinterpret_cast<const Vec<T, V> *>(strip + off[j]);
+            v[ST][j] = *reinterpret_cast<const Raw<T, V> *>(strip + off[j]);
     }
     template <int ST>
     __device__ __forceinline__ void commit(T *lds) const {
 #pragma unroll
         for (int j = 0; j < NG; ++j)
-            if (used[j]) *reinterpret_cast<Vec<T, V> *>(lds + off[j]) = v[ST][j];
+            *reinterpret_cast<Raw<T, V> *>(lds + off[j]) = v[ST][j];
     }
 };
 
@@ -638,12 +751,16 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         ok[m] = m < g.nslots && row < ww.nrows && col < g.cols;
         lb[m] = (row * S) * g.P + col * S;     // lane-linear: no bank conflicts, idle lanes included
         ob[m] = ok[m] ? row * g.Wo + col : 0;
-        const T *sfp = sf + (ww.n * KK * g.Ho + y0) * g.Wo + ob[m];
 #pragma unroll
         for (int t = 0; t < KK; ++t) {
-            sfr[m][t] = MUL ? (A)ld(sfp + t * oplane) : A(0);
+            sfr[m][t] = 0;
             acc_sf[m][t] = 0;
         }
+    }
+    FilterStager<T, V, NG, KK> fst;
+    if (MUL) {
+        fst.init(ww.nrows * g.Wo, lane);
+        fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
     }
 
     Stg stg;
@@ -666,7 +783,10 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         sgo.template issue<3>(gs + (int64_t)min(3, nch1 - 1) * oplane);
     }
     zero_tile(lds_in, g.tile, lane);
-    if (MUL) tst.put(taps, nch, lane);
+    if (MUL) {
+        tst.put(taps, nch, lane);
+        fst.collect(lds_go, ob, sfr);
+    }
     wave_sync();
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
