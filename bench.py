@@ -49,6 +49,9 @@ WORKLOADS = {
 DEFAULT_WORKLOAD = 'r50_stage3_mul_fp32'
 DTYPE_NAME = {torch.float32: 'f32', torch.float16: 'f16', torch.float64: 'f64'}
 PHASES = ('fwd', 'dx', 'dfilters')
+# kernels behind each phase (one library call each)
+PHASE_KERNELS = {'fwd': 'ddf::wave::k_forward', 'dx': 'ddf::wave::k_backward_features',
+                 'dfilters': 'ddf::wave::k_backward_filters + ddf::wave::k_sum_partials'}
 
 
 def log(*a):
@@ -153,6 +156,18 @@ def timed(fn, count):
     stop.record()
     torch.cuda.synchronize()
     return start.elapsed_time(stop) / count
+
+
+# HBM bytes per library call of a phase, from hardware counters: two
+# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per
+# dispatch, summed over the kernels of the call), each scaled by what the same
+# counter reads for the 256 MiB device copy of --copy-probe (fetch x2.000,
+# write x1.000 on MI355X).  Counters cannot be read from inside a timed run, so
+# the figures are recorded here; a workload or phase that was not profiled
+# reports null.
+MEASURED_TRAFFIC = {
+    'r50_stage3_mul_fp32': {'fwd': 26885000, 'dx': 26895000, 'dfilters': 35840000},
+}
 
 
 def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
@@ -311,9 +326,10 @@ def main():
             'buffer_sets': res['buffer_sets']},
         'pct_of_hbm_peak': round(100 * res['gbps'] / HBM_PEAK_GBPS, 2),
         'images_per_s': round(res['images_per_s'], 1),
-        'roofline': {'bound': 'hbm', 'kernel': dominant, 'achieved': round(achieved, 2),
+        'roofline': {'bound': 'hbm', 'phase': dominant, 'kernel': PHASE_KERNELS[dominant], 'achieved': round(achieved, 2),
                      'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': None,
+                     'frac': round(achieved / HBM_PEAK_GBPS, 4),
+                     'traffic': MEASURED_TRAFFIC.get(res['workload'], {}).get(dominant),
                      'bytes_per_launch': dom_bytes,
                      'avg_launch_us': round(dom_s * 1e6, 3)},
         'phases_us': {p: round(res['phase_ms'][p] * 1e3, 3) for p in PHASES},
