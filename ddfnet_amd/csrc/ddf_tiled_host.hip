@@ -34,6 +34,7 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     if (p.N <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0) return false;
     if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
     const int esz = elem_size(dtype);
+    const int asz = (int)acc_size(dtype);
     const int K = p.k, D = p.d, S = p.s, R = p.r;
     const int H = (int)p.H, W = (int)p.W, Ho = (int)p.Ho, Wo = (int)p.Wo, C = (int)p.C;
 
@@ -128,8 +129,8 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
         }
         if (nv == 0) continue;
         const int nstrips = (t.rows + th - 1) / th;
-        const int64_t lds = (int64_t)esz * (2 * round_up(tile_rows(th) * t.P, 8) + 2 * wave::kSpare +
-                                            round_up(th * t.lin_rpc * t.lin_cols, 8)) + 4096;
+        const int64_t lds = (int64_t)asz * (2 * round_up(tile_rows(th) * t.P, 8) + wave::kSpare) +
+                            (int64_t)esz * (wave::kIdle + round_up(th * t.lin_rpc * t.lin_cols, 8)) + 4096;
         if (lds > 64 * 1024) continue;
         const int slots_used = ((th + RS - 1) / RS) * cseg;
         double cost = (double)nstrips * (slots_used * kWave * 2.0 * p.kk +
@@ -177,8 +178,9 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     t.cpb = cpw * waves_per_block;
     t.csplit = (C + t.cpb - 1) / t.cpb;
     // per wave: tiles, then the channel-filter taps of its channels (accumulator type)
-    t.lds_wave_bytes = round_up((t.tile + t.lin_tile + 2 * wave::kSpare) * esz +
-                                cpw * ((p.kk + 3) / 4 * 4) * acc_size(dtype), 16);
+    // per wave: tile (accumulator type), linear strip (storage type), taps
+    t.lds_wave_bytes = round_up((t.tile + wave::kSpare) * asz + (t.lin_tile + wave::kIdle) * esz +
+                                cpw * ((p.kk + 3) / 4 * 4) * asz, 16);
     t.lds_bytes = t.lds_wave_bytes * waves_per_block;
     if (filters)  // the cross-wave sum of the dSF accumulators reuses the block's LDS
         t.lds_bytes = std::max(t.lds_bytes, waves_per_block * p.kk * kWave * acc_size(dtype));
@@ -186,6 +188,12 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     t.src_magic = t.src_cols == 1 ? 0u : (unsigned)((0x100000000ull + t.src_cols - 1) / t.src_cols);
     const int64_t nblocks = base * t.csplit;
     if (nblocks > (1 << 30)) return false;
+    // magic-number division of the block id is exact while id * divisor < 2^32
+    if (nblocks * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
+    auto magic = [](int d) { return d == 1 ? 0u : (unsigned)((0x100000000ull + d - 1) / d); };
+    t.csplit_magic = magic(t.csplit);
+    t.nstrips_magic = magic(t.nstrips);
+    t.xcd_per = (unsigned)((nblocks + wave::kXcd - 1) / wave::kXcd);
     t.nblocks = (int)nblocks;
     *g = t;
     *ps_out = best_ps;

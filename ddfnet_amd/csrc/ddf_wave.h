@@ -50,6 +50,7 @@ struct WaveGeom {
     int lds_wave_bytes;       // LDS of one wave (filter-gradient blocks hold four)
     int vec, nv;              // elements per global access; vectors per lane per channel strip
     unsigned src_magic;       // ceil(2^32 / src_cols); 0 when src_cols == 1
+    unsigned csplit_magic, nstrips_magic, xcd_per;   // same for the block id split; blocks per XCD
     int nblocks;              // = N * nstrips * csplit
     int lds_bytes;
     int slot_row[kMaxSlots];  // cell row (within the strip) of lane row 0 in slot m
@@ -61,6 +62,9 @@ namespace wave {
 constexpr int kXcd = 8;
 // Spare LDS elements behind each tile: idle lanes write there instead of branching.
 constexpr int kSpare = 8;
+// Spare elements behind each linear result strip: one per lane, where idle
+// lanes put their (meaningless) results without an address conflict.
+constexpr int kIdle = kWave;
 
 template <typename T, int V>
 struct alignas(sizeof(T) * V) Vec {
@@ -89,21 +93,32 @@ __device__ __forceinline__ void wave_sync() {
 // Workgroups are handed to the 8 XCDs round-robin by hardware.  Renumber them
 // so that consecutive logical blocks (same sample, neighbouring channel
 // ranges: same spatial filter) share an XCD and its L2.
-__device__ __forceinline__ int logical_block(int nblocks) {
-    const int per = (nblocks + kXcd - 1) / kXcd;
-    return (int)(blockIdx.x % kXcd) * per + (int)(blockIdx.x / kXcd);
+// q = n / d through the host's magic number m = ceil(2^32 / d) (0: d == 1);
+// exact while n * d < 2^32, which the host checks.
+__device__ __forceinline__ int magic_div(int n, unsigned m) {
+    return m ? (int)__umulhi((unsigned)n, m) : n;
+}
+
+// Pins a wave-uniform value in a scalar register.  Without it the compiler
+// re-reads kernel arguments from memory inside the channel loop, and the wait
+// for such a read also waits for every LDS access in flight.
+__device__ __forceinline__ int pin(int v) {
+    v = __builtin_amdgcn_readfirstlane(v);
+    asm volatile("" : "+s"(v));
+    return v;
 }
 
 struct WaveWork {
     int cs, strip, row_first, nrows, c_begin, c_end;
     int64_t n;
     __device__ __forceinline__ bool init(const WaveGeom &g) {
-        const int b = logical_block(g.nblocks);
+        const int b = (int)(blockIdx.x % kXcd) * (int)g.xcd_per + (int)(blockIdx.x / kXcd);
         if (b >= g.nblocks) return false;
-        cs = b % g.csplit;
-        const int rest = b / g.csplit;
-        strip = rest % g.nstrips;
-        n = rest / g.nstrips;
+        const int rest = magic_div(b, g.csplit_magic);
+        cs = b - rest * g.csplit;
+        const int smp = magic_div(rest, g.nstrips_magic);
+        strip = rest - smp * g.nstrips;
+        n = smp;
         row_first = strip * g.TH;
         nrows = min(g.TH, g.rows - row_first);
         c_begin = cs * g.cpb;
@@ -169,7 +184,19 @@ struct Stager {
     // behind the tile, so that neither issue() nor commit() branches: the
     // compiler then counts outstanding loads exactly and a commit waits only
     // for its own stage.
-    __device__ __forceinline__ void init(const WaveGeom &g, int row0, int lane) {
+    // init_global() is all that issue() needs; init_tile() (the costly part)
+    // can run while the first loads are in flight.
+    __device__ __forceinline__ void init_global(const WaveGeom &g, int row0, int lane) {
+        const int r_lo = max(row0, 0);
+        const int n_rows = max(min(row0 + g.IH, g.src_rows) - r_lo, 0);
+        const int nvec = n_rows * g.src_cols / V;
+#pragma unroll
+        for (int j = 0; j < NV; ++j) {
+            const int f = lane + j * kWave;
+            goff[j] = f < nvec ? r_lo * g.src_cols + f * V : 0;
+        }
+    }
+    __device__ __forceinline__ void init_tile(const WaveGeom &g, int row0, int lane) {
         const int r_lo = max(row0, 0);
         const int n_rows = max(min(row0 + g.IH, g.src_rows) - r_lo, 0);
         const int nvec = n_rows * g.src_cols / V;
@@ -178,10 +205,9 @@ struct Stager {
         for (int j = 0; j < NV; ++j) {
             const int f = lane + j * kWave;
             const int e = f * V;
-            int row = g.src_magic ? (int)__umulhi((unsigned)e, g.src_magic) : e;
+            int row = magic_div(e, g.src_magic);
             int col = e - row * g.src_cols;
             const bool used = f < nvec;
-            goff[j] = used ? r_lo * g.src_cols + e : 0;
 #pragma unroll
             for (int k = 0; k < V; ++k) {
                 lo[j][k] = used ? (row_shift + row) * g.P + g.col_off + col : g.tile + k;
@@ -189,18 +215,25 @@ struct Stager {
             }
         }
     }
+    __device__ __forceinline__ void init(const WaveGeom &g, int row0, int lane) {
+        init_global(g, row0, lane);
+        init_tile(g, row0, lane);
+    }
     template <int ST>
     __device__ __forceinline__ void issue(const T *__restrict__ plane) {
 #pragma unroll
         for (int j = 0; j < NV; ++j)
             v[ST][j] = *reinterpret_cast<const Vec<T, V> *>(plane + goff[j]);
     }
+    // The tile holds accumulator-type values: fp16 is widened here, once per
+    // element, instead of once per tap read; the tap reads are then aligned
+    // 4-byte accesses for every storage type.
     template <int ST>
-    __device__ __forceinline__ void commit(T *lds) const {
+    __device__ __forceinline__ void commit(typename Acc<T>::type *lds) const {
 #pragma unroll
         for (int j = 0; j < NV; ++j)
 #pragma unroll
-            for (int k = 0; k < V; ++k) lds[lo[j][k]] = v[ST][j].e[k];
+            for (int k = 0; k < V; ++k) lds[lo[j][k]] = ld(&v[ST][j].e[k]);
     }
 };
 
@@ -276,12 +309,13 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
                                                    T *__restrict__ out) {
     using A = typename Acc<T>::type;
     constexpr int KK = K * K;
+    constexpr bool kFlat = KK <= 9;   // tap loop without branches (see there)
     using Stg = Stager<T, V, NV>;
     constexpr int NST = Stg::NST;
     extern __shared__ __align__(16) unsigned char smem[];
-    T *lds_in = reinterpret_cast<T *>(smem);
-    T *lds_out = lds_in + g.tile + kSpare;
-    A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kSpare);
+    A *lds_in = reinterpret_cast<A *>(smem);
+    T *lds_out = reinterpret_cast<T *>(lds_in + g.tile + kSpare);
+    A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kIdle);
 
     DDF_STAMP(0);
     WaveWork ww;
@@ -290,16 +324,32 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
     const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
     const int y0 = ww.row_first;
-    // every load of the prologue is issued before the first wait: the wave pays
-    // one trip to memory, not one per tensor
-    TapStager<KK, T, A> tst;
-    tst.issue(cf, ww.n * g.C + ww.c_begin, ww.c_end - ww.c_begin, lane);
+    const int nch = ww.c_end - ww.c_begin;
     const int n_out = ww.nrows * g.Wo;
+    // Every load of the prologue is issued before anything else is set up and
+    // before the first wait: the feature strips of the first NST channels
+    // (clamped to the last channel, so that they are unconditional), the
+    // spatial filter, the channel-filter taps.  The index arithmetic below
+    // then runs under one trip to memory.
+    Stg stg;
+    stg.init_global(g, y0 * S + g.row0_off, lane);
+    const T *xs = x + (ww.n * g.C + ww.c_begin) * iplane;
+    T *os = out + (ww.n * g.C + ww.c_begin) * oplane + (int64_t)y0 * g.Wo;
+    stg.template issue<0>(xs);
+    if constexpr (NST > 1) stg.template issue<1>(xs + (int64_t)min(1, nch - 1) * iplane);
+    if constexpr (NST > 2) stg.template issue<2>(xs + (int64_t)min(2, nch - 1) * iplane);
+    if constexpr (NST > 3) stg.template issue<3>(xs + (int64_t)min(3, nch - 1) * iplane);
+    FilterStager<T, V, (PS + V - 1) / V, KK> fst;
+    fst.init(n_out, lane);
+    fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
+    TapStager<KK, T, A> tst;
+    tst.issue(cf, ww.n * g.C + ww.c_begin, nch, lane);
+    DDF_STAMP(1);
 
     // per slot: is the cell real, where its taps start in the tile, where its
     // result goes in the linear strip; its spatial-filter taps in registers
     bool ok[PS];
-    int lb[PS], ob[PS];
+    int lb[PS], ob[PS], wb[PS];
     A sfr[PS][KK];
 #pragma unroll
     for (int m = 0; m < PS; ++m) {
@@ -310,23 +360,10 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
         // the working lanes and double the time of every tap read
         lb[m] = (row * S) * g.P + col * S;
         ob[m] = ok[m] ? row * g.Wo + col : 0;   // idle lanes pick up pixel 0 (unused)
+        wb[m] = ok[m] ? ob[m] : g.lin_tile + lane;   // ... and write behind the strip
     }
-    FilterStager<T, V, (PS + V - 1) / V, KK> fst;
-    fst.init(n_out, lane);
-    fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
-
-    Stg stg;
-    stg.init(g, y0 * S + g.row0_off, lane);
-    const T *xs = x + (ww.n * g.C + ww.c_begin) * iplane;
-    T *os = out + (ww.n * g.C + ww.c_begin) * oplane + (int64_t)y0 * g.Wo;
-    const int nch = ww.c_end - ww.c_begin;
-    // start the first NST channels' loads (clamped to the last channel, so that
-    // they are unconditional), then clear the tile under them
-    stg.template issue<0>(xs);
-    if constexpr (NST > 1) stg.template issue<1>(xs + (int64_t)min(1, nch - 1) * iplane);
-    if constexpr (NST > 2) stg.template issue<2>(xs + (int64_t)min(2, nch - 1) * iplane);
-    if constexpr (NST > 3) stg.template issue<3>(xs + (int64_t)min(3, nch - 1) * iplane);
-    DDF_STAMP(1);
+    stg.init_tile(g, y0 * S + g.row0_off, lane);
+    const int P = pin(g.P);
     zero_tile(lds_in, g.tile, lane);
     tst.put(taps, nch, lane);
     fst.collect(lds_out, ob, sfr);
@@ -341,17 +378,39 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
         A w[KK];
         load_taps<KK>(taps, ci, w);
         DDF_STAMP(4 + 4 * ci);
+        if constexpr (kFlat) {
+            // No branch in here: every slot is computed, idle lanes and idle
+            // slots included (their tile addresses are valid), and the results
+            // are written after all reads (a write in between would order the
+            // reads of the next slot behind it).  The compiler can then overlap
+            // the LDS reads of one slot with the arithmetic of another.
+            A acc[PS];
 #pragma unroll
-        for (int m = 0; m < PS; ++m) {
-            if (m >= g.nslots) break;
-            A acc = 0;
+            for (int m = 0; m < PS; ++m) {
+                acc[m] = 0;
 #pragma unroll
-            for (int i = 0; i < K; ++i)
+                for (int i = 0; i < K; ++i)
 #pragma unroll
-                for (int j = 0; j < K; ++j)
-                    acc += (A)ld(lds_in + lb[m] + i * D * g.P + j * D) *
-                           comb<MUL, A>(w[i * K + j], sfr[m][i * K + j]);
-            if (ok[m]) st(lds_out + ob[m], acc);
+                    for (int j = 0; j < K; ++j)
+                        acc[m] += (A)ld(lds_in + lb[m] + i * D * P + j * D) *
+                                  comb<MUL, A>(w[i * K + j], sfr[m][i * K + j]);
+            }
+#pragma unroll
+            for (int m = 0; m < PS; ++m) st(lds_out + wb[m], acc[m]);
+        } else {
+            // many taps: one slot at a time keeps the register count down
+#pragma unroll
+            for (int m = 0; m < PS; ++m) {
+                if (m >= g.nslots) break;
+                A acc = 0;
+#pragma unroll
+                for (int i = 0; i < K; ++i)
+#pragma unroll
+                    for (int j = 0; j < K; ++j)
+                        acc += (A)ld(lds_in + lb[m] + i * D * P + j * D) *
+                               comb<MUL, A>(w[i * K + j], sfr[m][i * K + j]);
+                if (ok[m]) st(lds_out + ob[m], acc);
+            }
         }
         wave_sync();
         DDF_STAMP(5 + 4 * ci);
@@ -424,7 +483,7 @@ struct NeighbourFilterStager {
         }
     }
     template <int TT = 0, int PS, typename A>
-    __device__ __forceinline__ void collect(T *tile, const int (&lo)[NV][V],
+    __device__ __forceinline__ void collect(A *tile, const int (&lo)[NV][V],
                                             const int (&lb)[PS], int P,
                                             A (&sfg)[PS][KK]) const {
         if constexpr (TT < KK) {
@@ -432,7 +491,7 @@ struct NeighbourFilterStager {
 #pragma unroll
             for (int q = 0; q < NV; ++q)
 #pragma unroll
-                for (int k = 0; k < V; ++k) tile[lo[q][k]] = v[TT][q].e[k];
+                for (int k = 0; k < V; ++k) tile[lo[q][k]] = ld(&v[TT][q].e[k]);
             wave_sync();
 #pragma unroll
             for (int m = 0; m < PS; ++m)
@@ -451,12 +510,13 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
     using A = typename Acc<T>::type;
     using TM = TapMap<K, D, S>;
     constexpr int KK = K * K;
+    constexpr bool kFlat = KK <= 9 && S == 1;   // tap loop without branches (see k_forward)
     using Stg = Stager<T, V, NV>;
     constexpr int NST = Stg::NST;
     extern __shared__ __align__(16) unsigned char smem[];
-    T *lds_in = reinterpret_cast<T *>(smem);
-    T *lds_out = lds_in + g.tile + kSpare;
-    A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kSpare);
+    A *lds_in = reinterpret_cast<A *>(smem);
+    T *lds_out = reinterpret_cast<T *>(lds_in + g.tile + kSpare);
+    A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kIdle);
 
     WaveWork ww;
     if (!ww.init(g) || ww.c_end <= ww.c_begin) return;
@@ -464,10 +524,25 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
     const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
     const int qy0 = ww.row_first;
-    TapStager<KK, T, A> tst;
-    tst.issue(cf, ww.n * g.C + ww.c_begin, ww.c_end - ww.c_begin, lane);
     const int u0 = qy0 * S;                                     // first dX row of the strip
     const int n_out = min(ww.nrows * S, g.H - u0) * g.W;        // its element count
+    const int nch = ww.c_end - ww.c_begin;
+    // all loads of the prologue first (see k_forward), index arithmetic under them
+    Stg stg;
+    stg.init_global(g, qy0 + g.row0_off, lane);
+    const T *gs = go + (ww.n * g.C + ww.c_begin) * oplane;
+    T *ds = dx + (ww.n * g.C + ww.c_begin) * iplane + (int64_t)u0 * g.W;
+    stg.template issue<0>(gs);
+    if constexpr (NST > 1) stg.template issue<1>(gs + (int64_t)min(1, nch - 1) * oplane);
+    if constexpr (NST > 2) stg.template issue<2>(gs + (int64_t)min(2, nch - 1) * oplane);
+    if constexpr (NST > 3) stg.template issue<3>(gs + (int64_t)min(3, nch - 1) * oplane);
+    // Few vectors per plane: bring the filter in through the tile.  Otherwise
+    // (scalar accesses, or more registers than the taps themselves) gather it.
+    constexpr bool kStageFilter = V > 1 && NV * V <= 8;
+    NeighbourFilterStager<T, V, kStageFilter ? NV : 1, K, D, S> nfs;
+    if constexpr (kStageFilter) nfs.issue(sf + ww.n * KK * oplane, oplane, stg.goff);
+    TapStager<KK, T, A> tst;
+    tst.issue(cf, ww.n * g.C + ww.c_begin, nch, lane);
 
     bool ok[PS];
     int lb[PS], ob[PS], cu[PS], cv[PS];
@@ -483,15 +558,7 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
         cu[m] = ok[m] ? cy * S : g.H;
         cv[m] = cx * S;
     }
-    Stg stg;
-    stg.init(g, qy0 + g.row0_off, lane);
-    // Few vectors per plane: bring the filter in through the tile.  Otherwise
-    // (scalar accesses, or more registers than the taps themselves) gather it.
-    constexpr bool kStageFilter = V > 1 && NV * V <= 8;
-    NeighbourFilterStager<T, V, kStageFilter ? NV : 1, K, D, S> nfs;
-    if constexpr (kStageFilter) {
-        nfs.issue(sf + ww.n * KK * oplane, oplane, stg.goff);
-    } else {
+    if constexpr (!kStageFilter) {
 #pragma unroll
         for (int m = 0; m < PS; ++m) {
             const int cy = qy0 + g.slot_row[m] + lr, cx = g.slot_col[m] + lc;
@@ -508,13 +575,9 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
                 }
         }
     }
-    const T *gs = go + (ww.n * g.C + ww.c_begin) * oplane;
-    T *ds = dx + (ww.n * g.C + ww.c_begin) * iplane + (int64_t)u0 * g.W;
-    const int nch = ww.c_end - ww.c_begin;
-    stg.template issue<0>(gs);
-    if constexpr (NST > 1) stg.template issue<1>(gs + (int64_t)min(1, nch - 1) * oplane);
-    if constexpr (NST > 2) stg.template issue<2>(gs + (int64_t)min(2, nch - 1) * oplane);
-    if constexpr (NST > 3) stg.template issue<3>(gs + (int64_t)min(3, nch - 1) * oplane);
+    stg.init_tile(g, qy0 + g.row0_off, lane);
+    const int P = pin(g.P);
+    const int idle = g.lin_tile + lane;
     zero_tile(lds_in, g.tile, lane);
     tst.put(taps, nch, lane);
     wave_sync();
@@ -527,30 +590,61 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
         wave_sync();
         A w[KK];
         load_taps<KK>(taps, ci, w);
+        if constexpr (kFlat) {
+            // branch-free, results written after all reads (see k_forward)
+            A acc[PS][S][S];
 #pragma unroll
-        for (int m = 0; m < PS; ++m) {
-            if (m >= g.nslots) break;
-            A acc[S][S];
+            for (int m = 0; m < PS; ++m) {
 #pragma unroll
-            for (int a = 0; a < S; ++a)
+                for (int a = 0; a < S; ++a)
 #pragma unroll
-                for (int c = 0; c < S; ++c) acc[a][c] = 0;
+                    for (int c = 0; c < S; ++c) acc[m][a][c] = 0;
 #pragma unroll
-            for (int i = 0; i < K; ++i)
+                for (int i = 0; i < K; ++i)
 #pragma unroll
-                for (int j = 0; j < K; ++j) {
-                    const A gv = ld(lds_in + lb[m] + (TM::dq(i) + TM::halo_lo) * g.P + TM::dq(j) +
-                                    TM::halo_lo);
-                    acc[TM::phase(i)][TM::phase(j)] +=
-                        gv * comb<MUL, A>(w[i * K + j], sfg[m][i * K + j]);
-                }
+                    for (int j = 0; j < K; ++j) {
+                        const A gv = ld(lds_in + lb[m] + (TM::dq(i) + TM::halo_lo) * P + TM::dq(j) +
+                                        TM::halo_lo);
+                        acc[m][TM::phase(i)][TM::phase(j)] +=
+                            gv * comb<MUL, A>(w[i * K + j], sfg[m][i * K + j]);
+                    }
+            }
 #pragma unroll
-            for (int a = 0; a < S; ++a)
+            for (int m = 0; m < PS; ++m)
 #pragma unroll
-                for (int c = 0; c < S; ++c) {
-                    if (cu[m] + a < g.H && cv[m] + c < g.W)
-                        st(lds_out + ob[m] + a * g.W + c, acc[a][c]);
-                }
+                for (int a = 0; a < S; ++a)
+#pragma unroll
+                    for (int c = 0; c < S; ++c) {
+                        // pixels outside the image (idle cells, odd H or W) go behind the strip
+                        const bool in = cu[m] + a < g.H && cv[m] + c < g.W;
+                        st(lds_out + (in ? ob[m] + a * g.W + c : idle), acc[m][a][c]);
+                    }
+        } else {
+#pragma unroll
+            for (int m = 0; m < PS; ++m) {
+                if (m >= g.nslots) break;
+                A acc[S][S];
+#pragma unroll
+                for (int a = 0; a < S; ++a)
+#pragma unroll
+                    for (int c = 0; c < S; ++c) acc[a][c] = 0;
+#pragma unroll
+                for (int i = 0; i < K; ++i)
+#pragma unroll
+                    for (int j = 0; j < K; ++j) {
+                        const A gv = ld(lds_in + lb[m] + (TM::dq(i) + TM::halo_lo) * P +
+                                        TM::dq(j) + TM::halo_lo);
+                        acc[TM::phase(i)][TM::phase(j)] +=
+                            gv * comb<MUL, A>(w[i * K + j], sfg[m][i * K + j]);
+                    }
+#pragma unroll
+                for (int a = 0; a < S; ++a)
+#pragma unroll
+                    for (int c = 0; c < S; ++c) {
+                        if (cu[m] + a < g.H && cv[m] + c < g.W)
+                            st(lds_out + ob[m] + a * g.W + c, acc[a][c]);
+                    }
+            }
         }
         wave_sync();
         store_strip<T, V>(lds_out, ds + (int64_t)ci * iplane, n_out, lane);
@@ -723,9 +817,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     // private LDS of this wave: X tile, dO strip, taps
-    T *lds_in = reinterpret_cast<T *>(smem + (size_t)wave * g.lds_wave_bytes);
-    T *lds_go = lds_in + g.tile + kSpare;
-    A *taps = reinterpret_cast<A *>(lds_go + g.lin_tile + kSpare);
+    A *lds_in = reinterpret_cast<A *>(smem + (size_t)wave * g.lds_wave_bytes);
+    T *lds_go = reinterpret_cast<T *>(lds_in + g.tile + kSpare);
+    A *taps = reinterpret_cast<A *>(lds_go + g.lin_tile + kIdle);
 
     WaveWork ww;
     if (!ww.init(g)) return;   // whole block leaves together
@@ -739,32 +833,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     const int nch = min(g.cpw, ww.c_end - c_begin);
     const int nch1 = max(nch, 1);   // a wave without channels still issues (harmless) loads
 
-    TapStager<KK, T, A> tst;
-    if (MUL) tst.issue(cf, ww.n * g.C + min(c_begin, g.C - 1), nch1, lane);
-
-    bool ok[PS];
-    int lb[PS], ob[PS];
-    A sfr[PS][KK], acc_sf[PS][KK];
-#pragma unroll
-    for (int m = 0; m < PS; ++m) {
-        const int row = g.slot_row[m] + lr, col = g.slot_col[m] + lc;
-        ok[m] = m < g.nslots && row < ww.nrows && col < g.cols;
-        lb[m] = (row * S) * g.P + col * S;     // lane-linear: no bank conflicts, idle lanes included
-        ob[m] = ok[m] ? row * g.Wo + col : 0;
-#pragma unroll
-        for (int t = 0; t < KK; ++t) {
-            sfr[m][t] = 0;
-            acc_sf[m][t] = 0;
-        }
-    }
-    FilterStager<T, V, NG, KK> fst;
-    if (MUL) {
-        fst.init(ww.nrows * g.Wo, lane);
-        fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
-    }
-
+    // all loads of the prologue first (see k_forward), index arithmetic under them
     Stg stg;
-    stg.init(g, y0 * S + g.row0_off, lane);
+    stg.init_global(g, y0 * S + g.row0_off, lane);
     LinStager<T, V, NG, NST> sgo;
     sgo.init(ww.nrows * g.Wo, lane);
     const int c_first = min(c_begin, g.C - 1);
@@ -782,12 +853,37 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         stg.template issue<3>(xs + (int64_t)min(3, nch1 - 1) * iplane);
         sgo.template issue<3>(gs + (int64_t)min(3, nch1 - 1) * oplane);
     }
+    FilterStager<T, V, NG, KK> fst;
+    TapStager<KK, T, A> tst;
+    if (MUL) {
+        fst.init(ww.nrows * g.Wo, lane);
+        fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
+        tst.issue(cf, ww.n * g.C + c_first, nch1, lane);
+    }
+
+    bool ok[PS];
+    int lb[PS], ob[PS];
+    A sfr[PS][KK], acc_sf[PS][KK];
+#pragma unroll
+    for (int m = 0; m < PS; ++m) {
+        const int row = g.slot_row[m] + lr, col = g.slot_col[m] + lc;
+        ok[m] = m < g.nslots && row < ww.nrows && col < g.cols;
+        lb[m] = (row * S) * g.P + col * S;     // lane-linear: no bank conflicts, idle lanes included
+        ob[m] = ok[m] ? row * g.Wo + col : 0;
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            sfr[m][t] = 0;
+            acc_sf[m][t] = 0;
+        }
+    }
+    stg.init_tile(g, y0 * S + g.row0_off, lane);
     zero_tile(lds_in, g.tile, lane);
     if (MUL) {
         tst.put(taps, nch, lane);
         fst.collect(lds_go, ob, sfr);
     }
     wave_sync();
+    const int P = pin(g.P);
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
@@ -803,6 +899,8 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         for (int t = 0; t < KK; ++t) pcf[t] = 0;
 #pragma unroll
         for (int m = 0; m < PS; ++m) {
+            // (this branch also keeps the scheduler from overlapping slots, which
+            // costs more registers than this kernel has)
             if (m >= g.nslots) break;
             // idle lanes read dO element 0 and are zeroed: they add nothing
             const A gval = ok[m] ? (A)ld(lds_go + ob[m]) : A(0);
@@ -811,7 +909,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
 #pragma unroll
                 for (int j = 0; j < K; ++j) {
                     const int t = i * K + j;
-                    const A gx = gval * (A)ld(lds_in + lb[m] + i * D * g.P + j * D);
+                    const A gx = gval * (A)ld(lds_in + lb[m] + i * D * P + j * D);
                     if (MUL) {
                         acc_sf[m][t] += gx * w[t];
                         pcf[t] += gx * sfr[m][t];
