@@ -98,7 +98,8 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     // sets per slot and is built for 4 (k=3) or 2 (k=5) only
     const bool filters = kind == kWaveFilters;
     const int ps_lo = filters ? (p.kk > 9 ? 2 : 4) : 4;
-    const int ps_hi = filters ? ps_lo : kMaxSlots;
+    // 25 taps: the spatial-filter registers of 8 slots would leave one wave per SIMD
+    const int ps_hi = filters ? ps_lo : (p.kk > 9 ? 4 : kMaxSlots);
     for (int ps = ps_lo; ps <= ps_hi; ps *= 2) {
         if (forced_ps && !filters && ps != forced_ps) continue;
         if (ps < cseg) continue;
@@ -181,7 +182,14 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     // per wave: tile (accumulator type), linear strip (storage type), taps
     t.lds_wave_bytes = round_up((t.tile + wave::kSpare) * asz + (t.lin_tile + wave::kIdle) * esz +
                                 cpw * ((p.kk + 3) / 4 * 4) * asz, 16);
-    t.lds_bytes = t.lds_wave_bytes * waves_per_block;
+    // Forward and feature gradient: several independent waves share a workgroup
+    // (workgroups are dispatched at a limited rate; waves of one start together).
+    t.wpb = 1;
+    if (!filters) {
+        t.wpb = std::max(1, std::min(env_int("DDF_TUNE_WPB", 1), wave::kMaxWpb));
+        while (t.wpb > 1 && t.lds_wave_bytes * t.wpb > 48 * 1024) --t.wpb;
+    }
+    t.lds_bytes = t.lds_wave_bytes * (filters ? waves_per_block : t.wpb);
     if (filters)  // the cross-wave sum of the dSF accumulators reuses the block's LDS
         t.lds_bytes = std::max(t.lds_bytes, waves_per_block * p.kk * kWave * acc_size(dtype));
     if (t.lds_bytes > 64 * 1024) return false;
@@ -193,7 +201,8 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     auto magic = [](int d) { return d == 1 ? 0u : (unsigned)((0x100000000ull + d - 1) / d); };
     t.csplit_magic = magic(t.csplit);
     t.nstrips_magic = magic(t.nstrips);
-    t.xcd_per = (unsigned)((nblocks + wave::kXcd - 1) / wave::kXcd);
+    const int64_t ngroups = (nblocks + t.wpb - 1) / t.wpb;   // workgroups launched
+    t.xcd_per = (unsigned)((ngroups + wave::kXcd - 1) / wave::kXcd);
     t.nblocks = (int)nblocks;
     *g = t;
     *ps_out = best_ps;

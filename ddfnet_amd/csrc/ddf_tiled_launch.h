@@ -10,9 +10,6 @@
 namespace ddf {
 namespace tiled {
 
-inline unsigned padded_grid(int nblocks) {
-    return (unsigned)((nblocks + wave::kXcd - 1) / wave::kXcd * wave::kXcd);
-}
 
 // Expands BODY for the (K, D, S) of the problem; BODY sees constexpr KK_, DD_, SS_.
 #define DDF_DISPATCH_KDS(p, ...)                                           \
@@ -55,7 +52,7 @@ inline bool aligned_for(int v, std::initializer_list<const void *> ptrs) {
 template <typename T, int K, int D, int S>
 hipError_t launch_forward(const Problem &p, const WaveGeom &g, int ps, int nv, const T *x,
                           const T *cf, const T *sf, T *out, hipStream_t st) {
-    const dim3 grid(padded_grid(g.nblocks)), block(kWave);
+    const dim3 grid(g.xcd_per * wave::kXcd), block(kWave * g.wpb);
     DDF_DISPATCH_WAVE(ps, nv, g.vec, {
         if constexpr (sizeof(T) == 8 && VV_ != 1) return hipErrorNotSupported;
         else if (p.mul)
@@ -71,7 +68,7 @@ hipError_t launch_forward(const Problem &p, const WaveGeom &g, int ps, int nv, c
 template <typename T, int K, int D, int S>
 hipError_t launch_features(const Problem &p, const WaveGeom &g, int ps, int nv, const T *go,
                            const T *cf, const T *sf, T *dx, hipStream_t st) {
-    const dim3 grid(padded_grid(g.nblocks)), block(kWave);
+    const dim3 grid(g.xcd_per * wave::kXcd), block(kWave * g.wpb);
     DDF_DISPATCH_WAVE(ps, nv, g.vec, {
         if constexpr (sizeof(T) == 8 && VV_ != 1) return hipErrorNotSupported;
         else if (p.mul)
@@ -92,7 +89,7 @@ hipError_t launch_filters_nv(const Problem &p, const WaveGeom &g, const T *go, c
                              typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                              unsigned need, hipStream_t st) {
     constexpr int PS = K == 3 ? 4 : 2;
-    const dim3 grid(padded_grid(g.nblocks)), block(kWave * wave::kFilterWaves);
+    const dim3 grid(g.xcd_per * wave::kXcd), block(kWave * wave::kFilterWaves);
     if (p.mul)
         hipLaunchKernelGGL((wave::k_backward_filters<T, K, D, S, true, PS, NV, V>), grid, block,
                            g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
@@ -186,18 +183,13 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
         if (err != hipSuccess) return err;
         if (ws_sf) {
             // dSF[n, t, pix] = sum over channel splits
-            const int64_t inner = p.kk * p.Ho * p.Wo, total = p.N * inner;
-            hipLaunchKernelGGL((wave::k_sum_partials<T>), dim3((unsigned)cdiv(total, 256)),
-                               dim3(256), 0, st, ws_sf, dsf, p.N, g.csplit, inner);
-            if ((err = hipGetLastError()) != hipSuccess) return err;
+            err = wave::sum_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, st);
+            if (err != hipSuccess) return err;
         }
         if (ws_cf) {
             // dCF[nc, t] = sum over strips
-            const int64_t total = p.N * p.C * p.kk;
-            hipLaunchKernelGGL((wave::k_sum_partials<T>), dim3((unsigned)cdiv(total, 256)),
-                               dim3(256), 0, st, ws_cf, dcf, p.N * p.C, g.nstrips,
-                               (int64_t)p.kk);
-            if ((err = hipGetLastError()) != hipSuccess) return err;
+            err = wave::sum_partials<T>(ws_cf, dcf, p.N * p.C, g.nstrips, (int64_t)p.kk, st);
+            if (err != hipSuccess) return err;
         }
     }
     return err;

@@ -47,6 +47,7 @@ struct WaveGeom {
     int lin_cols, lin_rpc, lin_rows, lin_tile;
     int cpw, csplit;          // channels per wave; number of channel ranges (of cpw * waves per block)
     int cpb;                  // channels per block (= cpw for the one-wave kernels)
+    int wpb;                  // independent waves per workgroup (forward, feature gradient)
     int lds_wave_bytes;       // LDS of one wave (filter-gradient blocks hold four)
     int vec, nv;              // elements per global access; vectors per lane per channel strip
     unsigned src_magic;       // ceil(2^32 / src_cols); 0 when src_cols == 1
@@ -60,6 +61,8 @@ struct WaveGeom {
 namespace wave {
 
 constexpr int kXcd = 8;
+// Most independent waves a workgroup of the forward / feature-gradient kernels holds.
+constexpr int kMaxWpb = 4;
 // Spare LDS elements behind each tile: idle lanes write there instead of branching.
 constexpr int kSpare = 8;
 // Spare elements behind each linear result strip: one per lane, where idle
@@ -111,9 +114,12 @@ __device__ __forceinline__ int pin(int v) {
 struct WaveWork {
     int cs, strip, row_first, nrows, c_begin, c_end;
     int64_t n;
-    __device__ __forceinline__ bool init(const WaveGeom &g) {
-        const int b = (int)(blockIdx.x % kXcd) * (int)g.xcd_per + (int)(blockIdx.x / kXcd);
-        if (b >= g.nblocks) return false;
+    // `wave`: index of the calling wave among the g.wpb independent waves of
+    // its workgroup (0 for kernels whose workgroup is the unit of work)
+    __device__ __forceinline__ bool init(const WaveGeom &g, int wave = 0) {
+        const int wg = (int)(blockIdx.x % kXcd) * (int)g.xcd_per + (int)(blockIdx.x / kXcd);
+        const int b = wg * g.wpb + wave;
+        if (wave >= g.wpb || b >= g.nblocks) return false;
         const int rest = magic_div(b, g.csplit_magic);
         cs = b - rest * g.csplit;
         const int smp = magic_div(rest, g.nstrips_magic);
@@ -303,7 +309,7 @@ struct FilterStager {
 // Forward: work cell = output pixel.
 // ---------------------------------------------------------------------------
 template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V>
-__global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restrict__ x,
+__global__ __launch_bounds__(kWave * kMaxWpb) void k_forward(WaveGeom g, const T *__restrict__ x,
                                                    const T *__restrict__ cf,
                                                    const T *__restrict__ sf,
                                                    T *__restrict__ out) {
@@ -313,14 +319,16 @@ __global__ __launch_bounds__(kWave) void k_forward(WaveGeom g, const T *__restri
     using Stg = Stager<T, V, NV>;
     constexpr int NST = Stg::NST;
     extern __shared__ __align__(16) unsigned char smem[];
-    A *lds_in = reinterpret_cast<A *>(smem);
+    // the waves of a workgroup are independent: each has its own work and LDS
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    A *lds_in = reinterpret_cast<A *>(smem + (size_t)wave * g.lds_wave_bytes);
     T *lds_out = reinterpret_cast<T *>(lds_in + g.tile + kSpare);
     A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kIdle);
 
     DDF_STAMP(0);
     WaveWork ww;
-    if (!ww.init(g) || ww.c_end <= ww.c_begin) return;
-    const int lane = threadIdx.x;
+    if (!ww.init(g, wave) || ww.c_end <= ww.c_begin) return;
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
     const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
     const int y0 = ww.row_first;
@@ -504,7 +512,7 @@ struct NeighbourFilterStager {
 };
 
 template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V>
-__global__ __launch_bounds__(kWave) void k_backward_features(
+__global__ __launch_bounds__(kWave * kMaxWpb) void k_backward_features(
     WaveGeom g, const T *__restrict__ go, const T *__restrict__ cf,
     const T *__restrict__ sf, T *__restrict__ dx) {
     using A = typename Acc<T>::type;
@@ -514,13 +522,14 @@ __global__ __launch_bounds__(kWave) void k_backward_features(
     using Stg = Stager<T, V, NV>;
     constexpr int NST = Stg::NST;
     extern __shared__ __align__(16) unsigned char smem[];
-    A *lds_in = reinterpret_cast<A *>(smem);
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    A *lds_in = reinterpret_cast<A *>(smem + (size_t)wave * g.lds_wave_bytes);
     T *lds_out = reinterpret_cast<T *>(lds_in + g.tile + kSpare);
     A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kIdle);
 
     WaveWork ww;
-    if (!ww.init(g) || ww.c_end <= ww.c_begin) return;
-    const int lane = threadIdx.x;
+    if (!ww.init(g, wave) || ww.c_end <= ww.c_begin) return;
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
     const int64_t oplane = (int64_t)g.Ho * g.Wo, iplane = (int64_t)g.H * g.W;
     const int qy0 = ww.row_first;
@@ -972,18 +981,56 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     }
 }
 
-// out[o, i] = sum_p part[o, p, i] for o < outer, p < parts, i < inner.
-template <typename T>
+// out[o, i] = sum_p part[o, p, i] for o < outer, p < parts, i < inner.  A
+// thread adds up VEC neighbouring i (inner % VEC == 0) and keeps 8 loads in
+// flight; the order of the additions is fixed, so results are reproducible.
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void k_sum_partials(
     const typename Acc<T>::type *__restrict__ part, T *__restrict__ out, int64_t outer,
     int parts, int64_t inner) {
     using A = typename Acc<T>::type;
+    const int64_t iv = inner / VEC;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= outer * inner) return;
-    const int64_t o = idx / inner, i = idx - o * inner;
-    A tot = 0;
-    for (int p = 0; p < parts; ++p) tot += part[(o * parts + p) * inner + i];
-    st(out + idx, tot);
+    if (idx >= outer * iv) return;
+    const int64_t o = idx / iv, i = (idx - o * iv) * VEC;
+    const A *src = part + o * parts * inner + i;
+    A tot[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) tot[k] = 0;
+    int p = 0;
+    for (; p + 8 <= parts; p += 8) {
+        Vec<A, VEC> v[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+            v[q] = *reinterpret_cast<const Vec<A, VEC> *>(src + (int64_t)(p + q) * inner);
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) tot[k] += v[q].e[k];
+    }
+    for (; p < parts; ++p) {
+        const Vec<A, VEC> v = *reinterpret_cast<const Vec<A, VEC> *>(src + (int64_t)p * inner);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) tot[k] += v.e[k];
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) st(out + o * inner + i + k, tot[k]);
+}
+
+// Launches k_sum_partials with the widest access the sizes allow (the
+// workspace is 256-byte aligned).
+template <typename T>
+inline hipError_t sum_partials(const typename Acc<T>::type *part, T *out, int64_t outer,
+                               int parts, int64_t inner, hipStream_t st) {
+    using A = typename Acc<T>::type;
+    const bool wide = sizeof(A) == 4 && inner % 4 == 0;
+    const int64_t threads = outer * (wide ? inner / 4 : inner);
+    const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+    if (wide)
+        hipLaunchKernelGGL((k_sum_partials<T, 4>), grid, block, 0, st, part, out, outer, parts, inner);
+    else
+        hipLaunchKernelGGL((k_sum_partials<T, 1>), grid, block, 0, st, part, out, outer, parts, inner);
+    return hipGetLastError();
 }
 
 }  // namespace wave
