@@ -48,10 +48,20 @@ WORKLOADS = {
 }
 DEFAULT_WORKLOAD = 'r50_stage3_mul_fp32'
 DTYPE_NAME = {torch.float32: 'f32', torch.float16: 'f16', torch.float64: 'f64'}
-PHASES = ('fwd', 'dx', 'dfilters')
-# kernels behind each phase (one library call each)
-PHASE_KERNELS = {'fwd': 'ddf::wave::k_forward', 'dx': 'ddf::wave::k_backward_features',
-                 'dfilters': 'ddf::wave::k_backward_filters + ddf::wave::k_sum_partials'}
+# Library calls timed on their own, back to back.  The step is fwd + bwd; dx
+# and dfilters are the two halves of the backward pass requested separately
+# (autograd does that when only some inputs need gradients).
+PHASES = ('fwd', 'bwd', 'dx', 'dfilters')
+STEP_PHASES = ('fwd', 'bwd')
+# kernels behind each call.  At 3x3 / stride 1 with short strips the whole
+# backward pass is one launch of k_backward_filters<..., DX=true> (it also
+# writes the feature gradient); otherwise bwd = the dx call + the dfilters call.
+PHASE_KERNELS = {
+    'fwd': 'ddf::wave::k_forward',
+    'bwd': 'ddf::wave::k_backward_filters<DX=true> + ddf::wave::k_sum_partials',
+    'dx': 'ddf::wave::k_backward_features',
+    'dfilters': 'ddf::wave::k_backward_filters<DX=false> + ddf::wave::k_sum_partials',
+}
 
 
 def log(*a):
@@ -140,6 +150,8 @@ class Launcher(object):
     def phase(self, name, i):
         if name == 'fwd':
             self.fwd(i)
+        elif name == 'bwd':
+            self.bwd(i, 7)
         elif name == 'dx':
             self.bwd(i, 1)
         else:
@@ -166,7 +178,7 @@ def timed(fn, count):
 # the figures are recorded here; a workload or phase that was not profiled
 # reports null.
 MEASURED_TRAFFIC = {
-    'r50_stage3_mul_fp32': {'fwd': 26885000, 'dx': 26895000, 'dfilters': 35840000},
+    'r50_stage3_mul_fp32': {'fwd': 26907648, 'bwd': 48412364, 'dx': 26927104, 'dfilters': 35570483},
 }
 
 
@@ -310,7 +322,7 @@ def main():
                 extra[name] = run_workload(name, args.steps, args.warmup, lib)
     res = run_workload(args.workload, args.steps, args.warmup, lib, copy_probe=args.copy_probe)
 
-    dominant = max(PHASES, key=lambda p: res['phase_ms'][p])
+    dominant = max(STEP_PHASES, key=lambda p: res['phase_ms'][p])
     dom_bytes = res['bytes'][dominant]
     dom_s = res['phase_ms'][dominant] * 1e-3
     achieved = dom_bytes / dom_s / 1e9

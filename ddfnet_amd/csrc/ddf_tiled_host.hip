@@ -21,6 +21,8 @@ int round_up(int v, int m) { return (v + m - 1) / m * m; }
 
 }  // namespace
 
+int tune_int(const char *name, int fallback) { return env_int(name, fallback); }
+
 bool tiled_shape_instantiated(int k, int d, int s) {
     return (k == 3 || k == 5) && (d == 1 || d == 2) && (s == 1 || s == 2);
 }
@@ -31,6 +33,7 @@ bool tiled_shape_instantiated(int k, int d, int s) {
 bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom *g, int *ps_out,
                    int *nv_out) {
     if (!tiled_shape_instantiated(p.k, p.d, p.s)) return false;
+    if (kind == kWaveFused && (p.s != 1 || p.k != 3)) return false;
     if (p.N <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0) return false;
     if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
     const int esz = elem_size(dtype);
@@ -96,7 +99,8 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     int best_ps = 0, best_th = 0, best_v = 0, best_nv = 0;
     // slots per lane: 4 or 8; the filter-gradient kernel keeps two register
     // sets per slot and is built for 4 (k=3) or 2 (k=5) only
-    const bool filters = kind == kWaveFilters;
+    const bool fused = kind == kWaveFused;   // filter gradients + feature gradient in one kernel
+    const bool filters = kind == kWaveFilters || fused;
     const int ps_lo = filters ? (p.kk > 9 ? 2 : 4) : 4;
     // 25 taps: the spatial-filter registers of 8 slots would leave one wave per SIMD
     const int ps_hi = filters ? ps_lo : (p.kk > 9 ? 4 : kMaxSlots);
@@ -141,6 +145,10 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
         if (cost < best) { best = cost; best_ps = ps; best_th = th; best_v = v; best_nv = nv; }
     }
     if (best_ps == 0) return false;
+    // The fused kernel is built for strips of one 16-byte vector per lane only:
+    // with longer strips its registers leave no room to prefetch, and two
+    // launches are faster.
+    if (fused && !(best_v == 4 && best_nv == 1)) return false;
     t.TH = best_th;
     t.nstrips = (t.rows + t.TH - 1) / t.TH;
     t.nslots = ((t.TH + RS - 1) / RS) * cseg;
@@ -180,7 +188,8 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     t.csplit = (C + t.cpb - 1) / t.cpb;
     // per wave: tiles, then the channel-filter taps of its channels (accumulator type)
     // per wave: tile (accumulator type), linear strip (storage type), taps
-    t.lds_wave_bytes = round_up((t.tile + wave::kSpare) * asz + (t.lin_tile + wave::kIdle) * esz +
+    t.lds_wave_bytes = round_up((fused ? 2 : 1) * (t.tile + wave::kSpare) * asz +
+                                (t.lin_tile + wave::kIdle) * esz +
                                 cpw * ((p.kk + 3) / 4 * 4) * asz, 16);
     // Forward and feature gradient: several independent waves share a workgroup
     // (workgroups are dispatched at a limited rate; waves of one start together).

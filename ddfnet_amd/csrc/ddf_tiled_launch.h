@@ -83,41 +83,52 @@ hipError_t launch_features(const Problem &p, const WaveGeom &g, int ps, int nv, 
 
 // Filter gradients: 4 pixel slots per lane for k=3, 2 for k=5 (two register
 // sets per slot); V=4 with NV 1, 2, 4 and V=1 with NV 4 (and 8 for k=3).
-template <typename T, int K, int D, int S, int NV, int V>
+// DX: the same launch also writes the feature gradient (3x3, stride 1).
+template <typename T, int K, int D, int S, int NV, int V, bool DX>
 hipError_t launch_filters_nv(const Problem &p, const WaveGeom &g, const T *go, const T *x,
-                             const T *cf, const T *sf, T *dcf, T *dsf,
+                             const T *cf, const T *sf, T *dx, T *dcf, T *dsf,
                              typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                              unsigned need, hipStream_t st) {
     constexpr int PS = K == 3 ? 4 : 2;
     const dim3 grid(g.xcd_per * wave::kXcd), block(kWave * wave::kFilterWaves);
     if (p.mul)
-        hipLaunchKernelGGL((wave::k_backward_filters<T, K, D, S, true, PS, NV, V>), grid, block,
-                           g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
+        hipLaunchKernelGGL((wave::k_backward_filters<T, K, D, S, true, PS, NV, V, DX>), grid,
+                           block, g.lds_bytes, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf,
+                           need);
     else
-        hipLaunchKernelGGL((wave::k_backward_filters<T, K, D, S, false, PS, NV, V>), grid, block,
-                           g.lds_bytes, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need);
+        hipLaunchKernelGGL((wave::k_backward_filters<T, K, D, S, false, PS, NV, V, DX>), grid,
+                           block, g.lds_bytes, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf,
+                           need);
     return hipGetLastError();
 }
 
-template <typename T, int K, int D, int S>
+template <typename T, int K, int D, int S, bool DX>
 hipError_t launch_filters(const Problem &p, const WaveGeom &g, int ps, int nv, const T *go,
-                          const T *x, const T *cf, const T *sf, T *dcf, T *dsf,
+                          const T *x, const T *cf, const T *sf, T *dx, T *dcf, T *dsf,
                           typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                           unsigned need, hipStream_t st) {
     if (ps != (K == 3 ? 4 : 2)) return hipErrorNotSupported;
+    if constexpr (DX && (K != 3 || S != 1)) {
+        return hipErrorNotSupported;
+    } else {
 #define DDF_FILTERS_CASE(NV_, V_)                                                             \
     if (g.vec == V_ && nv == NV_)                                                             \
-        return launch_filters_nv<T, K, D, S, NV_, V_>(p, g, go, x, cf, sf, dcf, dsf, ws_sf,   \
-                                                      ws_cf, need, st);
-    if constexpr (sizeof(T) != 8) {
-        DDF_FILTERS_CASE(1, 4)
-        DDF_FILTERS_CASE(2, 4)
-        DDF_FILTERS_CASE(4, 4)
-    }
-    DDF_FILTERS_CASE(4, 1)
-    if constexpr (K == 3) { DDF_FILTERS_CASE(8, 1) }
+        return launch_filters_nv<T, K, D, S, NV_, V_, DX>(p, g, go, x, cf, sf, dx, dcf, dsf,  \
+                                                          ws_sf, ws_cf, need, st);
+        if constexpr (sizeof(T) != 8) {
+            DDF_FILTERS_CASE(1, 4)
+            if constexpr (!DX) {
+                DDF_FILTERS_CASE(2, 4)
+                DDF_FILTERS_CASE(4, 4)
+            }
+        }
+        if constexpr (!DX) {
+            DDF_FILTERS_CASE(4, 1)
+            if constexpr (K == 3) { DDF_FILTERS_CASE(8, 1) }
+        }
 #undef DDF_FILTERS_CASE
-    return hipErrorNotSupported;
+        return hipErrorNotSupported;
+    }
 }
 
 }  // namespace tiled
@@ -155,8 +166,18 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     using A = typename Acc<T>::type;
     const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
     hipError_t err = hipSuccess;
-    if (need & DDF_NEED_DX) {
-        WaveGeom g; int ps, nv;
+    const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
+    // One launch for all gradients where the fused kernel exists and cuts the
+    // problem exactly as the workspace was sized for.
+    WaveGeom g; int ps, nv;
+    bool fuse = false;
+    if ((need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_FUSED", 1) != 0) {
+        WaveGeom gp; int pps, pnv;
+        fuse = wave_plan<T>(p, kWaveFused, {go, x, sf, dx}, &g, &ps, &nv) &&
+               wave_geometry(p, dtype, kWaveFilters, 0, &gp, &pps, &pnv) && gp.TH == g.TH &&
+               gp.csplit == g.csplit;
+    }
+    if ((need & DDF_NEED_DX) && !fuse) {
         if (!wave_plan<T>(p, kWaveFeatures, {go, sf, dx}, &g, &ps, &nv)) {
             err = generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, DDF_NEED_DX, st);
         } else {
@@ -164,10 +185,8 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
         }
         if (err != hipSuccess) return err;
     }
-    const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
     if (fneed) {
-        WaveGeom g; int ps, nv;
-        if (!wave_plan<T>(p, kWaveFilters, {go, x, sf}, &g, &ps, &nv))
+        if (!fuse && !wave_plan<T>(p, kWaveFilters, {go, x, sf}, &g, &ps, &nv))
             return generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, fneed, st);
         // carve the workspace exactly as tiled_backward_workspace() sized it
         unsigned char *wp = static_cast<unsigned char *>(ws);
@@ -178,8 +197,14 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
             wp += ((size_t)n_sf * g.csplit * sizeof(A) + 255) / 256 * 256;
         }
         if ((fneed & DDF_NEED_DCF) && g.nstrips > 1) ws_cf = reinterpret_cast<A *>(wp);
-        DDF_DISPATCH_KDS(p, err = tiled::launch_filters<T, KK_, DD_, SS_>(
-                                p, g, ps, nv, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, fneed, st));
+        if (fuse)
+            DDF_DISPATCH_KDS(p, err = tiled::launch_filters<T, KK_, DD_, SS_, true>(
+                                    p, g, ps, nv, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, fneed,
+                                    st));
+        else
+            DDF_DISPATCH_KDS(p, err = tiled::launch_filters<T, KK_, DD_, SS_, false>(
+                                    p, g, ps, nv, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, fneed,
+                                    st));
         if (err != hipSuccess) return err;
         if (ws_sf) {
             // dSF[n, t, pix] = sum over channel splits

@@ -179,9 +179,9 @@ constexpr int stages() { return NV <= 1 ? 4 : (NV <= 2 ? 2 : 1); }
 // Source strip -> zero-bordered LDS tile, through registers.  The strip of one
 // channel is a run of n_in contiguous elements; lane l owns vectors
 // f = l, l + 64, ... of it.  Their tile offsets are computed once.
-template <typename T, int V, int NV>
+template <typename T, int V, int NV, int MAXST = 4>
 struct Stager {
-    static constexpr int NST = stages<NV>();
+    static constexpr int NST = stages<NV>() < MAXST ? stages<NV>() : MAXST;
     int goff[NV];        // element offset of the vector inside a source plane
     int lo[NV][V];       // tile offset of each element
     Vec<T, V> v[NST][NV];
@@ -812,22 +812,35 @@ constexpr int bfly_writers() {
 // ---------------------------------------------------------------------------
 constexpr int kFilterWaves = 4;
 
-template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V>
+//
+// With DX (stride 1 only) the same walk also produces the feature gradient:
+// dO then sits in a zero-bordered tile of its own (same shape and offsets as
+// the X tile), the lane gathers it at the flipped tap offsets against the
+// neighbour cells' spatial filter (held in registers like the cell's own), and
+// the linear strip carries the dX results out.  One launch instead of two, and
+// dO, CF and SF are read once for the whole backward pass.
+template <typename T, int K, int D, int S, bool MUL, int PS, int NV, int V, bool DX>
 __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     WaveGeom g, const T *__restrict__ go, const T *__restrict__ x,
-    const T *__restrict__ cf, const T *__restrict__ sf, T *__restrict__ dcf,
-    T *__restrict__ dsf, typename Acc<T>::type *__restrict__ ws_sf,
+    const T *__restrict__ cf, const T *__restrict__ sf, T *__restrict__ dx,
+    T *__restrict__ dcf, T *__restrict__ dsf, typename Acc<T>::type *__restrict__ ws_sf,
     typename Acc<T>::type *__restrict__ ws_cf, unsigned need) {
+    static_assert(!DX || S == 1, "the fused feature gradient needs stride 1");
     using A = typename Acc<T>::type;
     constexpr int KK = K * K;
-    using Stg = Stager<T, V, NV>;
+    constexpr int R = (K - 1) / 2;
+    constexpr bool kFilters = MUL || DX;   // CF and SF values are needed at all
+    // (two channels in flight at most with DX: it stages two planes per channel
+    // and holds a third set of filter registers)
+    using Stg = Stager<T, V, NV, DX ? 2 : 4>;
     constexpr int NST = Stg::NST;
     constexpr int NG = (PS + V - 1) / V;
     extern __shared__ __align__(16) unsigned char smem[];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    // private LDS of this wave: X tile, dO strip, taps
+    // private LDS of this wave: X tile, [dO tile,] linear strip (dO in, or dX out), taps
     A *lds_in = reinterpret_cast<A *>(smem + (size_t)wave * g.lds_wave_bytes);
-    T *lds_go = reinterpret_cast<T *>(lds_in + g.tile + kSpare);
+    A *lds_g = lds_in + g.tile + kSpare;
+    T *lds_go = reinterpret_cast<T *>(lds_g + (DX ? g.tile + kSpare : 0));
     A *taps = reinterpret_cast<A *>(lds_go + g.lin_tile + kIdle);
 
     WaveWork ww;
@@ -845,34 +858,52 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     // all loads of the prologue first (see k_forward), index arithmetic under them
     Stg stg;
     stg.init_global(g, y0 * S + g.row0_off, lane);
+    // dO: a bordered tile with the X tile's offsets (DX), else a linear strip
+    Stg stg_g;
     LinStager<T, V, NG, NST> sgo;
-    sgo.init(ww.nrows * g.Wo, lane);
+    if constexpr (DX) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j) stg_g.goff[j] = stg.goff[j];
+    } else {
+        sgo.init(ww.nrows * g.Wo, lane);
+    }
     const int c_first = min(c_begin, g.C - 1);
     const T *xs = x + (ww.n * g.C + c_first) * iplane;
-    const T *gs = go + (ww.n * g.C + c_first) * oplane + (int64_t)y0 * g.Wo;
+    const T *gs = go + (ww.n * g.C + c_first) * oplane + (DX ? 0 : (int64_t)y0 * g.Wo);
+    auto issue_go = [&](auto st_tag, const T *plane) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        if constexpr (DX) stg_g.template issue<ST>(plane);
+        else sgo.template issue<ST>(plane);
+    };
     stg.template issue<0>(xs);
-    sgo.template issue<0>(gs);
+    issue_go(std::integral_constant<int, 0>{}, gs);
     if constexpr (NST > 1) {
         stg.template issue<1>(xs + (int64_t)min(1, nch1 - 1) * iplane);
-        sgo.template issue<1>(gs + (int64_t)min(1, nch1 - 1) * oplane);
+        issue_go(std::integral_constant<int, 1>{}, gs + (int64_t)min(1, nch1 - 1) * oplane);
     }
     if constexpr (NST > 2) {
         stg.template issue<2>(xs + (int64_t)min(2, nch1 - 1) * iplane);
-        sgo.template issue<2>(gs + (int64_t)min(2, nch1 - 1) * oplane);
+        issue_go(std::integral_constant<int, 2>{}, gs + (int64_t)min(2, nch1 - 1) * oplane);
         stg.template issue<3>(xs + (int64_t)min(3, nch1 - 1) * iplane);
-        sgo.template issue<3>(gs + (int64_t)min(3, nch1 - 1) * oplane);
+        issue_go(std::integral_constant<int, 3>{}, gs + (int64_t)min(3, nch1 - 1) * oplane);
     }
     FilterStager<T, V, NG, KK> fst;
     TapStager<KK, T, A> tst;
-    if (MUL) {
+    // neighbour cells' spatial filter for dX: through the tile when it is a
+    // few vectors per plane, gathered otherwise (see k_backward_features)
+    constexpr bool kStageFilter = DX && V > 1 && NV * V <= 8;
+    NeighbourFilterStager<T, V, kStageFilter ? NV : 1, K, D, 1> nfs;
+    if (kFilters) {
         fst.init(ww.nrows * g.Wo, lane);
         fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
+        if constexpr (kStageFilter) nfs.issue(sf + ww.n * KK * oplane, oplane, stg.goff);
         tst.issue(cf, ww.n * g.C + c_first, nch1, lane);
     }
 
     bool ok[PS];
     int lb[PS], ob[PS];
     A sfr[PS][KK], acc_sf[PS][KK];
+    A sfg[DX ? PS : 1][KK];   // spatial filter at the neighbour cells (DX)
 #pragma unroll
     for (int m = 0; m < PS; ++m) {
         const int row = g.slot_row[m] + lr, col = g.slot_col[m] + lc;
@@ -884,25 +915,52 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
             sfr[m][t] = 0;
             acc_sf[m][t] = 0;
         }
+        if constexpr (DX && !kStageFilter) {
+            const int cy = y0 + row;
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const int sy = cy - (i - R) * D, sx = col - (j - R) * D;
+                    const bool in = ok[m] && sy >= 0 && sy < g.Ho && sx >= 0 && sx < g.Wo;
+                    // out-of-range neighbours read element 0 and are zeroed: no branch
+                    const A val = ld(sf + (ww.n * KK + i * K + j) * oplane +
+                                     (in ? (int64_t)sy * g.Wo + sx : 0));
+                    sfg[m][i * K + j] = in ? val : A(0);
+                }
+        }
     }
     stg.init_tile(g, y0 * S + g.row0_off, lane);
+    if constexpr (DX) {
+#pragma unroll
+        for (int j = 0; j < NV; ++j)
+#pragma unroll
+            for (int k = 0; k < V; ++k) stg_g.lo[j][k] = stg.lo[j][k];
+    }
+    const int P = pin(g.P);
     zero_tile(lds_in, g.tile, lane);
-    if (MUL) {
+    if constexpr (DX) zero_tile(lds_g, g.tile, lane);
+    if (kFilters) {
         tst.put(taps, nch, lane);
         fst.collect(lds_go, ob, sfr);
+        wave_sync();
+        if constexpr (kStageFilter) nfs.collect(lds_g, stg.lo, lb, P, sfg);
     }
     wave_sync();
-    const int P = pin(g.P);
+    const int idle = g.lin_tile + lane;   // where idle lanes put their dX values
+    T *ds = DX ? dx + (ww.n * g.C + c_first) * iplane + (int64_t)y0 * g.W : nullptr;
+    const int n_out = ww.nrows * g.W;      // elements of the dX strip (DX: stride 1)
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         stg.template commit<ST>(lds_in);
-        sgo.template commit<ST>(lds_go);
+        if constexpr (DX) stg_g.template commit<ST>(lds_g);
+        else sgo.template commit<ST>(lds_go);
         stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch1 - 1) * iplane);
-        sgo.template issue<ST>(gs + (int64_t)min(ci + NST, nch1 - 1) * oplane);
+        issue_go(st_tag, gs + (int64_t)min(ci + NST, nch1 - 1) * oplane);
         wave_sync();
         A w[KK];
-        if (MUL) load_taps<KK>(taps, ci, w);
+        if (kFilters) load_taps<KK>(taps, ci, w);
         A pcf[KK];
 #pragma unroll
         for (int t = 0; t < KK; ++t) pcf[t] = 0;
@@ -911,8 +969,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
             // (this branch also keeps the scheduler from overlapping slots, which
             // costs more registers than this kernel has)
             if (m >= g.nslots) break;
-            // idle lanes read dO element 0 and are zeroed: they add nothing
-            const A gval = ok[m] ? (A)ld(lds_go + ob[m]) : A(0);
+            // idle lanes read a valid dO element and are zeroed: they add nothing
+            const A gread = DX ? (A)ld(lds_g + lb[m] + R * D * P + R * D) : (A)ld(lds_go + ob[m]);
+            const A gval = ok[m] ? gread : A(0);
 #pragma unroll
             for (int i = 0; i < K; ++i)
 #pragma unroll
@@ -927,6 +986,21 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
                         pcf[t] += gx;
                     }
                 }
+            if constexpr (DX) {
+                // dX of the cell: dO at the flipped tap offsets, filters of those cells
+                A accx = 0;
+#pragma unroll
+                for (int i = 0; i < K; ++i)
+#pragma unroll
+                    for (int j = 0; j < K; ++j)
+                        accx += (A)ld(lds_g + lb[m] + (2 * R - i) * D * P + (2 * R - j) * D) *
+                                comb<MUL, A>(w[i * K + j], sfg[m][i * K + j]);
+                st(lds_go + (ok[m] ? ob[m] : idle), accx);
+            }
+        }
+        if constexpr (DX) {
+            wave_sync();
+            store_strip<T, V>(lds_go, ds + (int64_t)ci * iplane, n_out, lane);
         }
         if (want_cf) {
             const A tot = bfly_sum<KK, 0, A>(pcf, lane);
@@ -1035,7 +1109,10 @@ inline hipError_t sum_partials(const typename Acc<T>::type *part, T *out, int64_
 
 }  // namespace wave
 
-enum WaveKind { kWaveForward = 0, kWaveFeatures = 1, kWaveFilters = 2 };
+// Integer tuning knob from the environment (for experiments), else `fallback`.
+int tune_int(const char *name, int fallback);
+
+enum WaveKind { kWaveForward = 0, kWaveFeatures = 1, kWaveFilters = 2, kWaveFused = 3 };
 // Host-side geometry (ddf_tiled_host.hip).  *ps and *nv select the kernel.
 // max_vec > 0 caps the elements per global access (1 = scalar accesses).
 bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom *g, int *ps,

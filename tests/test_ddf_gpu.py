@@ -221,6 +221,27 @@ def test_needs_input_grad_subsets():
                 assert g_part is None
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16], ids=_ids)
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('shape,d', [((3, 40, 14, 14), 1), ((2, 24, 14, 14), 2), ((2, 9, 12, 16), 1),
+                                     ((1, 130, 8, 8), 1)])
+def test_one_launch_backward_equals_two_launches(shape, d, combine, dtype, monkeypatch):
+    """All three gradients requested together come from one fused kernel where
+    it exists (3x3, stride 1, short strips); switched off, the feature gradient
+    and the filter gradients come from their own kernels.  Same sums in the same
+    order: the results must be identical, and both must match the oracle."""
+    N, C, H, W = shape
+    x, cf, sf, go = random_case(N, C, H, W, 3, 1, dtype, seed=11)
+    fused = run_ddf(x, cf, sf, go, 3, d, 1, combine)
+    monkeypatch.setenv('DDF_TUNE_FUSED', '0')
+    split = run_ddf(x, cf, sf, go, 3, d, 1, combine)
+    for a, b in zip(fused, split):
+        assert torch.equal(a, b)
+    want = oracle.backward(go, x, cf, sf, 3, d, 1, combine)
+    for got, w in zip(fused[1:], want):
+        assert rel_err(got, w) <= TOL[dtype]
+
+
 def test_mixed_dtypes_are_promoted():
     """fp16 features with fp32 filters: the reference widens the fp16 operand
     (ddf/ddf.py:37-42); result is fp32."""
