@@ -1,23 +1,27 @@
-// Wavefront-per-strip DDF kernels for gfx950: forward and feature gradient.
+// Wavefront-per-strip DDF kernels for gfx950: forward, feature gradient, filter
+// gradients (optionally with the feature gradient fused in).
 //
-// One 64-lane wavefront (a workgroup of its own) owns a full-width row strip of
-// one sample and walks a range of its channels.  Lanes are laid out 2-D over
-// the strip's work cells - LW = 2^k >= cols lanes per cell row, 64/LW cell rows
-// per pass ("slot"), PS slots per lane - so that LDS addresses are linear in
-// the lane id (no bank conflicts) and no division is needed to find a cell.
+// One 64-lane wavefront owns a full-width row strip of one sample and walks a
+// range of its channels.  Lanes are laid out 2-D over the strip's work cells -
+// LW = 2^k >= cols lanes per cell row, 64/LW cell rows per pass ("slot"), PS
+// slots per lane - so that LDS addresses are linear in the lane id (no bank
+// conflicts) and no division is needed to find a cell.
 //
 // Per channel the wave
-//   1. copies the source strip (X, or dO for the feature gradient) from global
-//      memory with 16-byte loads, a few channels ahead of use, and scatters it
-//      into a zero-bordered LDS tile (the border makes the tap loop free of
-//      bounds tests),
+//   1. copies the source strip (X, dO) from global memory with 16-byte loads, a
+//      few channels ahead of use, and scatters it into a zero-bordered LDS tile
+//      of accumulator-type values (the border makes the tap loop free of bounds
+//      tests; fp16 is widened here, once per element),
 //   2. runs the tap loop for its PS cells out of LDS, with the spatial-filter
 //      taps of those cells held in registers for the whole channel walk and
-//      the channel-filter taps of the current channel in scalar registers,
+//      the channel-filter taps of its channels staged once in LDS (read back as
+//      wave-uniform values),
 //   3. writes the results to a linear LDS copy of the result strip and stores
 //      that with 16-byte accesses.
-// The global side is therefore a plain linear copy in both directions, and a
-// wave never waits for another wave: there is no workgroup barrier at all.
+// The global side is therefore a plain linear copy in both directions, and in
+// the channel walk a wave never waits for another wave: there is no workgroup
+// barrier in forward and feature gradient, and only the final dSF sum over a
+// block's four waves has barriers in the filter-gradient kernel.
 #pragma once
 
 #include <type_traits>
@@ -173,6 +177,8 @@ __device__ __forceinline__ void load_taps(const A *taps, int ci, A (&w)[KK]) {
 }
 
 // Channels in flight per wave for a given number of vectors per channel.
+// (Deeper pipelines for the narrow element types were measured and do not pay:
+// the extra registers cost more occupancy than the prefetch distance gains.)
 template <int NV>
 constexpr int stages() { return NV <= 1 ? 4 : (NV <= 2 ? 2 : 1); }
 
