@@ -205,6 +205,39 @@ def test_closed_form_depthwise_conv_on_device():
 
 
 # ---------------------------------------------------------------------------
+# committed known-answer fixtures
+# ---------------------------------------------------------------------------
+def _golden_paths():
+    import glob
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
+    return sorted(glob.glob(os.path.join(here, '*.npz')))
+
+
+@pytest.mark.parametrize('version', VERSIONS)
+@pytest.mark.parametrize('dtype', DTYPES, ids=_ids)
+@pytest.mark.parametrize('path', _golden_paths(), ids=lambda p: p.split('/')[-1][:-4])
+def test_golden_fixtures(path, dtype, version):
+    """HIP kernels against tests/golden/*.npz (inputs and fp64 results frozen by
+    tests/golden/make_fixtures.py).  For fp32 and fp16 the inputs are rounded
+    first, so the expected values are recomputed from the rounded inputs by the
+    oracle, which test_oracle.py holds to the same fixtures."""
+    import numpy as np
+    z = np.load(path, allow_pickle=False)
+    k, d, s = int(z['k']), int(z['d']), int(z['s'])
+    combine = 'mul' if int(z['combine']) == 0 else 'add'
+    x, cf, sf, go = (torch.from_numpy(z[n]).to(dtype) for n in ('x', 'cf', 'sf', 'go'))
+    got = run_ddf(x, cf, sf, go, k, d, s, combine, version)
+    if dtype == torch.float64:
+        want = [torch.from_numpy(z[n]) for n in ('out', 'dx', 'dcf', 'dsf')]
+    else:
+        want = [oracle.forward(x, cf, sf, k, d, s, combine)] + \
+            list(oracle.backward(go, x, cf, sf, k, d, s, combine))
+    for g, w, name in zip(got, want, ('out', 'dX', 'dCF', 'dSF')):
+        assert rel_err(g, w) <= TOL[dtype], name
+
+
+# ---------------------------------------------------------------------------
 # API behaviour
 # ---------------------------------------------------------------------------
 def test_needs_input_grad_subsets():

@@ -180,3 +180,43 @@ def test_make_inputs_is_deterministic_and_standardized():
     assert (cf.view(2, 4, 9).std(2) - 1).abs().max() < 1e-5
     assert sf.mean(1).abs().max() < 1e-6
     assert (sf.std(1) - 1).abs().max() < 1e-5
+
+
+# ---------------------------------------------------------------------------
+# committed known-answer fixtures (tests/golden/*.npz, written by
+# tests/golden/make_fixtures.py from the loop form and torch autograd)
+# ---------------------------------------------------------------------------
+def golden_cases():
+    import glob
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'golden')
+    return sorted(glob.glob(os.path.join(here, '*.npz')))
+
+
+def load_golden(path):
+    import numpy as np
+    z = np.load(path, allow_pickle=False)
+    t = {n: torch.from_numpy(z[n]) for n in ('x', 'cf', 'sf', 'go', 'out', 'dx', 'dcf', 'dsf')}
+    return t, int(z['k']), int(z['d']), int(z['s']), 'mul' if int(z['combine']) == 0 else 'add'
+
+
+def test_golden_fixtures_exist():
+    assert len(golden_cases()) >= 8
+
+
+@pytest.mark.parametrize('path', golden_cases(), ids=lambda p: p.split('/')[-1][:-4])
+def test_c_oracle_reproduces_golden_fixtures(path):
+    """The compiled oracle (the checker of every GPU test) against the frozen
+    loop-form / autograd results: fp64 to 1e-12, fp32 entry points to 1e-5."""
+    t, k, d, s, combine = load_golden(path)
+    out = oracle.forward(t['x'], t['cf'], t['sf'], k, d, s, combine)
+    grads = oracle.backward(t['go'], t['x'], t['cf'], t['sf'], k, d, s, combine)
+    for got, name in zip((out,) + tuple(grads), ('out', 'dx', 'dcf', 'dsf')):
+        scale = max(t[name].abs().max().item(), 1e-30)
+        assert (got - t[name]).abs().max().item() / scale < 1e-12, name
+    f = [t[n].float() for n in ('x', 'cf', 'sf', 'go')]
+    out32 = oracle.forward_f32(f[0], f[1], f[2], k, d, s, combine)
+    g32 = oracle.backward_f32(f[3], f[0], f[1], f[2], k, d, s, combine)
+    for got, name in zip((out32,) + tuple(g32), ('out', 'dx', 'dcf', 'dsf')):
+        scale = max(t[name].abs().max().item(), 1e-30)
+        assert (got.double() - t[name]).abs().max().item() / scale < 1e-5, name
