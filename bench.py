@@ -294,6 +294,43 @@ def model_inference(batch=128, steps=10, warmup=3):
             'ddf_ms_per_batch': round(ddf_ms, 3), 'ddf_layers': layers}
 
 
+def test_time_table(iters=20, warmup=5):
+    """The reference's own micro-benchmark (test_time.py:54-145): a 3x3
+    convolution, a depthwise 3x3 convolution, a DDFPack layer and the bare ddf
+    operator ('mul', k=3) on fp32 feature maps of 256 channels, inference only.
+    Times are per call in milliseconds, between stream events."""
+    import torch.nn as nn
+    from ddfnet_amd import DDFPack, ddf
+    shapes = [(2, 200, 300), (32, 224, 224), (32, 112, 112), (32, 56, 56), (32, 28, 28),
+              (32, 14, 14), (32, 7, 7)]
+    torch.manual_seed(0)
+    conv = nn.Conv2d(256, 256, 3, padding=1).cuda().eval()
+    dw_conv = nn.Conv2d(256, 256, 3, padding=1, groups=256).cuda().eval()
+    layer = DDFPack(256).cuda().eval()
+    rows = []
+    with torch.no_grad():
+        for n, h, w in shapes:
+            feat = torch.randn(n, 256, h, w, device='cuda')
+            spatial = torch.rand(n, 9, h, w, device='cuda')
+            channel = torch.rand(n, 256, 3, 3, device='cuda')
+            row = {'shape': [n, 256, h, w]}
+            for name, fn in (('conv', lambda: conv(feat)), ('dw_conv', lambda: dw_conv(feat)),
+                             ('ddf_layer', lambda: layer(feat)),
+                             ('ddf_op', lambda: ddf(feat, channel, spatial, 3, 1, 1, 'mul'))):
+                for _ in range(warmup):
+                    fn()
+                row[name + '_ms'] = round(timed(lambda i: fn(), iters), 4)
+            ab = algorithmic_bytes(n, 256, h, w, 3, 1, 4)['fwd']
+            row['ddf_op_gbps'] = round(ab / (row['ddf_op_ms'] * 1e-3) / 1e9, 1)
+            rows.append(row)
+            log('[test_time] %s conv %.3f  dw_conv %.3f  ddf_layer %.3f  ddf_op %.3f ms (%.0f GB/s)' % (
+                row['shape'], row['conv_ms'], row['dw_conv_ms'], row['ddf_layer_ms'],
+                row['ddf_op_ms'], row['ddf_op_gbps']))
+            del feat, spatial, channel
+            torch.cuda.empty_cache()
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -302,6 +339,9 @@ def main():
     ap.add_argument('--workload', default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument('--all', action='store_true', help='also time the other workloads')
     ap.add_argument('--model', action='store_true', help='also time ddf_mul_resnet50 inference')
+    ap.add_argument('--test-time', action='store_true',
+                    help="also run the reference's micro-benchmark table (conv, depthwise conv, "
+                         "DDFPack, ddf at seven 256-channel shapes)")
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--copy-probe', action='store_true',
                     help='also run a plain 256 MiB device copy (calibrates hardware counters)')
@@ -358,6 +398,8 @@ def main():
         log('[model] %s bs%d %s: %.1f images/s (%.2f ms/batch, DDF layers %.2f ms)' % (
             mi['model'], mi['batch'], mi['dtype'], mi['images_per_s'], mi['ms_per_batch'],
             mi['ddf_ms_per_batch']))
+    if args.test_time:
+        line['test_time'] = test_time_table()
     if not args.no_cpu:
         line['cpu_baseline'] = cpu_baseline(args.workload)
         cb = line['cpu_baseline']
