@@ -27,6 +27,8 @@ SYMBOLS = {
     'ddf_hip_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 6 + [_vp]),
     'ddf_hip_backward_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u, _i]),
     'ddf_hip_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
+    'ddf_hip_filter_norm': (_i, [_vp] * 2 + [_i64] * 2 + [_i, _i64, ctypes.c_double] + [_vp] * 2 +
+                            [_i, _vp]),
 }
 
 _lib = None
@@ -67,8 +69,32 @@ def _ptr(t):
     return None if t is None else ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, '_cuda_getCurrentRawStream', None)
+
+
 def _stream():
+    """torch's current stream on the current device, as a hipStream_t."""
+    if _raw_stream is not None:   # same value, without building a Stream object
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class on_device_of(object):
+    """Device guard that costs nothing when the tensor already lives on the
+    current device (the common case)."""
+
+    def __init__(self, tensor):
+        idx = tensor.device.index
+        self.guard = None if idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
 
 
 def forward(features, channel_filter, spatial_filter, output, k, d, s, combine, variant=''):
@@ -97,3 +123,16 @@ def backward(grad_output, features, channel_filter, spatial_filter, grad_feature
         _ptr(grad_features), _ptr(grad_channel_filter), _ptr(grad_spatial_filter),
         _ptr(workspace), ws_bytes, N, C, H, W, k, d, s, COMBINE[combine],
         DTYPE[features.dtype], need, VARIANT[variant], _stream()))
+
+
+def filter_norm(x, outer, groups, taps, inner, gain, gain_vec=None, offset_vec=None):
+    """y = gain * standardised(x) + offset over the taps of a contiguous
+    (outer, groups, taps, inner) device tensor; returns a new tensor shaped
+    like ``x``.  Enqueued on torch's current stream."""
+    y = torch.empty_like(x)
+    with on_device_of(x):
+        rc = lib().ddf_hip_filter_norm(
+            _ptr(x), _ptr(y), outer, groups, taps, inner, float(gain), _ptr(gain_vec),
+            _ptr(offset_vec), DTYPE[x.dtype], _stream())
+    check(rc)
+    return y

@@ -195,4 +195,34 @@ int ddf_hip_backward(const void *grad_output, const void *features,
     }
 }
 
+int ddf_hip_filter_norm(const void *x, void *y, int64_t outer, int64_t groups, int taps,
+                        int64_t inner, double gain, const void *gain_vec, const void *offset_vec,
+                        int dtype, void *stream) {
+    if (outer < 0 || groups < 0 || taps < 0 || inner < 0)
+        return fail(DDF_ERR_BAD_ARG, "negative tensor size");
+    if (dtype != DDF_F16 && dtype != DDF_F32 && dtype != DDF_F64)
+        return fail(DDF_ERR_BAD_ARG, "unknown dtype %d", dtype);
+    if (outer * groups * taps * inner == 0) return DDF_OK;
+    if (!x || !y) return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t err;
+    switch (dtype) {
+        case DDF_F16:
+            err = ddf::filter_norm<__half>((const __half *)x, (__half *)y, outer, groups, taps,
+                                           inner, gain, (const __half *)gain_vec,
+                                           (const __half *)offset_vec, st);
+            break;
+        case DDF_F32:
+            err = ddf::filter_norm<float>((const float *)x, (float *)y, outer, groups, taps, inner,
+                                          gain, (const float *)gain_vec,
+                                          (const float *)offset_vec, st);
+            break;
+        default:
+            err = ddf::filter_norm<double>((const double *)x, (double *)y, outer, groups, taps,
+                                           inner, gain, (const double *)gain_vec,
+                                           (const double *)offset_vec, st);
+    }
+    return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_filter_norm launch");
+}
+
 }  // extern "C"

@@ -56,6 +56,13 @@ hipError_t generic_backward(const Problem &p, const T *go, const T *x, const T *
                             const T *sf, T *dx, T *dcf, T *dsf, unsigned need,
                             hipStream_t st);
 
+// y = gain * standardised(x) + offset over the `taps` axis of an
+// (outer, groups, taps, inner) tensor; gain_vec / offset_vec are (groups, taps)
+// or null (then the scalar `gain` / no offset).
+template <typename T>
+hipError_t filter_norm(const T *x, T *y, int64_t outer, int64_t groups, int taps, int64_t inner,
+                       double gain, const T *gain_vec, const T *offset_vec, hipStream_t st);
+
 bool tiled_forward_supported(const Problem &p, int dtype);
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,

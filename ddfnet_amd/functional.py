@@ -56,7 +56,7 @@ class _NativeOp(object):
                                     ('channel_filter', channel_filter),
                                     ('spatial_filter', spatial_filter),
                                     ('output', output)))
-        with torch.cuda.device(features.device):
+        with _lib.on_device_of(features):
             _lib.forward(features, channel_filter, spatial_filter, output,
                          kernel_size, dilation, stride, self.combine, self.variant)
         return 1
@@ -77,7 +77,7 @@ class _NativeOp(object):
                                     ('spatial_filter', spatial_filter)) +
                                    tuple((n, t) for n, t, _ in grads))
         need = sum(bit for _, t, bit in grads if t is not None)
-        with torch.cuda.device(features.device):
+        with _lib.on_device_of(features):
             nbytes = _lib.backward_workspace_bytes(
                 features.shape, kernel_size, dilation, stride, self.combine,
                 features.dtype, need, self.variant)

@@ -11,6 +11,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 from torch.nn.init import calculate_gain
 
+from . import _lib
 from .functional import ddf
 
 __all__ = ['FilterNorm', 'build_spatial_branch', 'build_channel_branch',
@@ -57,7 +58,30 @@ class FilterNorm(nn.Module):
             x = x + self.mean.view(shape)
         return x
 
+    def _fused(self, x, outer, inner):
+        """One HIP launch instead of the chain of elementwise ops below.  Used
+        where no gradient is wanted (the kernel has no backward): inference."""
+        taps = x.numel() // max(outer * self.in_channels * inner, 1)
+        gain_vec = self.std.to(x.dtype) if self.runing_std else None
+        offset_vec = self.mean.to(x.dtype) if self.runing_mean else None
+        return _lib.filter_norm(x.contiguous(), outer, self.in_channels, taps, inner,
+                                1.0 if self.runing_std else self.std, gain_vec, offset_vec)
+
+    def _use_fused(self, x):
+        if not x.is_cuda or x.dtype not in _lib.DTYPE or x.numel() == 0:
+            return False
+        if not torch.is_grad_enabled():
+            return True
+        params = [p for p in (self.std, getattr(self, 'mean', None)) if isinstance(p, nn.Parameter)]
+        return not (x.requires_grad or any(p.requires_grad for p in params))
+
     def forward(self, x):
+        if self._use_fused(x):
+            if self.filter_type == 'spatial':
+                b, ch, h, w = x.size()
+                return self._fused(x, b, h * w).reshape(b, ch, h, w)
+            b = x.size(0)
+            return self._fused(x.reshape(b, -1), b, 1)
         if self.filter_type == 'spatial':
             b, ch, h, w = x.size()
             x = _standardize(x.reshape(b, self.in_channels, -1, h, w), 2)
@@ -111,11 +135,27 @@ class DDFPack(nn.Module):
         self.channel_branch = build_channel_branch(
             in_channels, kernel_size, nonlinearity, se_ratio)
 
+    def _channel_filter(self, x):
+        """The channel branch.  Its two 1x1 convolutions act on a pooled
+        (b, c, 1, 1) tensor, i.e. they are matrix products: evaluating them as
+        such (same parameters, same arithmetic) avoids the convolution
+        library's launch path, which costs more host time than the whole layer
+        has GPU work at small feature maps."""
+        branch = self.channel_branch
+        if not (x.is_cuda and isinstance(branch, nn.Sequential) and len(branch) == 5 and
+                isinstance(branch[0], nn.AdaptiveAvgPool2d) and isinstance(branch[2], nn.ReLU) and
+                all(isinstance(m, nn.Conv2d) and m.kernel_size == (1, 1) for m in (branch[1], branch[3]))):
+            return branch(x)   # not the stock branch: run it as it is
+        fc1, fc2, norm = branch[1], branch[3], branch[4]
+        v = x.mean((2, 3))
+        v = F.relu(F.linear(v, fc1.weight.flatten(1), fc1.bias))
+        return norm(F.linear(v, fc2.weight.flatten(1), fc2.bias))
+
     def forward(self, x):
         b, c, h, w = x.shape
         g, k, s = self.head, self.kernel_size, self.stride
         ho, wo = h // s, w // s
-        cf = self.channel_branch(x).reshape(b * g, c // g, k, k)
+        cf = self._channel_filter(x).reshape(b * g, c // g, k, k)
         sf = self.spatial_branch(x).reshape(b * g, k * k, ho, wo)
         out = ddf(x.reshape(b * g, c // g, h, w), cf, sf,
                   k, self.dilation, s, self.kernel_combine)

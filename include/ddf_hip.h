@@ -124,6 +124,24 @@ int ddf_hip_backward(const void *grad_output, const void *features,
                      int combine, int dtype, unsigned need_mask, int variant,
                      void *stream);
 
+/*
+ * Filter normalisation of the two filter branches, one launch.  Restates
+ * FilterNorm.forward of the reference (ddf/ddf.py:145-173), which is a chain
+ * of elementwise and reduction ops there.  `x` and `y` are dense
+ * (outer, groups, taps, inner) tensors; every filter, i.e. the `taps` values
+ * at fixed (outer, group, inner), is standardised with its own mean and
+ * unbiased standard deviation (+1e-10 in the denominator), multiplied by
+ * `gain_vec[group*taps + tap]` (or by the scalar `gain` when gain_vec is
+ * NULL) and shifted by `offset_vec[group*taps + tap]` (unless NULL).
+ * Spatial branch: (b, head, k*k, h*w).  Channel branch: (b, c, k*k, 1).
+ * `y` may alias `x`.  Forward only: training keeps the framework's autograd
+ * through the unfused formulation.
+ */
+int ddf_hip_filter_norm(const void *x, void *y, int64_t outer, int64_t groups,
+                        int taps, int64_t inner, double gain,
+                        const void *gain_vec, const void *offset_vec,
+                        int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

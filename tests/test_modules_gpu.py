@@ -118,3 +118,45 @@ def test_resnet50_fp16_inference_and_layer_timing():
     want = ([(64, 56, 1)] * 3 + [(128, 56, 2)] + [(128, 28, 1)] * 3 + [(256, 28, 2)] +
             [(256, 14, 1)] * 5 + [(512, 14, 2)] + [(512, 7, 1)] * 2)
     assert shapes == want
+
+
+# ---------------------------------------------------------------------------
+# fused filter normalisation (inference path of FilterNorm)
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize('dtype,tol', [(torch.float64, 1e-12), (torch.float32, 1e-5),
+                                       (torch.float16, 1e-2)])
+@pytest.mark.parametrize('ftype,shape,groups,k,rstd,rmean', [
+    ('spatial', (3, 9, 13, 11), 1, 3, False, False),
+    ('spatial', (2, 4 * 9, 7, 5), 4, 3, True, True),
+    ('spatial', (1, 25, 6, 6), 1, 5, False, True),
+    ('channel', (4, 16 * 9), 16, 3, True, False),
+    ('channel', (2, 5 * 25, 1, 1), 5, 5, True, True),
+    ('channel', (3, 7 * 9), 7, 3, False, False),
+])
+def test_fused_filter_norm_matches_formula(ftype, shape, groups, k, rstd, rmean, dtype, tol):
+    """One HIP launch (no gradient wanted) against the op-by-op formulation of
+    the same module evaluated in fp64 on the CPU."""
+    torch.manual_seed(3)
+    fn = ddfnet_amd.FilterNorm(groups, k, ftype, 'relu', running_std=rstd,
+                               running_mean=rmean).cuda().to(dtype)
+    x = (torch.randn(*shape) * 2 + 0.5).to(dtype).cuda()
+    with torch.no_grad():
+        assert fn._use_fused(x)
+        got = fn(x)
+    assert got.dtype == dtype
+    ref = copy.deepcopy(fn).cpu().double()
+    want = ref(x.detach().cpu().double().requires_grad_(True))   # grad wanted: unfused path
+    assert got.shape == want.shape
+    err = (got.cpu().double() - want.detach()).abs().max().item() / want.abs().max().item()
+    assert err <= tol, err
+
+
+def test_filter_norm_training_path_keeps_autograd():
+    fn = ddfnet_amd.FilterNorm(8, 3, 'channel', 'relu', running_std=True).cuda()
+    x = torch.randn(2, 72, device='cuda', requires_grad=True)
+    assert not fn._use_fused(x)
+    fn(x).sum().backward()
+    assert x.grad is not None and fn.std.grad is not None
+    with torch.no_grad():
+        fused = fn(x)
+    assert torch.allclose(fused, fn(x).detach(), rtol=1e-5, atol=1e-6)
