@@ -255,8 +255,8 @@ __device__ __forceinline__ void store_strip(const T *lds, T *__restrict__ dst, i
                                             int lane) {
     const int nvec = n_elems / V;
     for (int f = lane; f < nvec; f += kWave)
-        *reinterpret_cast<Raw<T, V> *>(dst + f * V) =
-            *reinterpret_cast<const Raw<T, V> *>(lds + f * V);
+        __builtin_nontemporal_store(*reinterpret_cast<const Raw<T, V> *>(lds + f * V),
+                                    reinterpret_cast<Raw<T, V> *>(dst + f * V));
 }
 
 template <typename T>
