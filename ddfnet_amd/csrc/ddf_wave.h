@@ -842,13 +842,17 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     constexpr int NST = Stg::NST;
     constexpr int NG = (PS + V - 1) / V;
     extern __shared__ __align__(16) unsigned char smem[];
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    // (the wave index is the same in all lanes: say so, or everything derived from
+    // it - channel range, pointers, loop bounds - is computed per lane)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     // private LDS of this wave: X tile, [dO tile,] linear strip (dO in, or dX out), taps
     A *lds_in = reinterpret_cast<A *>(smem + (size_t)wave * g.lds_wave_bytes);
     A *lds_g = lds_in + g.tile + kSpare;
     T *lds_go = reinterpret_cast<T *>(lds_g + (DX ? g.tile + kSpare : 0));
     A *taps = reinterpret_cast<A *>(lds_go + g.lin_tile + kIdle);
 
+    DDF_STAMP(0);
     WaveWork ww;
     if (!ww.init(g)) return;   // whole block leaves together
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
@@ -905,6 +909,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         if constexpr (kStageFilter) nfs.issue(sf + ww.n * KK * oplane, oplane, stg.goff);
         tst.issue(cf, ww.n * g.C + c_first, nch1, lane);
     }
+    DDF_STAMP(1);
 
     bool ok[PS];
     int lb[PS], ob[PS];
@@ -953,7 +958,10 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         if constexpr (kStageFilter) nfs.collect(lds_g, stg.lo, lb, P, sfg);
     }
     wave_sync();
-    const int idle = g.lin_tile + lane;   // where idle lanes put their dX values
+    DDF_STAMP(2);
+    int wb[PS];   // where the dX value of a slot goes: idle lanes write behind the strip
+#pragma unroll
+    for (int m = 0; m < PS; ++m) wb[m] = ok[m] ? ob[m] : g.lin_tile + lane;
     T *ds = DX ? dx + (ww.n * g.C + c_first) * iplane + (int64_t)y0 * g.W : nullptr;
     const int n_out = ww.nrows * g.W;      // elements of the dX strip (DX: stride 1)
 
@@ -962,6 +970,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         stg.template commit<ST>(lds_in);
         if constexpr (DX) stg_g.template commit<ST>(lds_g);
         else sgo.template commit<ST>(lds_go);
+        DDF_STAMP(3 + 4 * ci);
         stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch1 - 1) * iplane);
         issue_go(st_tag, gs + (int64_t)min(ci + NST, nch1 - 1) * oplane);
         wave_sync();
@@ -1001,13 +1010,15 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
                     for (int j = 0; j < K; ++j)
                         accx += (A)ld(lds_g + lb[m] + (2 * R - i) * D * P + (2 * R - j) * D) *
                                 comb<MUL, A>(w[i * K + j], sfg[m][i * K + j]);
-                st(lds_go + (ok[m] ? ob[m] : idle), accx);
+                st(lds_go + wb[m], accx);
             }
         }
+        DDF_STAMP(4 + 4 * ci);
         if constexpr (DX) {
             wave_sync();
             store_strip<T, V>(lds_go, ds + (int64_t)ci * iplane, n_out, lane);
         }
+        DDF_STAMP(5 + 4 * ci);
         if (want_cf) {
             const A tot = bfly_sum<KK, 0, A>(pcf, lane);
             if (lane < bfly_writers<KK>()) {
@@ -1017,6 +1028,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
             }
         }
         wave_sync();
+        DDF_STAMP(6 + 4 * ci);
     };
     auto group = [&](int c) __attribute__((always_inline)) {
         channel(std::integral_constant<int, 0>{}, c);
@@ -1037,9 +1049,11 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         }
     }
 
+    DDF_STAMP(70);
     if (!want_sf) return;
     // Add the waves' dSF accumulators: one pixel slot at a time through LDS.
     __syncthreads();
+    DDF_STAMP(71);
     A *red = reinterpret_cast<A *>(smem);
 #pragma unroll
     for (int m = 0; m < PS; ++m) {
@@ -1059,6 +1073,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         }
         __syncthreads();
     }
+    DDF_STAMP(72);
 }
 
 // out[o, i] = sum_p part[o, p, i] for o < outer, p < parts, i < inner.  A
