@@ -199,6 +199,8 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
         while (t.wpb > 1 && t.lds_wave_bytes * t.wpb > 48 * 1024) --t.wpb;
     }
     t.lds_bytes = t.lds_wave_bytes * (filters ? waves_per_block : t.wpb);
+    if (fused)    // the spatial-filter tiles shared by the block's waves
+        t.lds_bytes += p.kk * (t.tile + wave::kSpare) * asz;
     if (filters)  // the cross-wave sum of the dSF accumulators reuses the block's LDS
         t.lds_bytes = std::max(t.lds_bytes, waves_per_block * p.kk * kWave * acc_size(dtype));
     if (t.lds_bytes > 64 * 1024) return false;

@@ -899,14 +899,30 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     }
     FilterStager<T, V, NG, KK> fst;
     TapStager<KK, T, A> tst;
-    // neighbour cells' spatial filter for dX: through the tile when it is a
-    // few vectors per plane, gathered otherwise (see k_backward_features)
-    constexpr bool kStageFilter = DX && V > 1 && NV * V <= 8;
-    NeighbourFilterStager<T, V, kStageFilter ? NV : 1, K, D, 1> nfs;
+    // DX: the block's four waves need the same spatial filter (same sample, same
+    // strip), at their cells and at the neighbour cells.  Each wave brings in
+    // every fourth tap plane, laid out like a dO tile (zero border), into LDS
+    // shared by the block; after one barrier every wave picks its registers
+    // out of the nine tiles.
+    static_assert(!DX || (V > 1 && NV * V <= 8), "fused kernel: short strips only");
+    constexpr int kTapsPerWave = (KK + kFilterWaves - 1) / kFilterWaves;
+    A *sf_tiles = reinterpret_cast<A *>(smem + (size_t)kFilterWaves * g.lds_wave_bytes);
+    const int sf_pitch = g.tile + kSpare;
+    Vec<T, V> sfv[DX ? kTapsPerWave : 1][NV];
     if (kFilters) {
-        fst.init(ww.nrows * g.Wo, lane);
-        fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
-        if constexpr (kStageFilter) nfs.issue(sf + ww.n * KK * oplane, oplane, stg.goff);
+        if constexpr (DX) {
+#pragma unroll
+            for (int q = 0; q < kTapsPerWave; ++q) {
+                const int t = min(wave + q * kFilterWaves, KK - 1);   // clamped: no branch
+#pragma unroll
+                for (int j = 0; j < NV; ++j)
+                    sfv[q][j] = *reinterpret_cast<const Vec<T, V> *>(
+                        sf + (ww.n * KK + t) * oplane + stg.goff[j]);
+            }
+        } else {
+            fst.init(ww.nrows * g.Wo, lane);
+            fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
+        }
         tst.issue(cf, ww.n * g.C + c_first, nch1, lane);
     }
     DDF_STAMP(1);
@@ -926,20 +942,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
             sfr[m][t] = 0;
             acc_sf[m][t] = 0;
         }
-        if constexpr (DX && !kStageFilter) {
-            const int cy = y0 + row;
-#pragma unroll
-            for (int i = 0; i < K; ++i)
-#pragma unroll
-                for (int j = 0; j < K; ++j) {
-                    const int sy = cy - (i - R) * D, sx = col - (j - R) * D;
-                    const bool in = ok[m] && sy >= 0 && sy < g.Ho && sx >= 0 && sx < g.Wo;
-                    // out-of-range neighbours read element 0 and are zeroed: no branch
-                    const A val = ld(sf + (ww.n * KK + i * K + j) * oplane +
-                                     (in ? (int64_t)sy * g.Wo + sx : 0));
-                    sfg[m][i * K + j] = in ? val : A(0);
-                }
-        }
     }
     stg.init_tile(g, y0 * S + g.row0_off, lane);
     if constexpr (DX) {
@@ -953,9 +955,35 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     if constexpr (DX) zero_tile(lds_g, g.tile, lane);
     if (kFilters) {
         tst.put(taps, nch, lane);
-        fst.collect(lds_go, ob, sfr);
-        wave_sync();
-        if constexpr (kStageFilter) nfs.collect(lds_g, stg.lo, lb, P, sfg);
+        if constexpr (DX) {
+#pragma unroll
+            for (int q = 0; q < kTapsPerWave; ++q) {
+                const int t = wave + q * kFilterWaves;
+                if (t < KK) {
+                    A *tile_t = sf_tiles + t * sf_pitch;
+                    zero_tile(tile_t, g.tile, lane);
+                    wave_sync();
+#pragma unroll
+                    for (int j = 0; j < NV; ++j)
+#pragma unroll
+                        for (int k = 0; k < V; ++k) tile_t[stg.lo[j][k]] = ld(&sfv[q][j].e[k]);
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const A *tile_t = sf_tiles + (i * K + j) * sf_pitch;
+#pragma unroll
+                    for (int m = 0; m < PS; ++m) {
+                        sfr[m][i * K + j] = tile_t[lb[m] + R * D * P + R * D];
+                        sfg[m][i * K + j] = tile_t[lb[m] + (2 * R - i) * D * P + (2 * R - j) * D];
+                    }
+                }
+        } else {
+            fst.collect(lds_go, ob, sfr);
+        }
     }
     wave_sync();
     DDF_STAMP(2);
