@@ -151,3 +151,60 @@ def test_ddf_resnet_has_sixteen_packs():
     packs = [m for m in model.modules() if isinstance(m, DDFPack)]
     assert len(packs) == 16
     assert [p.stride for p in packs].count(2) == 3
+
+
+# ---------------------------------------------------------------------------
+# host logic of the library and of bench.py (no device needed)
+# ---------------------------------------------------------------------------
+def test_workspace_size_is_host_arithmetic():
+    """The workspace query needs no device.  At the stage-3 benchmark shape the
+    filter gradients split the 256 channels 8 ways and keep the 14 rows in one
+    strip: 8 partial dSF tensors in fp32, no dCF partials."""
+    lib = _lib.lib()
+    n_sf = 64 * 9 * 14 * 14
+    assert lib.ddf_hip_backward_workspace_bytes(64, 256, 14, 14, 3, 1, 1, 0, 1, 7, 0) == 8 * n_sf * 4
+    # fp16 partial sums are fp32 as well; only the filter gradients need scratch
+    assert lib.ddf_hip_backward_workspace_bytes(64, 256, 14, 14, 3, 1, 1, 0, 0, 7, 0) == 8 * n_sf * 4
+    assert lib.ddf_hip_backward_workspace_bytes(64, 256, 14, 14, 3, 1, 1, 0, 1, 1, 0) == 0
+    # the generic kernels need none, whatever the shape
+    assert lib.ddf_hip_backward_workspace_bytes(64, 256, 14, 14, 3, 1, 1, 0, 1, 7, 1) == 0
+    assert lib.ddf_hip_backward_workspace_bytes(2, 3, 9, 9, 7, 1, 1, 0, 2, 7, 0) == 0
+
+
+def test_filter_norm_argument_validation_needs_no_gpu():
+    lib = _lib.lib()
+    assert lib.ddf_hip_filter_norm(None, None, -1, 1, 9, 4, 1.0, None, None, 1, None) == 1
+    assert lib.ddf_hip_filter_norm(None, None, 1, 1, 9, 4, 1.0, None, None, 7, None) == 1
+    assert lib.ddf_hip_filter_norm(None, None, 0, 1, 9, 4, 1.0, None, None, 1, None) == 0
+    assert lib.ddf_hip_filter_norm(None, None, 2, 1, 9, 4, 1.0, None, None, 1, None) == 1
+    assert b'null' in lib.ddf_hip_last_error()
+
+
+def _load_bench():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location('ddf_bench', os.path.join(ROOT, 'bench.py'))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_bench_algorithmic_bytes_match_the_measurement_plan():
+    """Bytes per call with every tensor touched once, at the stage-3 shape:
+    forward 26 731 520, backward 40 617 984."""
+    bench = _load_bench()
+    ab = bench.algorithmic_bytes(64, 256, 14, 14, 3, 1, 4)
+    assert ab['fwd'] == 26731520 and ab['bwd'] == 40617984
+    assert ab['dx'] + ab['dfilters'] > ab['bwd']   # two calls read dO, CF and SF twice
+    half = bench.algorithmic_bytes(64, 64, 56, 56, 3, 1, 2)
+    assert half['fwd'] == 55066624 and half['bwd'] == 84443136
+    s2 = bench.algorithmic_bytes(32, 128, 56, 56, 3, 2, 4)
+    assert s2['fwd'] == 65275904 and s2['bwd'] == 117706752
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--gpus', '2'],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 2
+    assert 'one GPU' in proc.stderr and proc.stdout.strip() == ''
