@@ -59,6 +59,17 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
         t.col_off = R * D; t.row0_off = -R * D;
         t.lin_cols = Wo; t.lin_rpc = 1; t.lin_rows = Ho;
     }
+    // Rows whose length is a multiple of 4 elements: widen the left border to 4
+    // columns and the pitch to a multiple of 4, so that every 4-element source
+    // vector lands on 4 neighbouring, 16-byte aligned tile elements.
+    const bool can_widen = dtype != DDF_F64 && t.src_cols % 4 == 0 && max_vec != 1 &&
+                           env_int("DDF_TUNE_VEC", 0) != 1 && env_int("DDF_TUNE_WIDE", 1) != 0;
+    if (can_widen) {
+        const int natural = t.col_off;
+        t.col_off = round_up(natural, 4);
+        t.lb_shift = t.col_off - natural;
+        t.P = round_up(t.P + t.lb_shift, 4);
+    }
     auto tile_rows = [&](int th) {
         return kind == kWaveFeatures ? th + halo_lo + halo_hi : (th - 1) * S + (K - 1) * D + 1;
     };
@@ -164,11 +175,12 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
         const int last_row = (t.slot_row[t.nslots - 1] + RS - 1) * step;
         const int last_col = (t.slot_col[t.nslots - 1] + LW - 1) * step;
         const int reach = kind == kWaveFeatures ? halo_lo + halo_hi : (K - 1) * D;
-        const int extent = (last_row + reach) * t.P + last_col + reach + 1;
+        const int extent = (last_row + reach) * t.P + last_col + reach + 1 + t.lb_shift;
         t.tile = round_up(std::max(t.IH * t.P, extent), 8);
     }
     t.lin_tile = round_up(t.TH * t.lin_rpc * t.lin_cols, 8);
     t.vec = best_v;
+    t.wide = (can_widen && best_v == 4) ? 1 : 0;
     t.nv = best_nv;
 
     // Channels per wave: enough waves to fill the machine several times over,

@@ -47,6 +47,8 @@ struct WaveGeom {
     int src_rows, src_cols;
     int P, IH, tile;          // tile: IH rows of pitch P elements, `tile` elements reserved
     int row0_off, col_off;    // source row of tile row 0 in strip 0; tile column of source column 0
+    int lb_shift;             // tile columns left of the leftmost tap (border wider than the halo)
+    int wide;                 // 1: a source vector lands on 4 aligned tile elements (one 16-byte LDS write)
     // result strip (out, or dX): `lin_cols` elements per row, `lin_rpc` rows per cell row
     int lin_cols, lin_rpc, lin_rows, lin_tile;
     int cpw, csplit;          // channels per wave; number of channel ranges (of cpw * waves per block)
@@ -240,8 +242,25 @@ struct Stager {
     // The tile holds accumulator-type values: fp16 is widened here, once per
     // element, instead of once per tap read; the tap reads are then aligned
     // 4-byte accesses for every storage type.
+    // `wide`: the geometry guarantees that the V = 4 elements of a vector are
+    // neighbours in the tile and start on a 16-byte boundary, so they go out as
+    // one write; the element-wise scatter has lanes 4 elements apart, an
+    // 8-way bank conflict per instruction.
     template <int ST>
-    __device__ __forceinline__ void commit(typename Acc<T>::type *lds) const {
+    __device__ __forceinline__ void commit(typename Acc<T>::type *lds, bool wide = false) const {
+        using A = typename Acc<T>::type;
+        if constexpr (V == 4 && sizeof(A) == 4) {
+            if (wide) {
+#pragma unroll
+                for (int j = 0; j < NV; ++j) {
+                    Vec<A, 4> w;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) w.e[k] = ld(&v[ST][j].e[k]);
+                    *reinterpret_cast<Raw<A, 4> *>(lds + lo[j][0]) = __builtin_bit_cast(Raw<A, 4>, w);
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int j = 0; j < NV; ++j)
 #pragma unroll
@@ -372,12 +391,13 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_forward(WaveGeom g, const T
         // idle lanes keep their lane-linear tile address (inside the LDS
         // allocation): a shared dummy address would collide with the banks of
         // the working lanes and double the time of every tap read
-        lb[m] = (row * S) * g.P + col * S;
+        lb[m] = (row * S) * g.P + col * S + g.lb_shift;
         ob[m] = ok[m] ? row * g.Wo + col : 0;   // idle lanes pick up pixel 0 (unused)
         wb[m] = ok[m] ? ob[m] : g.lin_tile + lane;   // ... and write behind the strip
     }
     stg.init_tile(g, y0 * S + g.row0_off, lane);
     const int P = pin(g.P);
+    const bool wide = g.wide != 0;
     zero_tile(lds_in, g.tile, lane);
     tst.put(taps, nch, lane);
     fst.collect(lds_out, ob, sfr);
@@ -385,7 +405,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_forward(WaveGeom g, const T
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
-        stg.template commit<ST>(lds_in);
+        stg.template commit<ST>(lds_in, wide);
         DDF_STAMP(3 + 4 * ci);
         stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch - 1) * iplane);
         wave_sync();
@@ -567,7 +587,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_backward_features(
         const int ql = g.slot_row[m] + lr, cx = g.slot_col[m] + lc;
         const int cy = qy0 + ql;
         ok[m] = m < g.nslots && ql < ww.nrows && cx < g.cols;
-        lb[m] = ql * g.P + cx;   // idle lanes keep a lane-linear (bank-conflict-free) address
+        lb[m] = ql * g.P + cx + g.lb_shift;   // idle lanes keep a lane-linear (bank-conflict-free) address
         ob[m] = ok[m] ? (ql * S) * g.W + cx * S : 0;
         // idle cells get coordinates outside the image: none of their results is kept
         cu[m] = ok[m] ? cy * S : g.H;
@@ -592,6 +612,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_backward_features(
     }
     stg.init_tile(g, qy0 + g.row0_off, lane);
     const int P = pin(g.P);
+    const bool wide = g.wide != 0;
     const int idle = g.lin_tile + lane;
     zero_tile(lds_in, g.tile, lane);
     tst.put(taps, nch, lane);
@@ -600,7 +621,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_backward_features(
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
-        stg.template commit<ST>(lds_in);
+        stg.template commit<ST>(lds_in, wide);
         stg.template issue<ST>(gs + (int64_t)min(ci + NST, nch - 1) * oplane);
         wave_sync();
         A w[KK];
@@ -935,7 +956,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     for (int m = 0; m < PS; ++m) {
         const int row = g.slot_row[m] + lr, col = g.slot_col[m] + lc;
         ok[m] = m < g.nslots && row < ww.nrows && col < g.cols;
-        lb[m] = (row * S) * g.P + col * S;     // lane-linear: no bank conflicts, idle lanes included
+        lb[m] = (row * S) * g.P + col * S + g.lb_shift;   // lane-linear: no bank conflicts, idle lanes included
         ob[m] = ok[m] ? row * g.Wo + col : 0;
 #pragma unroll
         for (int t = 0; t < KK; ++t) {
@@ -951,6 +972,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
             for (int k = 0; k < V; ++k) stg_g.lo[j][k] = stg.lo[j][k];
     }
     const int P = pin(g.P);
+    const bool wide = g.wide != 0;
     zero_tile(lds_in, g.tile, lane);
     if constexpr (DX) zero_tile(lds_g, g.tile, lane);
     if (kFilters) {
@@ -995,8 +1017,8 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
-        stg.template commit<ST>(lds_in);
-        if constexpr (DX) stg_g.template commit<ST>(lds_g);
+        stg.template commit<ST>(lds_in, wide);
+        if constexpr (DX) stg_g.template commit<ST>(lds_g, wide);
         else sgo.template commit<ST>(lds_go);
         DDF_STAMP(3 + 4 * ci);
         stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch1 - 1) * iplane);
