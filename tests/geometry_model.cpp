@@ -1,0 +1,196 @@
+// CPU model of the wave kernels' addressing.  For a list of problem shapes it asks the
+// library's own host code (ddf_tiled_host.hip, compiled into this program) for the launch
+// geometry and replays, lane by lane, every global and LDS address the kernels form from
+// it: vector offsets of the staged strips, tile offsets, the tap reach of every cell slot,
+// result strips, the block-id split, the LDS layout.  Prints one line per geometry and a
+// VIOLATION line for anything out of bounds or misaligned.  Built and run by
+// tests/test_geometry.py; no kernel is launched.
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+
+#include "ddf_tiled_host.hip"
+
+using namespace ddf;
+
+static int g_fails = 0;
+#define CHECK(cond, ...)                      \
+    do {                                      \
+        if (!(cond)) {                        \
+            if (g_fails < 10) {               \
+                printf("  VIOLATION: ");      \
+                printf(__VA_ARGS__);          \
+                printf("\n");                 \
+            }                                 \
+            ++g_fails;                        \
+        }                                     \
+    } while (0)
+
+static bool is_filters(int kind) { return kind == kWaveFilters || kind == kWaveFused; }
+
+// floor(n / d) through the magic number the kernels use (0 means d == 1)
+static long magic_div(long n, unsigned m) {
+    return m ? (long)(((unsigned long long)(unsigned)n * m) >> 32) : n;
+}
+
+static void check_geometry(int kind, long N, long C, long H, long W, int k, int d, int s, int dtype,
+                           int max_vec) {
+    const Problem p = make_problem(N, C, H, W, k, d, s, 0);
+    WaveGeom g;
+    int ps, nv;
+    if (!wave_geometry(p, dtype, kind, max_vec, &g, &ps, &nv)) {
+        printf("kind %d %ldx%ldx%ldx%ld k%d d%d s%d dt%d: unsupported\n", kind, N, C, H, W, k, d, s,
+               dtype);
+        return;
+    }
+    const int esz = dtype == 0 ? 2 : dtype == 1 ? 4 : 8, asz = dtype == 2 ? 8 : 4;
+    const int V = g.vec, KK = k * k, tap_pitch = (KK + 3) / 4 * 4;
+    const int S = s, D = d, R = (k - 1) / 2;
+    printf("kind %d %ldx%ldx%ldx%ld k%d d%d s%d dt%d: ps=%d nv=%d vec=%d wide=%d TH=%d nstrips=%d "
+           "nslots=%d lw=%d P=%d IH=%d tile=%d lin_tile=%d cpw=%d cpb=%d wpb=%d csplit=%d "
+           "nblocks=%d lds=%d (wave %d)\n",
+           kind, N, C, H, W, k, d, s, dtype, ps, nv, V, g.wide, g.TH, g.nstrips, g.nslots,
+           1 << g.lw_shift, g.P, g.IH, g.tile, g.lin_tile, g.cpw, g.cpb, g.wpb, g.csplit, g.nblocks,
+           g.lds_bytes, g.lds_wave_bytes);
+
+    CHECK(g.nslots <= ps, "nslots %d > ps %d", g.nslots, ps);
+    const long tile_elems = (long)g.tile + 8;   // tile plus its spare elements
+    const long plane_in = (long)g.src_rows * g.src_cols;
+    const int LW = 1 << g.lw_shift;
+
+    for (int strip = 0; strip < g.nstrips; ++strip) {
+        const int row_first = strip * g.TH, nrows = std::min(g.TH, g.rows - row_first);
+
+        // --- staged source strip: global vector offsets and tile offsets (Stager) ---
+        const int row0 = (kind == kWaveFeatures ? row_first : row_first * S) + g.row0_off;
+        const int r_lo = std::max(row0, 0);
+        const int n_rows = std::max(std::min(row0 + g.IH, g.src_rows) - r_lo, 0);
+        const int nvec = n_rows * g.src_cols / V, row_shift = r_lo - row0;
+        CHECK((n_rows * g.src_cols) % V == 0, "strip %d: staged %d elements, not a multiple of V",
+              strip, n_rows * g.src_cols);
+        CHECK(nvec <= 64 * nv, "strip %d: %d vectors > 64 * nv (%d)", strip, nvec, 64 * nv);
+        for (int lane = 0; lane < 64; ++lane)
+            for (int j = 0; j < nv; ++j) {
+                const int f = lane + 64 * j, e = f * V;
+                if (f >= nvec) continue;
+                int row = e / g.src_cols, col = e % g.src_cols;
+                const long goff = (long)r_lo * g.src_cols + e;
+                CHECK(goff + V <= plane_in, "strip %d: global source offset %ld + %d > plane %ld",
+                      strip, goff, V, plane_in);
+                CHECK((goff * esz) % (V * esz) == 0, "misaligned source vector");
+                if (g.wide) {
+                    const int lo0 = (row_shift + row) * g.P + g.col_off + col;
+                    CHECK(V == 4, "wide commits need V = 4");
+                    CHECK(lo0 % 4 == 0, "wide: tile offset %d not 16-byte aligned", lo0);
+                    CHECK(col + 3 < g.src_cols, "wide: vector straddles two rows");
+                }
+                for (int q = 0; q < V; ++q) {
+                    const int lo = (row_shift + row) * g.P + g.col_off + col;
+                    CHECK(lo >= 0 && lo < g.tile, "strip %d: tile offset %d outside tile %d (row %d col %d)",
+                          strip, lo, g.tile, row, col);
+                    if (++col >= g.src_cols) { col = 0; ++row; }
+                }
+            }
+
+        // --- cell slots: tap reach in the tile, position in the linear strip ---
+        for (int lane = 0; lane < 64; ++lane) {
+            const int lr = lane >> g.lw_shift, lc = lane & (LW - 1);
+            for (int m = 0; m < g.nslots; ++m) {
+                const int row = g.slot_row[m] + lr, col = g.slot_col[m] + lc;
+                const bool ok = row < nrows && col < g.cols;
+                const int step = kind == kWaveFeatures ? 1 : S;
+                const int reach = kind == kWaveFeatures ? (R * D) / S + (R * D + S - 1) / S : (k - 1) * D;
+                const long lb = (long)(row * step) * g.P + col * step + g.lb_shift;
+                const long far = lb + (long)reach * g.P + reach;
+                CHECK(far < tile_elems, "lane %d slot %d reads tile element %ld of %ld", lane, m, far,
+                      tile_elems);
+                if (!ok) continue;
+                if (kind != kWaveFeatures) {
+                    const long ob = (long)row * g.Wo + col;
+                    CHECK(ob < g.lin_tile, "strip offset %ld >= lin_tile %d", ob, g.lin_tile);
+                    CHECK((long)(row_first + row) * g.Wo + col < (long)g.Ho * g.Wo, "pixel outside plane");
+                } else {
+                    for (int a = 0; a < S; ++a)
+                        for (int c = 0; c < S; ++c) {
+                            const int u = (row_first + row) * S + a, v = col * S + c;
+                            if (u >= g.H || v >= g.W) continue;
+                            const long o = (long)(row * S + a) * g.W + v;
+                            CHECK(o < g.lin_tile, "dX strip offset %ld >= lin_tile %d", o, g.lin_tile);
+                        }
+                }
+            }
+        }
+
+        // --- result / linear strips: vector aligned, inside the plane, inside LDS ---
+        CHECK(plane_in % V == 0, "source plane %ld not a multiple of V", plane_in);
+        CHECK(((long)g.Ho * g.Wo) % V == 0, "output plane not a multiple of V");
+        if (kind == kWaveForward) {
+            const long n_out = (long)nrows * g.Wo;
+            const int NG = (ps + V - 1) / V;
+            CHECK(n_out % V == 0 && ((long)row_first * g.Wo) % V == 0, "output strip misaligned");
+            CHECK(n_out / V <= 64 * NG, "%ld spatial-filter vectors > 64 * NG (%d)", n_out / V, 64 * NG);
+            CHECK(n_out <= g.lin_tile, "output strip > lin_tile");
+            CHECK((long)row_first * g.Wo + n_out <= (long)g.Ho * g.Wo, "output strip outside plane");
+        }
+        if (kind == kWaveFeatures) {
+            const int u0 = row_first * S;
+            const long n_out = (long)std::min(nrows * S, g.H - u0) * g.W;
+            CHECK(n_out % V == 0 && ((long)u0 * g.W) % V == 0, "dX strip misaligned");
+            CHECK((long)u0 * g.W + n_out <= (long)g.H * g.W, "dX strip outside plane");
+            CHECK(n_out <= g.lin_tile, "dX strip %ld > lin_tile %d", n_out, g.lin_tile);
+        }
+        if (is_filters(kind)) {
+            const long n_go = (long)nrows * g.Wo;
+            const int NG = (ps + V - 1) / V;
+            CHECK(n_go % V == 0, "dO strip misaligned");
+            CHECK(n_go <= g.lin_tile, "dO strip > lin_tile");
+            CHECK(n_go / V <= 64 * NG, "%ld dO vectors > 64 * NG (%d)", n_go / V, 64 * NG);
+        }
+    }
+
+    // --- block id -> (sample, strip, channel split) through magic numbers ---
+    const long step = g.nblocks > 200000 ? 97 : 1;
+    for (long b = 0; b < g.nblocks; b += step) {
+        const long rest = magic_div(b, g.csplit_magic), cs = b - rest * g.csplit;
+        const long smp = magic_div(rest, g.nstrips_magic), strip = rest - smp * g.nstrips;
+        CHECK(rest == b / g.csplit && cs == b % g.csplit && smp == rest / g.nstrips &&
+                  strip == rest % g.nstrips,
+              "block split wrong at block %ld", b);
+    }
+    CHECK(magic_div(g.nblocks - 1, g.csplit_magic) == (g.nblocks - 1) / g.csplit, "split of the last block");
+    const long ngroups = ((long)g.nblocks + g.wpb - 1) / g.wpb;
+    CHECK((long)g.xcd_per * 8 >= ngroups && (long)(g.xcd_per - 1) * 8 < ngroups, "workgroups per XCD");
+
+    // --- LDS layout ---
+    const int waves = is_filters(kind) ? 4 : g.wpb;
+    const long used = (long)(g.tile + 8) * asz * (kind == kWaveFused ? 2 : 1) +
+                      (long)(g.lin_tile + 64) * esz + (long)g.cpw * tap_pitch * asz;
+    const long shared = kind == kWaveFused ? (long)KK * (g.tile + 8) * asz : 0;
+    CHECK(used <= g.lds_wave_bytes, "a wave uses %ld bytes of LDS, has %d", used, g.lds_wave_bytes);
+    CHECK(g.wpb >= 1 && g.wpb <= 4, "waves per workgroup %d", g.wpb);
+    CHECK((long)g.lds_wave_bytes * waves + shared <= g.lds_bytes, "workgroup LDS");
+    CHECK(g.lds_bytes <= 64 * 1024, "more than 64 KiB of LDS");
+    CHECK(g.cpw * KK <= 256, "%d taps staged, at most 256", g.cpw * KK);
+    CHECK((long)g.csplit * g.cpb >= C, "channels not covered");
+    if (g_fails) printf("  -> %d violations\n", g_fails);
+    g_fails = 0;
+}
+
+int main() {
+    const long shapes[][4] = {
+        {96, 64, 56, 56},   {64, 256, 14, 14}, {64, 128, 28, 28},  {64, 512, 7, 7},   {64, 64, 56, 56},
+        {32, 128, 56, 56},  {128, 512, 14, 14}, {1, 70, 10, 10},   {35, 1, 10, 10},   {1, 1, 50, 50},
+        {2, 3, 9, 11},      {1, 5, 2, 2},      {1, 2, 1, 1},       {1, 1, 1, 64},     {1, 1, 64, 1},
+        {2, 3, 20, 30},     {1, 2, 5, 200},    {1, 2, 31, 17},     {3, 65, 14, 14},   {2, 130, 7, 7},
+        {2, 256, 200, 300}, {32, 256, 224, 224}, {32, 256, 112, 112}, {1, 20, 40, 40}, {2, 9, 12, 16}};
+    const int kds[][3] = {{3, 1, 1}, {3, 2, 1}, {3, 1, 2}, {3, 2, 2}, {5, 1, 1}, {5, 2, 1}, {5, 1, 2}, {5, 2, 2}};
+    for (auto &sh : shapes)
+        for (auto &q : kds)
+            for (int dtype = 0; dtype < 3; ++dtype)
+                for (int kind = 0; kind < 4; ++kind)
+                    for (int max_vec = 0; max_vec < 2; ++max_vec) {
+                        if (sh[2] / q[2] == 0 || sh[3] / q[2] == 0) continue;
+                        check_geometry(kind, sh[0], sh[1], sh[2], sh[3], q[0], q[1], q[2], dtype, max_vec);
+                    }
+    return 0;
+}

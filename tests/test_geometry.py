@@ -1,0 +1,44 @@
+"""Host-side bounds model of the HIP kernels: no kernel is launched.
+
+tests/geometry_model.cpp includes the library's geometry code and replays the
+kernels' address arithmetic on the CPU for many shapes (the benchmark shapes,
+ragged ones, 1-pixel planes, wide images; every kernel size / dilation / stride
+the tuned family is built for; aligned and scalar-access plans).  A launch
+geometry that would make a kernel read or write out of bounds - the kind of
+mistake that faults a GPU - shows up here as a VIOLATION line instead."""
+import os
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _hipcc():
+    for cand in (os.environ.get('HIPCC'), '/opt/rocm/bin/hipcc', shutil.which('hipcc')):
+        if cand and os.path.exists(cand):
+            return cand
+    return None
+
+
+@pytest.mark.skipif(_hipcc() is None, reason='hipcc not available')
+def test_every_launch_geometry_stays_in_bounds(tmp_path):
+    exe = str(tmp_path / 'geometry_model')
+    cmd = [_hipcc(), '-O1', '-x', 'hip', '--cuda-host-only', '-w',
+           '-I' + os.path.join(ROOT, 'include'), '-I' + os.path.join(ROOT, 'ddfnet_amd', 'csrc'),
+           os.path.join(ROOT, 'tests', 'geometry_model.cpp'), '-o', exe]
+    build = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    assert build.returncode == 0, build.stdout + build.stderr
+    env = dict(os.environ)
+    for key in list(env):
+        if key.startswith('DDF_TUNE_'):
+            del env[key]
+    for extra in ({}, {'DDF_TUNE_WPB': '4'}, {'DDF_TUNE_WIDE': '0'}):
+        run = subprocess.run([exe], capture_output=True, text=True, timeout=600,
+                             env=dict(env, **extra))
+        assert run.returncode == 0
+        lines = run.stdout.splitlines()
+        assert sum(l.startswith('kind') and 'unsupported' not in l for l in lines) > 500
+        bad = [l for l in lines if 'VIOLATION' in l]
+        assert not bad, '\n'.join(bad[:10])
