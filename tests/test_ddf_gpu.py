@@ -371,3 +371,39 @@ def test_results_are_deterministic():
     b = run_ddf(x, cf, sf, go, 3, 1, 1, 'mul')
     for u, v in zip(a, b):
         assert torch.equal(u, v)
+
+
+def test_forward_and_backward_replay_in_a_hip_graph():
+    """The operator allocates nothing the capture cannot own and enqueues only
+    kernels (no memset nodes), so forward + backward can be captured once and
+    replayed.  Every replay - with ordinary eager work and synchronisation in
+    between - must reproduce the eager result bit for bit."""
+    from ddfnet_amd import ddf
+    shape = (4, 32, 14, 14)
+    host = [random_case(*shape, 3, 1, torch.float32, seed=s) for s in (21, 22, 23)]
+    x, cf, sf, go = (t.clone().requires_grad_(i < 3) for i, t in enumerate(to_dev(*host[0])))
+
+    def step():
+        out = ddf(x, cf, sf, 3, 1, 1, 'mul')
+        return (out,) + torch.autograd.grad(out, (x, cf, sf), go)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for case in host:
+        with torch.no_grad():
+            for dst, src in zip((x, cf, sf, go), to_dev(*case)):
+                dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in captured]
+        want = step()          # eager, between replays
+        torch.cuda.synchronize()
+        for g, w in zip(got, want):
+            assert torch.equal(g, w)
