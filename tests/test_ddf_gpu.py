@@ -293,6 +293,14 @@ def test_non_contiguous_inputs_are_accepted():
     assert not xt.is_contiguous()
     got = ddf(xt, cf.cuda(), sf.cuda(), 3, 1, 1, 'add')
     assert rel_err(got, oracle.forward(x, cf, sf, 3, 1, 1, 'add')) <= 1e-5
+    # channels_last features and gradients (what a channels_last network hands over)
+    xc = x.cuda().to(memory_format=torch.channels_last).requires_grad_(True)
+    assert not xc.is_contiguous()
+    out = ddf(xc, cf.cuda(), sf.cuda(), 3, 1, 1, 'mul')
+    go = torch.randn_like(out).to(memory_format=torch.channels_last)
+    (dx,) = torch.autograd.grad(out, xc, go)
+    want = oracle.backward(go.cpu().contiguous(), x, cf, sf, 3, 1, 1, 'mul')[0]
+    assert out.is_contiguous() and rel_err(dx, want) <= 1e-5
 
 
 def test_runs_on_the_current_stream():
