@@ -156,7 +156,9 @@ class DDFFunction(Function):
         output = features.new_empty((b, c, out_h, out_w))
         op.forward(features, channel_filter, spatial_filter,
                    kernel_size, dilation, stride, output)
-        if features.requires_grad or channel_filter.requires_grad or spatial_filter.requires_grad:
+        # (asked of ctx, not of the tensors: a dtype or layout conversion above
+        # yields new tensors that no longer carry the inputs' requires_grad)
+        if any(ctx.needs_input_grad[:3]):
             ctx.save_for_backward(features, channel_filter, spatial_filter)
         return output
 
