@@ -284,6 +284,15 @@ def test_mixed_dtypes_are_promoted():
     assert got.dtype == torch.float32
     want = oracle.forward(x.half(), cf, sf, 3, 1, 1, 'mul')
     assert rel_err(got, want) <= 1e-5
+    # ... and gradients flow back to every operand in that operand's own dtype
+    xh = x.half().cuda().requires_grad_(True)
+    cfd, sfd = cf.cuda().requires_grad_(True), sf.cuda().requires_grad_(True)
+    out = ddf(xh, cfd, sfd, 3, 1, 1, 'mul')
+    go = torch.randn_like(out)
+    dx, dcf, dsf = torch.autograd.grad(out, (xh, cfd, sfd), go)
+    assert dx.dtype == torch.float16 and dcf.dtype == torch.float32 and dsf.dtype == torch.float32
+    wx, wcf, wsf = oracle.backward(go.cpu(), x.half(), cf, sf, 3, 1, 1, 'mul')
+    assert rel_err(dx, wx) <= 1e-2 and rel_err(dcf, wcf) <= 1e-5 and rel_err(dsf, wsf) <= 1e-5
 
 
 def test_non_contiguous_inputs_are_accepted():

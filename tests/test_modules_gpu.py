@@ -85,6 +85,19 @@ def test_ddfpack_under_autocast():
     want = pack(x)
     assert torch.isfinite(out).all()
     assert (out.float() - want).abs().max() / want.abs().max() < 2e-2
+    # training step under autocast: gradients reach the input and every parameter
+    x.requires_grad_(True)
+    with torch.autocast('cuda', dtype=torch.float16):
+        loss = pack(x).float().square().mean()
+    loss.backward()
+    ref = ddfnet_amd.DDFPack(32).cuda()
+    ref.load_state_dict(pack.state_dict())
+    xr = x.detach().clone().requires_grad_(True)
+    ref(xr).square().mean().backward()
+    assert (x.grad - xr.grad).abs().max() / xr.grad.abs().max() < 5e-2
+    for (name, p_), (_, q) in zip(pack.named_parameters(), ref.named_parameters()):
+        assert p_.grad is not None, name
+        assert (p_.grad - q.grad).abs().max() / q.grad.abs().max().clamp_min(1e-12) < 5e-2, name
 
 
 def test_resnet50_forward_matches_cpu_reference(monkeypatch):
