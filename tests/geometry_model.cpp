@@ -192,5 +192,18 @@ int main() {
                         if (sh[2] / q[2] == 0 || sh[3] / q[2] == 0) continue;
                         check_geometry(kind, sh[0], sh[1], sh[2], sh[3], q[0], q[1], q[2], dtype, max_vec);
                     }
+    // seeded random shapes on top of the fixed list
+    unsigned long long state = 0x9E3779B97F4A7C15ull;
+    auto next = [&](int lo, int hi) {
+        state = state * 6364136223846793005ull + 1442695040888963407ull;
+        return lo + (int)((state >> 33) % (unsigned long long)(hi - lo + 1));
+    };
+    for (int i = 0; i < 150; ++i) {
+        const long N = next(1, 130), C = next(1, 600), H = next(1, 130), W = next(1, 330);
+        const int *q = kds[next(0, 7)];
+        if (H / q[2] == 0 || W / q[2] == 0) continue;
+        for (int kind = 0; kind < 4; ++kind)
+            check_geometry(kind, N, C, H, W, q[0], q[1], q[2], next(0, 2), next(0, 1));
+    }
     return 0;
 }

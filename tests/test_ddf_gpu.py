@@ -424,3 +424,34 @@ def test_forward_and_backward_replay_in_a_hip_graph():
         torch.cuda.synchronize()
         for g, w in zip(got, want):
             assert torch.equal(g, w)
+
+
+# ---------------------------------------------------------------------------
+# seeded random sweep over shapes and parameters
+# ---------------------------------------------------------------------------
+def _random_cases(count, seed):
+    import random
+    rng = random.Random(seed)
+    cases = []
+    while len(cases) < count:
+        k = rng.choice([1, 3, 3, 3, 5, 5, 7])
+        d = rng.choice([1, 1, 2, 3])
+        s = rng.choice([1, 1, 2, 3])
+        N, C = rng.randint(1, 4), rng.choice([1, 2, 3, 5, 8, 17, 33, 64, 70])
+        H, W = rng.randint(1, 40), rng.randint(1, 70)
+        if rng.random() < 0.3:          # the vector paths want friendly row lengths
+            W = rng.choice([8, 12, 16, 28, 32, 56, 64])
+        combine = rng.choice(['mul', 'add'])
+        dtype = rng.choice([torch.float32, torch.float32, torch.float16, torch.float64])
+        cases.append((N, C, H, W, k, d, s, combine, dtype))
+    return cases
+
+
+@pytest.mark.parametrize('chunk', range(6))
+def test_random_shapes_against_oracle(chunk):
+    """120 seeded random problems (all kernel families, ragged sizes, empty
+    outputs when the stride exceeds the image) through the default variant."""
+    for i, (N, C, H, W, k, d, s, combine, dtype) in enumerate(_random_cases(20, 1000 + chunk)):
+        case = random_case(N, C, H, W, k, s, dtype, seed=chunk * 100 + i)
+        check_against_oracle(*case, k, d, s, combine, '',
+                             what='chunk %d case %d %s' % (chunk, i, (N, C, H, W, str(dtype))))
