@@ -119,6 +119,10 @@ EDGE = [
     (1, 2, 5, 200, 5, 1, 2),    # wide and short
     (1, 2, 31, 17, 3, 2, 1),    # primes
     (1, 8, 3, 3, 3, 1, 4),      # stride larger than the window: Ho=Wo=0
+    (1, 4, 20, 300, 3, 1, 1),   # wide: several lane segments per row
+    (2, 8, 33, 224, 3, 1, 2),   # wide, strided, odd height
+    (1, 2, 5, 513, 5, 1, 1),    # wider than the tuned kernels' 8 x 64 columns
+    (1, 3, 130, 6, 3, 2, 1),    # tall and narrow
 ]
 
 
