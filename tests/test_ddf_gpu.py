@@ -279,6 +279,25 @@ def test_one_launch_backward_equals_two_launches(shape, d, combine, dtype, monke
         assert rel_err(got, w) <= TOL[dtype]
 
 
+@pytest.mark.parametrize('knob,value', [('DDF_TUNE_WPB', '2'), ('DDF_TUNE_WPB', '4'),
+                                        ('DDF_TUNE_WIDE', '0'), ('DDF_TUNE_WAVES', '512'),
+                                        ('DDF_TUNE_CPW', '3'), ('DDF_TUNE_VEC', '1')])
+def test_tuning_knobs_do_not_change_results(knob, value, monkeypatch):
+    """The launch geometry has experiment knobs (waves per workgroup, aligned
+    tile writes, wave count, channels per wave, access width).  Whatever they
+    are set to, the kernels must produce the same bits: the knobs change how
+    the work is cut, not the order of any sum."""
+    cases = [((3, 40, 14, 14), 3, 1, 1, torch.float32), ((2, 24, 28, 28), 3, 2, 1, torch.float16),
+             ((2, 16, 20, 24), 5, 1, 2, torch.float32)]
+    for (N, C, H, W), k, d, s, dtype in cases:
+        x, cf, sf, go = random_case(N, C, H, W, k, s, dtype, seed=31)
+        base = run_ddf(x, cf, sf, go, k, d, s, 'mul', need=(True, False, False))
+        monkeypatch.setenv(knob, value)
+        tuned = run_ddf(x, cf, sf, go, k, d, s, 'mul', need=(True, False, False))
+        monkeypatch.delenv(knob)
+        assert torch.equal(base[0], tuned[0]) and torch.equal(base[1], tuned[1])
+
+
 def test_mixed_dtypes_are_promoted():
     """fp16 features with fp32 filters: the reference widens the fp16 operand
     (ddf/ddf.py:37-42); result is fp32."""

@@ -34,7 +34,8 @@ def test_every_launch_geometry_stays_in_bounds(tmp_path):
     for key in list(env):
         if key.startswith('DDF_TUNE_'):
             del env[key]
-    for extra in ({}, {'DDF_TUNE_WPB': '4'}, {'DDF_TUNE_WIDE': '0'}):
+    for extra in ({}, {'DDF_TUNE_WPB': '4'}, {'DDF_TUNE_WIDE': '0'}, {'DDF_TUNE_WAVES': '512'},
+                  {'DDF_TUNE_CPW': '3', 'DDF_TUNE_CPW_FILTERS': '3'}, {'DDF_TUNE_VEC': '1'}):
         run = subprocess.run([exe], capture_output=True, text=True, timeout=600,
                              env=dict(env, **extra))
         assert run.returncode == 0
