@@ -478,3 +478,35 @@ def test_random_shapes_against_oracle(chunk):
         case = random_case(N, C, H, W, k, s, dtype, seed=chunk * 100 + i)
         check_against_oracle(*case, k, d, s, combine, '',
                              what='chunk %d case %d %s' % (chunk, i, (N, C, H, W, str(dtype))))
+
+
+def test_tensors_beyond_2_31_elements():
+    """66 x 512 x 256 x 256 fp16 is 2.2e9 elements: offsets no longer fit 32
+    bits (the reference indexes with int, ddf_mul_cuda_kernel.cu:28-33).  The
+    last sample, which lies wholly beyond 2^31, must come out exactly as when
+    it is run on its own, forward and all gradients."""
+    from ddfnet_amd import ddf
+    free, _ = torch.cuda.mem_get_info()
+    if free < 40 * 2 ** 30:
+        pytest.skip('needs about 40 GiB of device memory')
+    N, C, H, W = 66, 512, 256, 256
+    g = torch.Generator(device='cuda').manual_seed(77)
+    x = torch.randn(N, C, H, W, generator=g, device='cuda', dtype=torch.float16)
+    cf = torch.randn(N, C, 3, 3, generator=g, device='cuda', dtype=torch.float16)
+    sf = torch.randn(N, 9, H, W, generator=g, device='cuda', dtype=torch.float16)
+    assert x.numel() > 2 ** 31
+    x.requires_grad_(True); cf.requires_grad_(True); sf.requires_grad_(True)
+    out = ddf(x, cf, sf, 3, 1, 1, 'mul')
+    go = torch.randn(N, C, H, W, generator=g, device='cuda', dtype=torch.float16)
+    dx, dcf, dsf = torch.autograd.grad(out, (x, cf, sf), go)
+    n = N - 1
+    xs, cfs, sfs = (t[n:].detach().clone().requires_grad_(True) for t in (x, cf, sf))
+    outs = ddf(xs, cfs, sfs, 3, 1, 1, 'mul')
+    dxs, dcfs, dsfs = torch.autograd.grad(outs, (xs, cfs, sfs), go[n:].clone())
+    assert torch.equal(out[n:], outs) and torch.equal(dx[n:], dxs)
+    assert torch.equal(dcf[n:], dcfs) and torch.equal(dsf[n:], dsfs)
+    # and the single sample against the oracle (a few channels of it)
+    sl = slice(0, 4)
+    want = oracle.forward(xs[:, sl].detach().cpu(), cfs[:, sl].detach().cpu(), sfs.detach().cpu(),
+                          3, 1, 1, 'mul')
+    assert rel_err(outs[:, sl], want) <= TOL[torch.float16]
