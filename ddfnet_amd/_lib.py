@@ -29,6 +29,7 @@ SYMBOLS = {
     'ddf_hip_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
     'ddf_hip_filter_norm': (_i, [_vp] * 2 + [_i64] * 2 + [_i, _i64, ctypes.c_double] + [_vp] * 2 +
                             [_i, _vp]),
+    'ddf_hip_up_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 5 + [_vp]),
 }
 
 _lib = None
@@ -136,3 +137,22 @@ def filter_norm(x, outer, groups, taps, inner, gain, gain_vec=None, offset_vec=N
             _ptr(offset_vec), DTYPE[x.dtype], _stream())
     check(rc)
     return y
+
+
+def up_forward(features, channel_filters, spatial_filters, output, k, d, scale, combine):
+    """All ``scale*scale`` sub-pixel branches of an up-sampling DDF in one
+    launch; ``output`` is the pixel-shuffled (N, C, H*scale, W*scale) result.
+    Raises ``DDFHipError`` when the library does not cover (k, scale)."""
+    N, C, H, W = features.shape
+    branches = scale * scale
+    assert len(channel_filters) == branches and len(spatial_filters) == branches
+    cf = (ctypes.c_void_p * branches)(*[t.data_ptr() for t in channel_filters])
+    sf = (ctypes.c_void_p * branches)(*[t.data_ptr() for t in spatial_filters])
+    check(lib().ddf_hip_up_forward(
+        _ptr(features), cf, sf, _ptr(output), N, C, H, W, k, d, scale, COMBINE[combine],
+        DTYPE[features.dtype], _stream()))
+
+
+def up_forward_covers(k, scale):
+    """(kernel_size, scale) pairs ddf_hip_up_forward has kernels for."""
+    return (k in (1, 3) and 2 <= scale <= 4) or (k == 5 and scale == 2)

@@ -225,4 +225,44 @@ int ddf_hip_filter_norm(const void *x, void *y, int64_t outer, int64_t groups, i
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_filter_norm launch");
 }
 
+int ddf_hip_up_forward(const void *features, const void *const *channel_filters,
+                       const void *const *spatial_filters, void *output, int64_t N, int64_t C,
+                       int64_t H, int64_t W, int kernel_size, int dilation, int scale,
+                       int combine, int dtype, void *stream) {
+    int rc = check_problem(N, C, H, W, kernel_size, dilation, 1, combine, dtype, DDF_VARIANT_AUTO);
+    if (rc != DDF_OK) return rc;
+    if (scale < 2 || scale * scale > DDF_UP_MAX_BRANCHES)
+        return fail(DDF_ERR_BAD_ARG, "scale must be 2..4 (got %d)", scale);
+    if (!ddf::up_forward_supported(H, W, kernel_size, dilation, scale))
+        return fail(DDF_ERR_UNSUPPORTED,
+                    "fused up-sampling forward does not cover k=%d scale=%d H=%lld W=%lld",
+                    kernel_size, scale, (long long)H, (long long)W);
+    if (N * C * H * W == 0) return DDF_OK;
+    if (!features || !output || !channel_filters || !spatial_filters)
+        return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    for (int b = 0; b < scale * scale; ++b)
+        if (!channel_filters[b] || !spatial_filters[b])
+            return fail(DDF_ERR_BAD_ARG, "null filter pointer for branch %d", b);
+    hipStream_t st = (hipStream_t)stream;
+    const bool mul = combine == DDF_MUL;
+    hipError_t err;
+    switch (dtype) {
+        case DDF_F16:
+            err = ddf::up_forward<__half>(N, C, H, W, kernel_size, dilation, scale, mul,
+                                          (const __half *)features, channel_filters,
+                                          spatial_filters, (__half *)output, st);
+            break;
+        case DDF_F32:
+            err = ddf::up_forward<float>(N, C, H, W, kernel_size, dilation, scale, mul,
+                                         (const float *)features, channel_filters,
+                                         spatial_filters, (float *)output, st);
+            break;
+        default:
+            err = ddf::up_forward<double>(N, C, H, W, kernel_size, dilation, scale, mul,
+                                          (const double *)features, channel_filters,
+                                          spatial_filters, (double *)output, st);
+    }
+    return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_up_forward launch");
+}
+
 }  // extern "C"

@@ -63,6 +63,15 @@ template <typename T>
 hipError_t filter_norm(const T *x, T *y, int64_t outer, int64_t groups, int taps, int64_t inner,
                        double gain, const T *gain_vec, const T *offset_vec, hipStream_t st);
 
+// All scale*scale sub-pixel branches of an up-sampling DDF in one launch,
+// written into the pixel-shuffled (N, C, H*scale, W*scale) result; cf / sf are
+// host arrays of scale*scale device pointers.
+bool up_forward_supported(int64_t H, int64_t W, int k, int d, int scale);
+template <typename T>
+hipError_t up_forward(int64_t N, int64_t C, int64_t H, int64_t W, int k, int d, int scale,
+                      bool mul, const T *x, const void *const *cf, const void *const *sf, T *out,
+                      hipStream_t st);
+
 bool tiled_forward_supported(const Problem &p, int dtype);
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,

@@ -22,7 +22,7 @@ from torch.autograd import Function
 
 from . import _lib
 
-__all__ = ['DDFFunction', 'ddf', 'OP_DICT']
+__all__ = ['DDFFunction', 'ddf', 'OP_DICT', 'DDFUpFunction', 'ddf_up']
 
 
 def _require_device_contiguous(named_tensors):
@@ -181,3 +181,103 @@ class DDFFunction(Function):
 
 
 ddf = DDFFunction.apply
+
+
+class DDFUpFunction(Function):
+    """Up-sampling DDF: ``scale*scale`` filter branches on the same features,
+    result pixel-shuffled -- the loop, ``torch.stack`` and ``F.pixel_shuffle``
+    of ``DDFUpPack.forward`` (``ddf/ddf.py:264-272``) as one operator.
+
+    The forward is one launch that reads the features once and writes the
+    (N, C, H*scale, W*scale) result in place.  The backward splits the incoming
+    gradient into its ``scale*scale`` sub-pixel lattices with one copy and runs
+    the ``ddf`` backward kernels per branch; dX is their sum.
+    """
+
+    @staticmethod
+    def forward(ctx, features, kernel_size, dilation, scale, kernel_combine, *filters):
+        branches = scale * scale
+        assert len(filters) == 2 * branches, \
+            'expected {0} channel filters followed by {0} spatial filters'.format(branches)
+        assert features.is_cuda, 'input feature must be a CUDA tensor.'
+        assert kernel_combine in {'mul', 'add'}, \
+            'only support mul or add combination, instead of {}'.format(kernel_combine)
+        assert (kernel_size - 1) % 2 == 0 and kernel_size >= 1 and dilation >= 1
+        dtype = features.dtype
+        for other in filters:
+            assert other.is_cuda, 'filters must be CUDA tensors.'
+            dtype = torch.promote_types(dtype, other.dtype)
+        assert dtype in _lib.DTYPE, 'unsupported dtype {}'.format(dtype)
+        features = features.to(dtype).contiguous()
+        filters = [t.to(dtype).contiguous() for t in filters]
+        cfs, sfs = filters[:branches], filters[branches:]
+        b, c, h, w = features.size()
+        for cf in cfs:
+            assert tuple(cf.size()) == (b, c, kernel_size, kernel_size), \
+                "channel_filter size {} does not match feature size {}".format(
+                    cf.size(), features.size())
+        for sf in sfs:
+            assert tuple(sf.size()) == (b, kernel_size ** 2, h, w), \
+                "spatial_filter size {} does not match feature size {}".format(
+                    sf.size(), features.size())
+        ctx.kernel_size, ctx.dilation, ctx.scale = kernel_size, dilation, scale
+        ctx.op_type = kernel_combine
+
+        output = features.new_empty((b, c, h * scale, w * scale))
+        with _lib.on_device_of(features):
+            _lib.up_forward(features, cfs, sfs, output, kernel_size, dilation, scale,
+                            kernel_combine)
+        if any(ctx.needs_input_grad):
+            ctx.save_for_backward(features, *filters)
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        saved = ctx.saved_tensors
+        features, filters = saved[0], saved[1:]
+        r, k = ctx.scale, ctx.kernel_size
+        branches = r * r
+        b, c, h, w = features.size()
+        # (b, c, h, r, w, r) -> (r, r, b, c, h, w): lattice (i, j) becomes contiguous
+        lattices = grad_output.to(features.dtype).reshape(b, c, h, r, w, r) \
+            .permute(3, 5, 0, 1, 2, 4).contiguous()
+        want_x = ctx.needs_input_grad[0]
+        want_f = ctx.needs_input_grad[5:]
+        op = OP_DICT[ctx.op_type]
+        grad_x = None
+        grad_filters = [None] * (2 * branches)
+        for br in range(branches):
+            want_cf, want_sf = want_f[br], want_f[branches + br]
+            if not (want_x or want_cf or want_sf):
+                continue
+            cf, sf = filters[br], filters[branches + br]
+            dx = torch.empty_like(features) if want_x else None
+            dcf = torch.empty_like(cf) if want_cf else None
+            dsf = torch.empty_like(sf) if want_sf else None
+            op.backward(lattices[br // r, br % r], features, cf, sf, k, ctx.dilation, 1,
+                        None, None, None, dx, dcf, dsf)
+            grad_filters[br], grad_filters[branches + br] = dcf, dsf
+            if want_x:
+                grad_x = dx if grad_x is None else grad_x.add_(dx)
+        return (grad_x, None, None, None, None) + tuple(grad_filters)
+
+
+def ddf_up(features, channel_filters, spatial_filters, kernel_size=3, dilation=1,
+           scale_factor=2, kernel_combine='mul'):
+    """``pixel_shuffle`` of the ``scale_factor**2`` results ``ddf(features,
+    channel_filters[b], spatial_filters[b], kernel_size, dilation, 1,
+    kernel_combine)``, branch ``b`` going to sub-pixel ``divmod(b, scale_factor)``.
+
+    One fused launch where the library has a kernel for (kernel_size,
+    scale_factor); otherwise the reference's composition (``ddf/ddf.py:264-272``)
+    on the ``ddf`` kernels."""
+    channel_filters, spatial_filters = tuple(channel_filters), tuple(spatial_filters)
+    assert len(channel_filters) == len(spatial_filters) == scale_factor ** 2
+    if _lib.up_forward_covers(kernel_size, scale_factor):
+        return DDFUpFunction.apply(features, kernel_size, dilation, scale_factor, kernel_combine,
+                                   *(channel_filters + spatial_filters))
+    outs = [ddf(features, cf, sf, kernel_size, dilation, 1, kernel_combine)
+            for cf, sf in zip(channel_filters, spatial_filters)]
+    b, c, h, w = outs[0].shape
+    return torch.nn.functional.pixel_shuffle(torch.stack(outs, dim=2).reshape(b, -1, h, w),
+                                             scale_factor)

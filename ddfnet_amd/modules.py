@@ -12,7 +12,7 @@ import torch.nn.functional as F
 from torch.nn.init import calculate_gain
 
 from . import _lib
-from .functional import ddf
+from .functional import ddf, ddf_up
 
 __all__ = ['FilterNorm', 'build_spatial_branch', 'build_channel_branch',
            'DDFPack', 'DDFUpPack']
@@ -205,13 +205,10 @@ class DDFUpPack(nn.Module):
             joint_x = x
         b, c, h, w = x.shape
         g, k = self.head, self.kernel_size
+        r = self.scale_factor
         grouped = x.reshape(b * g, c // g, h, w)
-        subpixels = []
-        for spatial, channel in zip(self.spatial_branch, self.channel_branch):
-            cf = channel(x).reshape(b * g, c // g, k, k)
-            sf = spatial(joint_x).reshape(b * g, k * k, h, w)
-            o = ddf(grouped, cf, sf, k, self.dilation, 1, self.kernel_combine)
-            subpixels.append(o.type_as(x).reshape(b, c, h, w))
-        # (b, c, r*r, h, w) -> (b, c*r*r, h, w) -> pixel shuffle
-        out = torch.stack(subpixels, dim=2).reshape(b, -1, h, w)
-        return F.pixel_shuffle(out, self.scale_factor)
+        cfs = [channel(x).reshape(b * g, c // g, k, k) for channel in self.channel_branch]
+        sfs = [spatial(joint_x).reshape(b * g, k * k, h, w) for spatial in self.spatial_branch]
+        # all r*r branches, the stack and the pixel shuffle as one operator
+        out = ddf_up(grouped, cfs, sfs, k, self.dilation, r, self.kernel_combine)
+        return out.type_as(x).reshape(b, c, h * r, w * r)

@@ -142,6 +142,29 @@ int ddf_hip_filter_norm(const void *x, void *y, int64_t outer, int64_t groups,
                         const void *gain_vec, const void *offset_vec,
                         int dtype, void *stream);
 
+/*
+ * Up-sampling DDF forward (DDFUpPack.forward, ddf/ddf.py:257-272): the
+ * reference calls `ddf` once per sub-pixel branch b = 0 .. scale*scale-1 on
+ * the same features with that branch's filters (ddf.py:264-269), stacks the
+ * results and pixel-shuffles them (ddf.py:270-272).  This entry point does all
+ * of it in one launch:
+ *   output[n, c, y*scale + i, x*scale + j] =
+ *       ddf(features, channel_filters[i*scale + j], spatial_filters[i*scale + j],
+ *           kernel_size, dilation, stride 1, combine)[n, c, y, x]
+ * `channel_filters` and `spatial_filters` are host arrays of scale*scale device
+ * pointers, each a dense (N, C, k, k) resp. (N, k*k, H, W) tensor; `output`
+ * is dense (N, C, H*scale, W*scale).  Covered: k = 1 or 3 with scale 2..4 and
+ * k = 5 with scale 2; anything else returns DDF_ERR_UNSUPPORTED and the caller
+ * composes the result from ddf_hip_forward.  Forward only.
+ */
+#define DDF_UP_MAX_BRANCHES 16
+int ddf_hip_up_forward(const void *features,
+                       const void *const *channel_filters,
+                       const void *const *spatial_filters, void *output,
+                       int64_t N, int64_t C, int64_t H, int64_t W,
+                       int kernel_size, int dilation, int scale, int combine,
+                       int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,6 +18,10 @@ pin one another:
     ``ddf_oracle.c`` (plain C gather loops, fp64) through ctypes; fast enough
     for the full benchmark shapes.  ``*_f32`` variants are the timed CPU
     baseline.
+``up_forward`` / ``up_backward``
+    The up-sampling composition of ``DDFUpPack.forward``: ``forward`` per
+    sub-pixel branch, interleaved as ``F.pixel_shuffle`` would; pinned against
+    ``torch.stack`` + ``F.pixel_shuffle`` of the unfold form and its autograd.
 
 Parity status: every function here is pinned by ``tests/test_oracle.py``
 (closed forms against ``F.conv2d`` / pointwise / shift, mutual agreement of
@@ -177,6 +181,33 @@ def unfold_backward(go, x, cf, sf, k=3, d=1, s=1, combine='mul'):
     x, cf, sf = (t.detach().clone().requires_grad_(True) for t in (x, cf, sf))
     out = unfold_forward(x, cf, sf, k, d, s, combine)
     return torch.autograd.grad(out, (x, cf, sf), go)
+
+
+def up_forward(x, cfs, sfs, k=3, d=1, scale=2, combine='mul'):
+    """Up-sampling DDF as ``DDFUpPack.forward`` composes it
+    (``ddf/ddf.py:264-272``): one stride-1 ``forward`` per sub-pixel branch
+    ``b = i*scale + j``, whose result lands on the pixels ``(y*scale + i,
+    x*scale + j)`` -- what ``torch.stack(outs, 2)`` + ``F.pixel_shuffle`` do."""
+    N, C, H, W = x.shape
+    out = torch.zeros(N, C, H * scale, W * scale, dtype=torch.float64)
+    for b, (cf, sf) in enumerate(zip(cfs, sfs)):
+        i, j = divmod(b, scale)
+        out[:, :, i::scale, j::scale] = forward(x, cf, sf, k, d, 1, combine)
+    return out
+
+
+def up_backward(go, x, cfs, sfs, k=3, d=1, scale=2, combine='mul'):
+    """Gradients of ``up_forward``: ``(dX, [dCF_b], [dSF_b])``.  Branch ``b``
+    sees the gradient of its own sub-pixel lattice; dX sums over branches."""
+    dx, dcfs, dsfs = 0, [], []
+    for b, (cf, sf) in enumerate(zip(cfs, sfs)):
+        i, j = divmod(b, scale)
+        g = go[:, :, i::scale, j::scale].contiguous()
+        dxb, dcf, dsf = backward(g, x, cf, sf, k, d, 1, combine)
+        dx = dx + dxb
+        dcfs.append(dcf)
+        dsfs.append(dsf)
+    return dx, dcfs, dsfs
 
 
 def filter_standardize(f, dim):

@@ -180,6 +180,22 @@ def test_filter_norm_argument_validation_needs_no_gpu():
     assert b'null' in lib.ddf_hip_last_error()
 
 
+def test_up_forward_argument_validation_needs_no_gpu():
+    import ctypes
+    lib = _lib.lib()
+    none = (ctypes.c_void_p * 16)()
+    up = lib.ddf_hip_up_forward
+    assert up(None, none, none, None, 1, 1, 4, 4, 3, 1, 1, 0, 1, None) == 1     # scale 1
+    assert b'scale' in lib.ddf_hip_last_error()
+    assert up(None, none, none, None, 1, 1, 4, 4, 3, 1, 5, 0, 1, None) == 1     # 25 branches
+    assert up(None, none, none, None, 1, 1, 4, 4, 2, 1, 2, 0, 1, None) == 1     # even k
+    assert up(None, none, none, None, 1, 1, 4, 4, 7, 1, 2, 0, 1, None) == 2     # no fused kernel
+    assert up(None, none, none, None, 0, 8, 4, 4, 3, 1, 2, 0, 1, None) == 0     # empty
+    assert up(None, none, none, None, 1, 1, 4, 4, 3, 1, 2, 0, 1, None) == 1
+    assert b'null' in lib.ddf_hip_last_error()
+    assert _lib.up_forward_covers(3, 2) and not _lib.up_forward_covers(7, 2)
+
+
 def _load_bench():
     import importlib.util
     spec = importlib.util.spec_from_file_location('ddf_bench', os.path.join(ROOT, 'bench.py'))

@@ -20,9 +20,17 @@ class _OracleOp(object):
         return oracle.unfold_forward(x, cf, sf, k, d, s, combine)
 
 
+def _oracle_up(x, cfs, sfs, k=3, d=1, scale=2, combine='mul'):
+    """``ddf_up`` replacement: the reference's composition (ddf/ddf.py:264-272)."""
+    outs = [oracle.unfold_forward(x, cf, sf, k, d, 1, combine) for cf, sf in zip(cfs, sfs)]
+    b, c, h, w = outs[0].shape
+    return torch.nn.functional.pixel_shuffle(torch.stack(outs, dim=2).reshape(b, -1, h, w), scale)
+
+
 def cpu_reference(module, monkeypatch, *inputs):
     ref = copy.deepcopy(module).cpu().double()
     monkeypatch.setattr(ddf_modules, 'ddf', _OracleOp())
+    monkeypatch.setattr(ddf_modules, 'ddf_up', _oracle_up)
     ins = [t.detach().cpu().double().requires_grad_(True) for t in inputs]
     out = ref(*ins)
     monkeypatch.undo()
@@ -56,6 +64,29 @@ def test_ddfuppack_matches_cpu_reference(monkeypatch):
     assert out.shape == (2, 8, 20, 20)
     _, _, out_r = cpu_reference(up, monkeypatch, x)
     assert torch.allclose(out.detach().cpu().double(), out_r.detach(), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize('k,scale,head,combine', [(3, 2, 2, 'add'), (3, 3, 1, 'mul'), (5, 2, 1, 'mul'),
+                                                  (3, 4, 1, 'mul'), (7, 2, 1, 'mul')])
+def test_ddfuppack_trains_like_cpu_reference(k, scale, head, combine, monkeypatch):
+    """Forward, input gradient and every parameter gradient of the up-sampling
+    pack; (7, 2) has no fused kernel and takes the composed route."""
+    torch.manual_seed(3)
+    # the guidance convolution pads by kernel_size // 2 (ddf/ddf.py:244-245), so
+    # it keeps the plane size only when it is kernel_size wide
+    up = ddfnet_amd.DDFUpPack(8, kernel_size=k, scale_factor=scale, head=head,
+                              dw_kernel_size=k, kernel_combine=combine).cuda()
+    x = torch.randn(2, 8, 9, 7, device='cuda', requires_grad=True)
+    out = up(x)
+    assert out.shape == (2, 8, 9 * scale, 7 * scale)
+    go = torch.randn_like(out)
+    out.backward(go)
+    ref, (xr,), out_r = cpu_reference(up, monkeypatch, x)
+    out_r.backward(go.cpu().double())
+    assert torch.allclose(out.detach().cpu().double(), out_r.detach(), rtol=1e-4, atol=1e-5)
+    assert torch.allclose(x.grad.cpu().double(), xr.grad, rtol=1e-3, atol=1e-4)
+    for (name, p), (_, pr) in zip(up.named_parameters(), ref.named_parameters()):
+        assert torch.allclose(p.grad.cpu().double(), pr.grad, rtol=1e-3, atol=1e-4), name
 
 
 def test_ddfuppack_with_joint_guidance(monkeypatch):

@@ -220,3 +220,61 @@ def test_c_oracle_reproduces_golden_fixtures(path):
     for got, name in zip((out32,) + tuple(g32), ('out', 'dx', 'dcf', 'dsf')):
         scale = max(t[name].abs().max().item(), 1e-30)
         assert (got.double() - t[name]).abs().max().item() / scale < 1e-5, name
+
+
+# ---------------------------------------------------------------------------
+# up-sampling composition (DDFUpPack.forward, ddf/ddf.py:264-272)
+# ---------------------------------------------------------------------------
+def _up_inputs(N, C, H, W, k, scale, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(N, C, H, W, generator=g, dtype=torch.float64)
+    cfs = [torch.randn(N, C, k, k, generator=g, dtype=torch.float64) for _ in range(scale ** 2)]
+    sfs = [torch.randn(N, k * k, H, W, generator=g, dtype=torch.float64) for _ in range(scale ** 2)]
+    go = torch.randn(N, C, H * scale, W * scale, generator=g, dtype=torch.float64)
+    return x, cfs, sfs, go
+
+
+def _stack_and_shuffle(x, cfs, sfs, k, d, scale, combine):
+    """The reference's expression, on the differentiable unfold form."""
+    outs = [oracle.unfold_forward(x, cf, sf, k, d, 1, combine) for cf, sf in zip(cfs, sfs)]
+    b, c, h, w = outs[0].shape
+    return F.pixel_shuffle(torch.stack(outs, dim=2).reshape(b, -1, h, w), scale)
+
+
+@pytest.mark.parametrize('k,d,scale,combine', [(3, 1, 2, 'mul'), (3, 2, 3, 'add'), (5, 1, 2, 'mul'),
+                                               (1, 1, 4, 'add')])
+def test_up_forward_is_stack_plus_pixel_shuffle(k, d, scale, combine):
+    x, cfs, sfs, _ = _up_inputs(2, 3, 5, 4, k, scale, seed=k + scale)
+    got = oracle.up_forward(x, cfs, sfs, k, d, scale, combine)
+    want = _stack_and_shuffle(x, cfs, sfs, k, d, scale, combine)
+    assert torch.allclose(got, want, atol=1e-12)
+
+
+def test_up_forward_places_each_branch_on_its_own_lattice():
+    """With identity taps and unit spatial filters branch b returns b+1 times
+    the features; the result must hold (i*scale + j + 1) * x on lattice (i, j)."""
+    x = torch.arange(1., 13.).view(1, 1, 3, 4).double()
+    cfs = []
+    for b in range(4):
+        cf = torch.zeros(1, 1, 3, 3, dtype=torch.float64)
+        cf[0, 0, 1, 1] = b + 1
+        cfs.append(cf)
+    sfs = [torch.ones(1, 9, 3, 4, dtype=torch.float64) for _ in range(4)]
+    out = oracle.up_forward(x, cfs, sfs, 3, 1, 2, 'mul')
+    for i in range(2):
+        for j in range(2):
+            assert torch.equal(out[0, 0, i::2, j::2], (i * 2 + j + 1) * x[0, 0])
+
+
+@pytest.mark.parametrize('k,d,scale,combine', [(3, 1, 2, 'mul'), (3, 2, 2, 'add'), (1, 1, 3, 'mul')])
+def test_up_backward_is_autograd_of_the_composition(k, d, scale, combine):
+    x, cfs, sfs, go = _up_inputs(2, 3, 4, 5, k, scale, seed=7)
+    leaves = [t.clone().requires_grad_(True) for t in [x] + cfs + sfs]
+    n = scale ** 2
+    out = _stack_and_shuffle(leaves[0], leaves[1:1 + n], leaves[1 + n:], k, d, scale, combine)
+    want = torch.autograd.grad(out, leaves, go)
+    dx, dcfs, dsfs = oracle.up_backward(go, x, cfs, sfs, k, d, scale, combine)
+    assert torch.allclose(dx, want[0], atol=1e-11)
+    for b in range(n):
+        assert torch.allclose(dcfs[b], want[1 + b], atol=1e-11)
+        assert torch.allclose(dsfs[b], want[1 + n + b], atol=1e-11)

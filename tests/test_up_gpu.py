@@ -1,0 +1,149 @@
+"""The fused up-sampling operator (``ddf_up`` / ``ddf_hip_up_forward``) against
+the oracle's composition of per-branch forwards and a pixel shuffle."""
+import ctypes
+
+import pytest
+import torch
+
+import oracle
+import ddfnet_amd
+from ddfnet_amd import _lib, ddf, ddf_up
+from ddf_testlib import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def up_case(N, C, H, W, k, scale, dtype, seed=0):
+    """CPU tensors already rounded to ``dtype``: x, [cf_b], [sf_b], go."""
+    g = torch.Generator(device='cpu').manual_seed(seed)
+    base = torch.float64 if dtype == torch.float64 else torch.float32
+    x = torch.randn(N, C, H, W, generator=g, dtype=base).to(dtype)
+    cfs = [torch.randn(N, C, k, k, generator=g, dtype=base).to(dtype) for _ in range(scale ** 2)]
+    sfs = [torch.randn(N, k * k, H, W, generator=g, dtype=base).to(dtype)
+           for _ in range(scale ** 2)]
+    go = torch.randn(N, C, H * scale, W * scale, generator=g, dtype=base).to(dtype)
+    return x, cfs, sfs, go
+
+
+def check_up(N, C, H, W, k, d, scale, combine, dtype, backward=True, seed=0):
+    x, cfs, sfs, go = up_case(N, C, H, W, k, scale, dtype, seed)
+    xd = x.cuda().requires_grad_(backward)
+    cfd = [t.cuda().requires_grad_(backward) for t in cfs]
+    sfd = [t.cuda().requires_grad_(backward) for t in sfs]
+    out = ddf_up(xd, cfd, sfd, k, d, scale, combine)
+    assert out.dtype == dtype and out.shape == (N, C, H * scale, W * scale)
+    tol = TOL[dtype]
+    errs = {'out': rel_err(out, oracle.up_forward(x, cfs, sfs, k, d, scale, combine))}
+    if backward:
+        grads = torch.autograd.grad(out, [xd] + cfd + sfd, go.cuda())
+        want_x, want_cf, want_sf = oracle.up_backward(go, x, cfs, sfs, k, d, scale, combine)
+        errs['dX'] = rel_err(grads[0], want_x)
+        for b in range(scale ** 2):
+            errs['dCF%d' % b] = rel_err(grads[1 + b], want_cf[b])
+            errs['dSF%d' % b] = rel_err(grads[1 + scale ** 2 + b], want_sf[b])
+    bad = {n: e for n, e in errs.items() if not e <= tol}
+    assert not bad, (dict(N=N, C=C, H=H, W=W, k=k, d=d, scale=scale, combine=combine), errs)
+
+
+@pytest.mark.parametrize('dtype', [torch.float64, torch.float32, torch.float16])
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('k,scale', [(1, 2), (1, 3), (1, 4), (3, 2), (3, 3), (3, 4), (5, 2)])
+def test_every_fused_kernel(k, scale, combine, dtype):
+    """Odd plane (not a multiple of the block), odd channel count."""
+    check_up(2, 5, 9, 13, k, 1, scale, combine, dtype)
+
+
+@pytest.mark.parametrize('d', [2, 3])
+@pytest.mark.parametrize('k,scale', [(3, 2), (5, 2), (3, 3)])
+def test_dilation(k, scale, d):
+    check_up(1, 4, 11, 10, k, d, scale, 'mul', torch.float32)
+
+
+@pytest.mark.parametrize('N,C,H,W', [
+    (1, 70, 40, 36),    # channels split over blocks and staged in two rounds
+    (3, 33, 17, 16),    # last chunk shorter than the others
+    (1, 1, 1, 1), (1, 2, 1, 300), (1, 2, 300, 1),
+    (4, 8, 16, 16),     # block count a multiple of 8: renumbered across XCDs
+    (1, 200, 8, 8),     # many stages in one block
+])
+def test_shapes(N, C, H, W):
+    check_up(N, C, H, W, 3, 1, 2, 'mul', torch.float32)
+
+
+def test_empty_tensors():
+    for shape in ((0, 4, 5, 5), (2, 0, 5, 5), (2, 4, 0, 5)):
+        N, C, H, W = shape
+        x = torch.zeros(shape, device='cuda')
+        cfs = [torch.zeros(N, C, 3, 3, device='cuda') for _ in range(4)]
+        sfs = [torch.zeros(N, 9, H, W, device='cuda') for _ in range(4)]
+        assert ddf_up(x, cfs, sfs, 3, 1, 2).shape == (N, C, 2 * H, 2 * W)
+
+
+def test_unsupported_pair_composes_from_ddf():
+    """(k, scale) = (7, 2) and (5, 3) have no fused kernel."""
+    lib = _lib.lib()
+    x = torch.zeros(1, 1, 4, 4, device='cuda')
+    ptrs = (ctypes.c_void_p * 16)(*([x.data_ptr()] * 16))
+    rc = lib.ddf_hip_up_forward(x.data_ptr(), ptrs, ptrs, x.data_ptr(), 1, 1, 4, 4, 7, 1, 2, 0, 1,
+                                None)
+    assert rc == 2 and b'does not cover' in lib.ddf_hip_last_error()
+    check_up(2, 6, 10, 9, 7, 1, 2, 'mul', torch.float32)
+    check_up(1, 4, 8, 9, 5, 1, 3, 'add', torch.float32)
+
+
+def test_misaligned_output_takes_scalar_stores():
+    x, cfs, sfs, _ = up_case(2, 6, 7, 9, 3, 2, torch.float32, seed=5)
+    xd, cfd, sfd = x.cuda(), [t.cuda() for t in cfs], [t.cuda() for t in sfs]
+    n = 2 * 6 * 14 * 18
+    buf = torch.full((n + 2,), 7.0, device='cuda')
+    out = buf[1:1 + n].view(2, 6, 14, 18)
+    assert out.data_ptr() % 8 == 4
+    _lib.up_forward(xd, cfd, sfd, out, 3, 1, 2, 'mul')
+    torch.cuda.synchronize()
+    assert rel_err(out, oracle.up_forward(x, cfs, sfs, 3, 1, 2, 'mul')) <= 1e-5
+    assert buf[0].item() == 7.0 and buf[-1].item() == 7.0    # nothing outside the result
+
+
+def test_mixed_dtypes_and_partial_gradients():
+    """fp16 features with fp32 filters promote to fp32; only the gradients
+    asked for come back."""
+    x, cfs, sfs, go = up_case(1, 4, 6, 6, 3, 2, torch.float32, seed=2)
+    xd = x.half().cuda()
+    cfd = [t.cuda() for t in cfs]
+    sfd = [t.cuda().requires_grad_(b == 1) for b, t in enumerate(sfs)]
+    out = ddf_up(xd, cfd, sfd, 3, 1, 2, 'mul')
+    assert out.dtype == torch.float32
+    (g,) = torch.autograd.grad(out, [sfd[1]], go.cuda())
+    _, _, want_sf = oracle.up_backward(go, x.half().float(), cfs, sfs, 3, 1, 2, 'mul')
+    assert rel_err(g, want_sf[1]) <= 1e-5
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+def test_full_size_equals_composition_of_ddf(dtype):
+    """At a size the CPU oracle would take long for: the fused launch against
+    ``ddf`` per branch + ``pixel_shuffle`` (kernels that the parity tests of the
+    operator cover), and linearity in the features."""
+    N, C, H, W, k, scale = 4, 64, 96, 96, 3, 2
+    g = torch.Generator(device='cuda').manual_seed(0)
+    x = torch.randn(N, C, H, W, device='cuda', generator=g).to(dtype)
+    cfs = [torch.randn(N, C, k, k, device='cuda', generator=g).to(dtype) / 3 for _ in range(4)]
+    sfs = [torch.randn(N, k * k, H, W, device='cuda', generator=g).to(dtype) for _ in range(4)]
+    out = ddf_up(x, cfs, sfs, k, 1, scale, 'mul')
+    outs = [ddf(x, cf, sf, k, 1, 1, 'mul') for cf, sf in zip(cfs, sfs)]
+    want = torch.nn.functional.pixel_shuffle(torch.stack(outs, 2).reshape(N, -1, H, W), scale)
+    tol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert rel_err(out, want.cpu()) <= tol
+    if dtype == torch.float32:
+        x2 = torch.randn(N, C, H, W, device='cuda', generator=g)
+        both = ddf_up(x + 2 * x2, cfs, sfs, k, 1, scale, 'mul')
+        assert rel_err(both, (out + 2 * ddf_up(x2, cfs, sfs, k, 1, scale, 'mul')).cpu()) <= 1e-5
+
+
+def test_ddfuppack_uses_the_fused_operator(monkeypatch):
+    calls = []
+    real = _lib.up_forward
+    monkeypatch.setattr(_lib, 'up_forward', lambda *a: (calls.append(1), real(*a))[1])
+    up = ddfnet_amd.DDFUpPack(8, scale_factor=2).cuda()
+    with torch.no_grad():
+        up(torch.randn(1, 8, 6, 6, device='cuda'))
+    assert calls == [1]
