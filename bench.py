@@ -331,6 +331,55 @@ def test_time_table(iters=20, warmup=5):
     return rows
 
 
+def up_forward_table(lib, iters=50, warmup=10):
+    """The up-sampling operator of DDFUpPack (ddf/ddf.py:264-272), forward only:
+    one fused launch against the reference's composition (one ddf call per
+    sub-pixel branch, torch.stack, F.pixel_shuffle).  Algorithmic bytes: the
+    features once, every branch's two filters once, the up-sampled result once."""
+    import torch.nn.functional as F
+    from ddfnet_amd import ddf
+    cases = [(8, 64, 64, 64, 3, 2, torch.float32), (8, 64, 64, 64, 3, 2, torch.float16),
+             (4, 64, 128, 128, 3, 2, torch.float32), (16, 128, 32, 32, 3, 2, torch.float32),
+             (8, 64, 64, 64, 3, 3, torch.float32), (8, 64, 64, 64, 5, 2, torch.float32)]
+    rows = []
+    with torch.no_grad():
+        for n, c, h, w, k, r, dtype in cases:
+            x = torch.randn(n, c, h, w, device='cuda').to(dtype)
+            cfs = [torch.randn(n, c, k, k, device='cuda').to(dtype) for _ in range(r * r)]
+            sfs = [torch.randn(n, k * k, h, w, device='cuda').to(dtype) for _ in range(r * r)]
+
+            def composed():
+                outs = [ddf(x, cf, sf, k, 1, 1, 'mul') for cf, sf in zip(cfs, sfs)]
+                return F.pixel_shuffle(torch.stack(outs, dim=2).reshape(n, -1, h, w), r)
+
+            out = torch.empty(n, c, h * r, w * r, device='cuda', dtype=dtype)
+            cf_ptrs = (ctypes.c_void_p * (r * r))(*[t.data_ptr() for t in cfs])
+            sf_ptrs = (ctypes.c_void_p * (r * r))(*[t.data_ptr() for t in sfs])
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            entry = lib.lib().ddf_hip_up_forward
+
+            def fused():   # the C entry point, as the other figures of this file
+                rc = entry(x.data_ptr(), cf_ptrs, sf_ptrs, out.data_ptr(), n, c, h, w, k, 1, r,
+                           0, lib.DTYPE[dtype], stream)
+                assert rc == 0
+
+            esz = x.element_size()
+            nbytes = esz * (x.numel() * (1 + r * r) + sum(t.numel() for t in cfs + sfs))
+            row = {'shape': [n, c, h, w], 'k': k, 'scale': r, 'dtype': DTYPE_NAME[dtype],
+                   'bytes': nbytes}
+            for name, fn in (('fused', fused), ('composed', composed)):
+                for _ in range(warmup):
+                    fn()
+                row[name + '_us'] = round(timed(lambda i: fn(), iters) * 1e3, 2)
+            row['fused_gbps'] = round(nbytes / (row['fused_us'] * 1e-6) / 1e9, 1)
+            row['speedup'] = round(row['composed_us'] / row['fused_us'], 2)
+            rows.append(row)
+            log('[up] %s k%d x%d %s: fused %.1f us (%.0f GB/s, %.1f%% of HBM peak)  composed %.1f us  x%.2f' % (
+                row['shape'], k, r, row['dtype'], row['fused_us'], row['fused_gbps'],
+                100 * row['fused_gbps'] / HBM_PEAK_GBPS, row['composed_us'], row['speedup']))
+    return rows
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -342,6 +391,8 @@ def main():
     ap.add_argument('--test-time', action='store_true',
                     help="also run the reference's micro-benchmark table (conv, depthwise conv, "
                          "DDFPack, ddf at seven 256-channel shapes)")
+    ap.add_argument('--up-pack', action='store_true',
+                    help='also time the fused up-sampling forward against its composition')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--copy-probe', action='store_true',
                     help='also run a plain 256 MiB device copy (calibrates hardware counters)')
@@ -400,6 +451,8 @@ def main():
             mi['ddf_ms_per_batch']))
     if args.test_time:
         line['test_time'] = test_time_table()
+    if args.up_pack:
+        line['up_forward'] = up_forward_table(lib)
     if not args.no_cpu:
         line['cpu_baseline'] = cpu_baseline(args.workload)
         cb = line['cpu_baseline']

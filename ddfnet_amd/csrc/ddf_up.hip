@@ -48,6 +48,7 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
     int cpb, int csplit, int pblocks, int stage, int vec_ok) {
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RR = R * R, RAD = K / 2;
+    constexpr int U = KK <= 9 ? 4 : 2;              // channels whose loads are issued together
     extern __shared__ __align__(16) unsigned char up_smem[];
     A *taps = reinterpret_cast<A *>(up_smem);   // [channel][branch][tap]
 
@@ -84,6 +85,7 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
         }
 
     const int64_t orow = (int64_t)W * R;            // elements per result row
+    const int64_t ostep = (int64_t)H * R * orow;    // and per result plane
     const T *xp = x + (n * C + c0) * plane + pix;
     T *op = out + ((n * C + c0) * H + y) * R * orow + (int64_t)xx * R;
     for (int s0 = 0; s0 < nch; s0 += stage) {
@@ -100,29 +102,39 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
         }
         __syncthreads();
         if (!live) continue;
-        for (int ch = 0; ch < ns; ++ch, xp += plane, op += (int64_t)H * R * orow) {
-            A xv[KK];
+        // U channels at a time: all their loads are issued before the first
+        // result is needed, so a wave keeps U*K*K loads in flight
+        for (int ch = 0; ch < ns; ch += U, xp += (int64_t)U * plane, op += U * ostep) {
+            A xv[U][KK];
 #pragma unroll
-            for (int t = 0; t < KK; ++t) xv[t] = inside[t] ? (A)ld(xp + off[t]) : (A)0;
-            const A *w = taps + ch * RR * KK;
+            for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                Row<T, R> row;
+                for (int t = 0; t < KK; ++t)
+                    xv[u][t] = (ch + u < ns && inside[t]) ? (A)ld(xp + (int64_t)u * plane + off[t])
+                                                          : (A)0;
 #pragma unroll
-                for (int j = 0; j < R; ++j) {
-                    const int b = i * R + j;
-                    A acc = 0;
+            for (int u = 0; u < U; ++u) {
+                if (ch + u >= ns) break;
+                const A *w = taps + (ch + u) * RR * KK;
 #pragma unroll
-                    for (int t = 0; t < KK; ++t)
-                        acc += xv[t] * comb<MUL, A>(w[b * KK + t], sfr[b][t]);
-                    st(&row.e[j], acc);
-                }
-                T *dst = op + i * orow;
-                if ((R == 2 || R == 4) && vec_ok) {
-                    *reinterpret_cast<Row<T, R> *>(dst) = row;
-                } else {
+                for (int i = 0; i < R; ++i) {
+                    Row<T, R> row;
 #pragma unroll
-                    for (int j = 0; j < R; ++j) dst[j] = row.e[j];
+                    for (int j = 0; j < R; ++j) {
+                        const int b = i * R + j;
+                        A acc = 0;
+#pragma unroll
+                        for (int t = 0; t < KK; ++t)
+                            acc += xv[u][t] * comb<MUL, A>(w[b * KK + t], sfr[b][t]);
+                        st(&row.e[j], acc);
+                    }
+                    T *dst = op + u * ostep + i * orow;
+                    if ((R == 2 || R == 4) && vec_ok) {
+                        *reinterpret_cast<Row<T, R> *>(dst) = row;
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < R; ++j) dst[j] = row.e[j];
+                    }
                 }
             }
         }
