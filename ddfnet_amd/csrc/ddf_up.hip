@@ -13,6 +13,8 @@
 // taps of the block's chunk sit in LDS in accumulator precision and are read
 // with wave-uniform (broadcast) addresses.
 #include <algorithm>
+#include <atomic>
+#include <cstdlib>
 
 #include "ddf_common.h"
 
@@ -34,12 +36,73 @@ struct alignas((R & (R - 1)) == 0 ? sizeof(T) * R : sizeof(T)) Row {
     T e[R];
 };
 
+// Register image of one result row, so that it leaves as a single store.
+template <int BYTES> struct RowBits;
+template <> struct RowBits<4> { using type = uint32_t; };
+template <> struct RowBits<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct RowBits<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+template <> struct RowBits<32> { typedef uint32_t type __attribute__((ext_vector_type(8))); };
+
 // Workgroups reach the 8 XCDs round-robin; renumber so that consecutive
 // logical blocks (same sample and pixel block, neighbouring channel chunks,
 // hence the same spatial taps) run on one XCD and share its L2.
 __device__ __forceinline__ unsigned xcd_order(unsigned bid, unsigned nblocks) {
     if (nblocks % 8u != 0) return bid;
     return (bid % 8u) * (nblocks / 8u) + bid / 8u;
+}
+
+// UU channels of one pixel: every load is issued before the first result is
+// needed (a wave keeps UU*K*K loads in flight), then R rows of R results per
+// channel are formed and stored.  A neighbour outside the plane reads the
+// pixel itself (offset 0, always valid) and is zeroed afterwards, so there is
+// no branch between the loads.
+template <typename T, int K, int R, bool MUL, int UU, typename A>
+__device__ __forceinline__ void up_channels(const T *__restrict__ xp, T *__restrict__ op,
+                                            const A *__restrict__ w, int plane, int64_t orow,
+                                            int64_t ostep, const int (&off)[K * K],
+                                            const bool (&inside)[K * K],
+                                            const A (&sfr)[R * R][K * K], int vec_ok) {
+    constexpr int KK = K * K, RR = R * R;
+    A xv[UU][KK];
+#pragma unroll
+    for (int u = 0; u < UU; ++u)
+#pragma unroll
+        for (int t = 0; t < KK; ++t) xv[u][t] = (A)ld(xp + (int64_t)u * plane + off[t]);
+#pragma unroll
+    for (int u = 0; u < UU; ++u)
+#pragma unroll
+        for (int t = 0; t < KK; ++t)
+            if (!inside[t]) xv[u][t] = (A)0;
+#pragma unroll
+    for (int u = 0; u < UU; ++u) {
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            Row<T, R> row;
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                const int b = i * R + j;
+                A acc = 0;
+#pragma unroll
+                for (int t = 0; t < KK; ++t)
+                    acc += xv[u][t] * comb<MUL, A>(w[(u * RR + b) * KK + t], sfr[b][t]);
+                st(&row.e[j], acc);
+            }
+            T *dst = op + u * ostep + i * orow;
+            if constexpr (R == 2 || R == 4) {
+                if (vec_ok) {   // one store of R elements
+                    using Bits = typename RowBits<sizeof(T) * R>::type;
+                    Bits bits = __builtin_bit_cast(Bits, row);
+                    // opaque to the compiler, which would otherwise undo the
+                    // packing of 2-byte results into 2-byte stores
+                    if constexpr (sizeof(T) == 2) asm("" : "+v"(bits));
+                    __builtin_nontemporal_store(bits, reinterpret_cast<Bits *>(dst));
+                    continue;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < R; ++j) dst[j] = row.e[j];
+        }
+    }
 }
 
 template <typename T, int K, int R, bool MUL>
@@ -49,6 +112,7 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RR = R * R, RAD = K / 2;
     constexpr int U = KK <= 9 ? 4 : 2;              // channels whose loads are issued together
+    constexpr int Q = 4;                            // tap loads in flight per thread while staging
     extern __shared__ __align__(16) unsigned char up_smem[];
     A *taps = reinterpret_cast<A *>(up_smem);   // [channel][branch][tap]
 
@@ -61,16 +125,18 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
     const int nch = min(cpb, C - c0);
     const int plane = H * W;
 
-    const int pix = pb * kThreads + (int)threadIdx.x;
-    const bool live = pix < plane;     // idle lanes still take part in the barriers
-    const int y = live ? pix / W : 0, xx = live ? pix - y * W : 0;
+    // Lanes past the end of the plane work on its last pixel and store nothing:
+    // no branch around the loads, and they still take part in the barriers.
+    const int pix_raw = pb * kThreads + (int)threadIdx.x;
+    const bool live = pix_raw < plane;
+    const int pix = min(pix_raw, plane - 1);
+    const int y = pix / W, xx = pix - y * W;
 
     A sfr[RR][KK];
 #pragma unroll
     for (int b = 0; b < RR; ++b)
 #pragma unroll
-        for (int t = 0; t < KK; ++t)
-            sfr[b][t] = live ? (A)ld(f.sf[b] + (n * KK + t) * plane + pix) : (A)0;
+        for (int t = 0; t < KK; ++t) sfr[b][t] = (A)ld(f.sf[b] + (n * KK + t) * plane + pix);
 
     // neighbours of X: offset from the pixel and whether it lies in the plane
     int off[KK];
@@ -80,8 +146,8 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
 #pragma unroll
         for (int j = 0; j < K; ++j) {
             const int iy = y + (i - RAD) * D, ix = xx + (j - RAD) * D;
-            inside[i * K + j] = live && iy >= 0 && iy < H && ix >= 0 && ix < W;
-            off[i * K + j] = (i - RAD) * D * W + (j - RAD) * D;
+            inside[i * K + j] = iy >= 0 && iy < H && ix >= 0 && ix < W;
+            off[i * K + j] = inside[i * K + j] ? (i - RAD) * D * W + (j - RAD) * D : 0;
         }
 
     const int64_t orow = (int64_t)W * R;            // elements per result row
@@ -91,54 +157,49 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
     for (int s0 = 0; s0 < nch; s0 += stage) {
         const int ns = min(stage, nch - s0);
         if (s0 > 0) __syncthreads();                // the previous taps have been used
-        // channel taps of this stage: contiguous per branch, so coalesced
+        // Channel taps of this stage, widened to the accumulator type.  Per
+        // branch they are ns*KK contiguous elements; Q loads per thread are
+        // issued before the first is written to LDS.
+        const int per = ns * KK, total = RR * per;
+        const int64_t cf0 = (n * C + c0 + s0) * KK;
+        for (int e0 = threadIdx.x; e0 < total; e0 += Q * kThreads) {
+            A v[Q];
 #pragma unroll
-        for (int b = 0; b < RR; ++b) {
-            const T *src = f.cf[b] + (n * C + c0 + s0) * KK;
-            for (int e = threadIdx.x; e < ns * KK; e += kThreads) {
-                const int ch = e / KK, t = e - ch * KK;
-                taps[(ch * RR + b) * KK + t] = (A)ld(src + e);
+            for (int q = 0; q < Q; ++q) {
+                const int e = min(e0 + q * kThreads, total - 1);
+                const int b = e / per, r = e - b * per;
+                const T *src = f.cf[0];
+#pragma unroll
+                for (int bb = 1; bb < RR; ++bb)
+                    if (b == bb) src = f.cf[bb];
+                v[q] = (A)ld(src + cf0 + r);
+            }
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                const int e = e0 + q * kThreads;
+                if (e < total) {
+                    const int b = e / per, r = e - b * per;
+                    const int ch = r / KK, t = r - ch * KK;
+                    taps[(ch * RR + b) * KK + t] = v[q];
+                }
             }
         }
         __syncthreads();
         if (!live) continue;
-        // U channels at a time: all their loads are issued before the first
-        // result is needed, so a wave keeps U*K*K loads in flight
-        for (int ch = 0; ch < ns; ch += U, xp += (int64_t)U * plane, op += U * ostep) {
-            A xv[U][KK];
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int t = 0; t < KK; ++t)
-                    xv[u][t] = (ch + u < ns && inside[t]) ? (A)ld(xp + (int64_t)u * plane + off[t])
-                                                          : (A)0;
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (ch + u >= ns) break;
-                const A *w = taps + (ch + u) * RR * KK;
-#pragma unroll
-                for (int i = 0; i < R; ++i) {
-                    Row<T, R> row;
-#pragma unroll
-                    for (int j = 0; j < R; ++j) {
-                        const int b = i * R + j;
-                        A acc = 0;
-#pragma unroll
-                        for (int t = 0; t < KK; ++t)
-                            acc += xv[u][t] * comb<MUL, A>(w[b * KK + t], sfr[b][t]);
-                        st(&row.e[j], acc);
-                    }
-                    T *dst = op + u * ostep + i * orow;
-                    if ((R == 2 || R == 4) && vec_ok) {
-                        *reinterpret_cast<Row<T, R> *>(dst) = row;
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < R; ++j) dst[j] = row.e[j];
-                    }
-                }
-            }
-        }
+        int ch = 0;
+        for (; ch + U <= ns; ch += U, xp += (int64_t)U * plane, op += U * ostep)
+            up_channels<T, K, R, MUL, U, A>(xp, op, taps + ch * RR * KK, plane, orow, ostep, off,
+                                            inside, sfr, vec_ok);
+        for (; ch < ns; ++ch, xp += plane, op += ostep)
+            up_channels<T, K, R, MUL, 1, A>(xp, op, taps + ch * RR * KK, plane, orow, ostep, off,
+                                            inside, sfr, vec_ok);
     }
+}
+
+// Tuning knob from the environment (experiments only; results do not change).
+int up_tune(const char *name, int fallback) {
+    const char *v = std::getenv(name);
+    return (v && *v) ? std::atoi(v) : fallback;
 }
 
 template <typename T, int K, int R>
@@ -146,19 +207,42 @@ hipError_t launch(bool mul, const UpFilters<T> &f, const T *x, T *out, int64_t N
                   int W, int D, hipStream_t stream) {
     using A = typename Acc<T>::type;
     const int64_t pblocks = cdiv((int64_t)H * W, kThreads);
+    const int per_channel = R * R * K * K * (int)sizeof(A);
     // Split the channels only as far as it takes to fill the chip: every chunk
     // re-reads the R*R*K*K spatial taps of its pixels.
+    // Split the channels over blocks until the chip is full once: as many
+    // blocks as can be resident together (a second round of blocks would start
+    // late and finish alone), and no further, because every chunk re-reads the
+    // R*R*K*K spatial taps of its pixels.
+    auto kern = mul ? k_up_forward<T, K, R, true> : k_up_forward<T, K, R, false>;
+    static std::atomic<int> resident[2] = {{0}, {0}};     // blocks per CU, per combine
+    int per_cu = resident[mul].load(std::memory_order_relaxed);
+    if (per_cu == 0) {
+        const size_t lds_max = (size_t)std::min(kStageChannels, kStageBytes / per_channel) * per_channel;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, kThreads, lds_max) !=
+                hipSuccess || per_cu < 1) {
+            (void)hipGetLastError();
+            per_cu = 2;
+        }
+        resident[mul].store(per_cu, std::memory_order_relaxed);
+    }
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        cus = 256;
+    }
+    const int64_t target = up_tune("DDF_TUNE_UP_BLOCKS", per_cu * cus);
+    const int min_chunk = std::max(1, up_tune("DDF_TUNE_UP_MIN_CHUNK", 8));
     int csplit = 1;
-    while (N * pblocks * csplit < 2048 && C / (csplit * 2) >= 8) csplit *= 2;
+    while (N * pblocks * csplit * 2 <= target && C / (csplit * 2) >= min_chunk) csplit *= 2;
     const int cpb = (int)cdiv(C, csplit);
     csplit = (int)cdiv(C, cpb);
     const int64_t blocks = N * pblocks * csplit;
     if (blocks > 2147483647) return hipErrorInvalidConfiguration;
-    const int per_channel = R * R * K * K * (int)sizeof(A);
     const int stage = std::max(1, std::min({cpb, kStageChannels, kStageBytes / per_channel}));
     const size_t lds = (size_t)stage * per_channel;
     const int vec_ok = ((uintptr_t)out % (sizeof(T) * R)) == 0;
-    auto kern = mul ? k_up_forward<T, K, R, true> : k_up_forward<T, K, R, false>;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), lds, stream, f, x, out, C, H,
                        W, D, cpb, csplit, (int)pblocks, stage, vec_ok);
     return hipGetLastError();

@@ -91,16 +91,20 @@ def test_unsupported_pair_composes_from_ddf():
     check_up(1, 4, 8, 9, 5, 1, 3, 'add', torch.float32)
 
 
-def test_misaligned_output_takes_scalar_stores():
-    x, cfs, sfs, _ = up_case(2, 6, 7, 9, 3, 2, torch.float32, seed=5)
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+@pytest.mark.parametrize('scale', [2, 4])
+def test_misaligned_output(scale, dtype):
+    """A result that starts one element past an aligned address cannot take
+    one aligned store per row."""
+    x, cfs, sfs, _ = up_case(2, 6, 7, 9, 3, scale, dtype, seed=5)
     xd, cfd, sfd = x.cuda(), [t.cuda() for t in cfs], [t.cuda() for t in sfs]
-    n = 2 * 6 * 14 * 18
-    buf = torch.full((n + 2,), 7.0, device='cuda')
-    out = buf[1:1 + n].view(2, 6, 14, 18)
-    assert out.data_ptr() % 8 == 4
-    _lib.up_forward(xd, cfd, sfd, out, 3, 1, 2, 'mul')
+    n = 2 * 6 * 7 * 9 * scale * scale
+    buf = torch.full((n + 2,), 7.0, device='cuda', dtype=dtype)
+    out = buf[1:1 + n].view(2, 6, 7 * scale, 9 * scale)
+    assert out.data_ptr() % (2 * out.element_size()) == out.element_size()
+    _lib.up_forward(xd, cfd, sfd, out, 3, 1, scale, 'mul')
     torch.cuda.synchronize()
-    assert rel_err(out, oracle.up_forward(x, cfs, sfs, 3, 1, 2, 'mul')) <= 1e-5
+    assert rel_err(out, oracle.up_forward(x, cfs, sfs, 3, 1, scale, 'mul')) <= TOL[dtype]
     assert buf[0].item() == 7.0 and buf[-1].item() == 7.0    # nothing outside the result
 
 
