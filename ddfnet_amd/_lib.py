@@ -29,6 +29,8 @@ SYMBOLS = {
     'ddf_hip_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
     'ddf_hip_filter_norm': (_i, [_vp] * 2 + [_i64] * 2 + [_i, _i64, ctypes.c_double] + [_vp] * 2 +
                             [_i, _vp]),
+    'ddf_hip_filter_norm_backward': (_i, [_vp] * 4 + [_i64] * 2 + [_i, _i64, ctypes.c_double, _vp,
+                                          _i, _vp]),
     'ddf_hip_up_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 5 + [_vp]),
 }
 
@@ -137,6 +139,21 @@ def filter_norm(x, outer, groups, taps, inner, gain, gain_vec=None, offset_vec=N
             _ptr(offset_vec), DTYPE[x.dtype], _stream())
     check(rc)
     return y
+
+
+def filter_norm_backward(grad_y, x, outer, groups, taps, inner, gain, gain_vec=None,
+                         want_gain_terms=False):
+    """Gradient of ``filter_norm`` with respect to ``x``; also returns
+    ``grad_y * standardised(x)`` (or None), whose sum over (outer, inner) is
+    the gradient of ``gain_vec``."""
+    grad_x = torch.empty_like(x)
+    terms = torch.empty_like(x) if want_gain_terms else None
+    with on_device_of(x):
+        rc = lib().ddf_hip_filter_norm_backward(
+            _ptr(grad_y), _ptr(x), _ptr(grad_x), _ptr(terms), outer, groups, taps, inner,
+            float(gain), _ptr(gain_vec), DTYPE[x.dtype], _stream())
+    check(rc)
+    return grad_x, terms
 
 
 def up_forward(features, channel_filters, spatial_filters, output, k, d, scale, combine):

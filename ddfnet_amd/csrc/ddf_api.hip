@@ -225,6 +225,37 @@ int ddf_hip_filter_norm(const void *x, void *y, int64_t outer, int64_t groups, i
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_filter_norm launch");
 }
 
+int ddf_hip_filter_norm_backward(const void *grad_y, const void *x, void *grad_x,
+                                 void *gain_terms, int64_t outer, int64_t groups, int taps,
+                                 int64_t inner, double gain, const void *gain_vec, int dtype,
+                                 void *stream) {
+    if (outer < 0 || groups < 0 || taps < 0 || inner < 0)
+        return fail(DDF_ERR_BAD_ARG, "negative tensor size");
+    if (dtype != DDF_F16 && dtype != DDF_F32 && dtype != DDF_F64)
+        return fail(DDF_ERR_BAD_ARG, "unknown dtype %d", dtype);
+    if (outer * groups * taps * inner == 0) return DDF_OK;
+    if (!grad_y || !x || !grad_x) return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t err;
+    switch (dtype) {
+        case DDF_F16:
+            err = ddf::filter_norm_backward<__half>(
+                (const __half *)grad_y, (const __half *)x, (__half *)grad_x, (__half *)gain_terms,
+                outer, groups, taps, inner, gain, (const __half *)gain_vec, st);
+            break;
+        case DDF_F32:
+            err = ddf::filter_norm_backward<float>(
+                (const float *)grad_y, (const float *)x, (float *)grad_x, (float *)gain_terms,
+                outer, groups, taps, inner, gain, (const float *)gain_vec, st);
+            break;
+        default:
+            err = ddf::filter_norm_backward<double>(
+                (const double *)grad_y, (const double *)x, (double *)grad_x, (double *)gain_terms,
+                outer, groups, taps, inner, gain, (const double *)gain_vec, st);
+    }
+    return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_filter_norm_backward launch");
+}
+
 int ddf_hip_up_forward(const void *features, const void *const *channel_filters,
                        const void *const *spatial_filters, void *output, int64_t N, int64_t C,
                        int64_t H, int64_t W, int kernel_size, int dilation, int scale,

@@ -63,6 +63,13 @@ template <typename T>
 hipError_t filter_norm(const T *x, T *y, int64_t outer, int64_t groups, int taps, int64_t inner,
                        double gain, const T *gain_vec, const T *offset_vec, hipStream_t st);
 
+// Gradient of filter_norm with respect to x; `terms` (nullable) receives
+// dy * standardised(x), whose sum over (outer, inner) is the gain_vec gradient.
+template <typename T>
+hipError_t filter_norm_backward(const T *dy, const T *x, T *dx, T *terms, int64_t outer,
+                                int64_t groups, int taps, int64_t inner, double gain,
+                                const T *gain_vec, hipStream_t st);
+
 // All scale*scale sub-pixel branches of an up-sampling DDF in one launch,
 // written into the pixel-shuffled (N, C, H*scale, W*scale) result; cf / sf are
 // host arrays of scale*scale device pointers.

@@ -25,6 +25,37 @@ def _standardize(x, dim):
     return (x - mean) / (var.sqrt() + 1e-10)
 
 
+class _FilterNormFunction(torch.autograd.Function):
+    """``gain * standardised(x) + offset`` over the taps of an
+    ``(outer, groups, taps, inner)`` tensor, forward and backward one launch each."""
+
+    @staticmethod
+    def forward(ctx, x, gain_vec, offset_vec, outer, groups, taps, inner, gain):
+        x = x.contiguous()
+        ctx.save_for_backward(x, gain_vec)
+        ctx.dims = (outer, groups, taps, inner)
+        ctx.gain = gain
+        return _lib.filter_norm(x, outer, groups, taps, inner, gain, gain_vec, offset_vec)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_y):
+        x, gain_vec = ctx.saved_tensors
+        outer, groups, taps, inner = ctx.dims
+        grad_y = grad_y.to(x.dtype).contiguous()
+        want_gain = gain_vec is not None and ctx.needs_input_grad[1]
+        grad_x, terms = _lib.filter_norm_backward(grad_y, x, outer, groups, taps, inner, ctx.gain,
+                                                  gain_vec, want_gain)
+        grad_gain = grad_offset = None
+        if want_gain:
+            grad_gain = terms.view(outer, groups, taps, inner).sum(dim=(0, 3)).reshape(-1)
+        if ctx.needs_input_grad[2]:
+            grad_offset = grad_y.view(outer, groups, taps, inner).sum(dim=(0, 3)).reshape(-1)
+        if not ctx.needs_input_grad[0]:
+            grad_x = None
+        return grad_x, grad_gain, grad_offset, None, None, None, None, None
+
+
 class FilterNorm(nn.Module):
     """Standardise every predicted filter over its ``kernel_size**2`` taps, then
     scale by a gain: the constant ``calculate_gain(nonlinearity) / kernel_size``
@@ -59,21 +90,17 @@ class FilterNorm(nn.Module):
         return x
 
     def _fused(self, x, outer, inner):
-        """One HIP launch instead of the chain of elementwise ops below.  Used
-        where no gradient is wanted (the kernel has no backward): inference."""
+        """One HIP launch instead of the chain of elementwise ops below (and one
+        more for its gradient, instead of what autograd derives from the chain)."""
         taps = x.numel() // max(outer * self.in_channels * inner, 1)
         gain_vec = self.std.to(x.dtype) if self.runing_std else None
         offset_vec = self.mean.to(x.dtype) if self.runing_mean else None
-        return _lib.filter_norm(x.contiguous(), outer, self.in_channels, taps, inner,
-                                1.0 if self.runing_std else self.std, gain_vec, offset_vec)
+        gain = 1.0 if self.runing_std else self.std
+        return _FilterNormFunction.apply(x, gain_vec, offset_vec, outer, self.in_channels, taps,
+                                         inner, gain)
 
     def _use_fused(self, x):
-        if not x.is_cuda or x.dtype not in _lib.DTYPE or x.numel() == 0:
-            return False
-        if not torch.is_grad_enabled():
-            return True
-        params = [p for p in (self.std, getattr(self, 'mean', None)) if isinstance(p, nn.Parameter)]
-        return not (x.requires_grad or any(p.requires_grad for p in params))
+        return x.is_cuda and x.dtype in _lib.DTYPE and x.numel() > 0
 
     def forward(self, x):
         if self._use_fused(x):

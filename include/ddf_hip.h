@@ -134,13 +134,29 @@ int ddf_hip_backward(const void *grad_output, const void *features,
  * `gain_vec[group*taps + tap]` (or by the scalar `gain` when gain_vec is
  * NULL) and shifted by `offset_vec[group*taps + tap]` (unless NULL).
  * Spatial branch: (b, head, k*k, h*w).  Channel branch: (b, c, k*k, 1).
- * `y` may alias `x`.  Forward only: training keeps the framework's autograd
- * through the unfused formulation.
+ * `y` may alias `x` (not when ddf_hip_filter_norm_backward is to follow: it
+ * needs the original `x`).
  */
 int ddf_hip_filter_norm(const void *x, void *y, int64_t outer, int64_t groups,
                         int taps, int64_t inner, double gain,
                         const void *gain_vec, const void *offset_vec,
                         int dtype, void *stream);
+
+/*
+ * Gradient of ddf_hip_filter_norm with respect to `x` (what autograd derives
+ * from the op chain of FilterNorm.forward, ddf/ddf.py:145-173, in the
+ * reference).  `grad_y` and `x` are the (outer, groups, taps, inner) tensors of
+ * the forward call, `gain` / `gain_vec` the same gains; mean and deviation are
+ * recomputed from `x`.  `grad_x` is written in full.  `gain_terms`, unless
+ * NULL, receives grad_y * standardised(x) element by element: its sum over
+ * (outer, inner) is the gradient of `gain_vec`; the gradient of `offset_vec`
+ * is the same sum of `grad_y` itself.  `grad_x` may alias `grad_y`.
+ */
+int ddf_hip_filter_norm_backward(const void *grad_y, const void *x,
+                                 void *grad_x, void *gain_terms, int64_t outer,
+                                 int64_t groups, int taps, int64_t inner,
+                                 double gain, const void *gain_vec, int dtype,
+                                 void *stream);
 
 /*
  * Up-sampling DDF forward (DDFUpPack.forward, ddf/ddf.py:257-272): the

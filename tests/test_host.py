@@ -180,6 +180,16 @@ def test_filter_norm_argument_validation_needs_no_gpu():
     assert b'null' in lib.ddf_hip_last_error()
 
 
+def test_filter_norm_backward_argument_validation_needs_no_gpu():
+    lib = _lib.lib()
+    bwd = lib.ddf_hip_filter_norm_backward
+    assert bwd(None, None, None, None, 1, -1, 9, 4, 1.0, None, 1, None) == 1
+    assert bwd(None, None, None, None, 1, 1, 9, 4, 1.0, None, 3, None) == 1
+    assert bwd(None, None, None, None, 1, 1, 0, 4, 1.0, None, 1, None) == 0
+    assert bwd(None, None, None, None, 2, 1, 9, 4, 1.0, None, 1, None) == 1
+    assert b'null' in lib.ddf_hip_last_error()
+
+
 def test_up_forward_argument_validation_needs_no_gpu():
     import ctypes
     lib = _lib.lib()

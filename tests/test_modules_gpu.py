@@ -165,7 +165,7 @@ def test_resnet50_fp16_inference_and_layer_timing():
 
 
 # ---------------------------------------------------------------------------
-# fused filter normalisation (inference path of FilterNorm)
+# fused filter normalisation
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize('dtype,tol', [(torch.float64, 1e-12), (torch.float32, 1e-5),
                                        (torch.float16, 1e-2)])
@@ -178,8 +178,8 @@ def test_resnet50_fp16_inference_and_layer_timing():
     ('channel', (3, 7 * 9), 7, 3, False, False),
 ])
 def test_fused_filter_norm_matches_formula(ftype, shape, groups, k, rstd, rmean, dtype, tol):
-    """One HIP launch (no gradient wanted) against the op-by-op formulation of
-    the same module evaluated in fp64 on the CPU."""
+    """One HIP launch against the op-by-op formulation of the same module
+    evaluated in fp64 on the CPU."""
     torch.manual_seed(3)
     fn = ddfnet_amd.FilterNorm(groups, k, ftype, 'relu', running_std=rstd,
                                running_mean=rmean).cuda().to(dtype)
@@ -189,18 +189,64 @@ def test_fused_filter_norm_matches_formula(ftype, shape, groups, k, rstd, rmean,
         got = fn(x)
     assert got.dtype == dtype
     ref = copy.deepcopy(fn).cpu().double()
-    want = ref(x.detach().cpu().double().requires_grad_(True))   # grad wanted: unfused path
+    want = ref(x.detach().cpu().double())
     assert got.shape == want.shape
     err = (got.cpu().double() - want.detach()).abs().max().item() / want.abs().max().item()
     assert err <= tol, err
 
 
-def test_filter_norm_training_path_keeps_autograd():
+@pytest.mark.parametrize('dtype,tol', [(torch.float64, 1e-11), (torch.float32, 2e-5),
+                                       (torch.float16, 1e-2)])
+@pytest.mark.parametrize('ftype,shape,groups,k,rstd,rmean', [
+    ('spatial', (3, 9, 13, 11), 1, 3, False, False),
+    ('spatial', (2, 4 * 9, 7, 5), 4, 3, True, True),
+    ('spatial', (1, 25, 6, 6), 1, 5, False, True),
+    ('channel', (4, 16 * 9), 16, 3, True, False),
+    ('channel', (2, 5 * 25, 1, 1), 5, 5, True, True),
+    ('channel', (3, 7 * 9), 7, 3, False, False),
+])
+def test_fused_filter_norm_gradients(ftype, shape, groups, k, rstd, rmean, dtype, tol):
+    """The one-launch backward against torch.autograd through the op-by-op
+    formulation of the same module in fp64 on the CPU: gradient of the input,
+    of the learned gain and of the learned offset."""
+    torch.manual_seed(4)
+    fn = ddfnet_amd.FilterNorm(groups, k, ftype, 'relu', running_std=rstd,
+                               running_mean=rmean).cuda().to(dtype)
+    x = (torch.randn(*shape) * 2 + 0.5).to(dtype).cuda().requires_grad_(True)
+    assert fn._use_fused(x)
+    out = fn(x)
+    go = torch.randn(out.shape).to(dtype).cuda()
+    out.backward(go)
+    ref = copy.deepcopy(fn).cpu().double()
+    ref.zero_grad()
+    xr = x.detach().cpu().double().requires_grad_(True)
+    ref(xr).backward(go.cpu().double())
+
+    def err(got, want):
+        return (got.cpu().double() - want).abs().max().item() / want.abs().max().item()
+
+    assert err(x.grad, xr.grad) <= tol
+    if rstd:
+        assert err(fn.std.grad, ref.std.grad) <= tol
+    if rmean:
+        assert err(fn.mean.grad, ref.mean.grad) <= tol
+
+
+def test_filter_norm_gradient_only_where_asked():
     fn = ddfnet_amd.FilterNorm(8, 3, 'channel', 'relu', running_std=True).cuda()
+    fn.std.requires_grad_(False)
     x = torch.randn(2, 72, device='cuda', requires_grad=True)
+    fn(x).sum().backward()
+    assert x.grad is not None and fn.std.grad is None
+    x2 = torch.randn(2, 72, device='cuda')
+    fn.std.requires_grad_(True)
+    fn(x2).sum().backward()
+    assert fn.std.grad is not None
+
+
+def test_filter_norm_cpu_path_is_op_by_op():
+    fn = ddfnet_amd.FilterNorm(2, 3, 'spatial')
+    x = torch.randn(1, 18, 4, 4, requires_grad=True)
     assert not fn._use_fused(x)
     fn(x).sum().backward()
-    assert x.grad is not None and fn.std.grad is not None
-    with torch.no_grad():
-        fused = fn(x)
-    assert torch.allclose(fused, fn(x).detach(), rtol=1e-5, atol=1e-6)
+    assert x.grad is not None
