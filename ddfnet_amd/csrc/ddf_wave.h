@@ -28,11 +28,6 @@
 
 #include "ddf_common.h"
 
-// Hook for a timing harness; expands to nothing in the library.
-#ifndef DDF_STAMP
-#define DDF_STAMP(slot)
-#endif
-
 namespace ddf {
 
 constexpr int kMaxSlots = 8;
@@ -351,7 +346,6 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_forward(WaveGeom g, const T
     T *lds_out = reinterpret_cast<T *>(lds_in + g.tile + kSpare);
     A *taps = reinterpret_cast<A *>(lds_out + g.lin_tile + kIdle);
 
-    DDF_STAMP(0);
     WaveWork ww;
     if (!ww.init(g, wave) || ww.c_end <= ww.c_begin) return;
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
@@ -377,7 +371,6 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_forward(WaveGeom g, const T
     fst.issue(sf + (ww.n * KK * g.Ho + y0) * g.Wo, oplane);
     TapStager<KK, T, A> tst;
     tst.issue(cf, ww.n * g.C + ww.c_begin, nch, lane);
-    DDF_STAMP(1);
 
     // per slot: is the cell real, where its taps start in the tile, where its
     // result goes in the linear strip; its spatial-filter taps in registers
@@ -401,17 +394,14 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_forward(WaveGeom g, const T
     zero_tile(lds_in, g.tile, lane);
     tst.put(taps, nch, lane);
     fst.collect(lds_out, ob, sfr);
-    DDF_STAMP(2);
 
     auto channel = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         stg.template commit<ST>(lds_in, wide);
-        DDF_STAMP(3 + 4 * ci);
         stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch - 1) * iplane);
         wave_sync();
         A w[KK];
         load_taps<KK>(taps, ci, w);
-        DDF_STAMP(4 + 4 * ci);
         if constexpr (kFlat) {
             // No branch in here: every slot is computed, idle lanes and idle
             // slots included (their tile addresses are valid), and the results
@@ -447,10 +437,8 @@ __global__ __launch_bounds__(kWave * kMaxWpb) void k_forward(WaveGeom g, const T
             }
         }
         wave_sync();
-        DDF_STAMP(5 + 4 * ci);
         store_strip<T, V>(lds_out, os + (int64_t)ci * oplane, n_out, lane);
         wave_sync();
-        DDF_STAMP(6 + 4 * ci);
     };
 
     auto group = [&](int c) __attribute__((always_inline)) {
@@ -873,7 +861,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
     T *lds_go = reinterpret_cast<T *>(lds_g + (DX ? g.tile + kSpare : 0));
     A *taps = reinterpret_cast<A *>(lds_go + g.lin_tile + kIdle);
 
-    DDF_STAMP(0);
     WaveWork ww;
     if (!ww.init(g)) return;   // whole block leaves together
     const int lr = lane >> g.lw_shift, lc = lane & ((1 << g.lw_shift) - 1);
@@ -946,7 +933,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         }
         tst.issue(cf, ww.n * g.C + c_first, nch1, lane);
     }
-    DDF_STAMP(1);
 
     bool ok[PS];
     int lb[PS], ob[PS];
@@ -1008,7 +994,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         }
     }
     wave_sync();
-    DDF_STAMP(2);
     int wb[PS];   // where the dX value of a slot goes: idle lanes write behind the strip
 #pragma unroll
     for (int m = 0; m < PS; ++m) wb[m] = ok[m] ? ob[m] : g.lin_tile + lane;
@@ -1020,7 +1005,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         stg.template commit<ST>(lds_in, wide);
         if constexpr (DX) stg_g.template commit<ST>(lds_g, wide);
         else sgo.template commit<ST>(lds_go);
-        DDF_STAMP(3 + 4 * ci);
         stg.template issue<ST>(xs + (int64_t)min(ci + NST, nch1 - 1) * iplane);
         issue_go(st_tag, gs + (int64_t)min(ci + NST, nch1 - 1) * oplane);
         wave_sync();
@@ -1063,12 +1047,10 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
                 st(lds_go + wb[m], accx);
             }
         }
-        DDF_STAMP(4 + 4 * ci);
         if constexpr (DX) {
             wave_sync();
             store_strip<T, V>(lds_go, ds + (int64_t)ci * iplane, n_out, lane);
         }
-        DDF_STAMP(5 + 4 * ci);
         if (want_cf) {
             const A tot = bfly_sum<KK, 0, A>(pcf, lane);
             if (lane < bfly_writers<KK>()) {
@@ -1078,7 +1060,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
             }
         }
         wave_sync();
-        DDF_STAMP(6 + 4 * ci);
     };
     auto group = [&](int c) __attribute__((always_inline)) {
         channel(std::integral_constant<int, 0>{}, c);
@@ -1099,11 +1080,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         }
     }
 
-    DDF_STAMP(70);
     if (!want_sf) return;
     // Add the waves' dSF accumulators: one pixel slot at a time through LDS.
     __syncthreads();
-    DDF_STAMP(71);
     A *red = reinterpret_cast<A *>(smem);
 #pragma unroll
     for (int m = 0; m < PS; ++m) {
@@ -1123,7 +1102,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
         }
         __syncthreads();
     }
-    DDF_STAMP(72);
 }
 
 // out[o, i] = sum_p part[o, p, i] for o < outer, p < parts, i < inner.  A
