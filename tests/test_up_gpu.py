@@ -151,3 +151,56 @@ def test_ddfuppack_uses_the_fused_operator(monkeypatch):
     with torch.no_grad():
         up(torch.randn(1, 8, 6, 6, device='cuda'))
     assert calls == [1]
+
+
+def _random_up_cases(count, seed):
+    import random
+    rng = random.Random(seed)
+    for _ in range(count):
+        k, scale = rng.choice([(1, 2), (1, 3), (1, 4), (3, 2), (3, 2), (3, 3), (3, 4), (5, 2), (7, 2)])
+        yield (rng.randint(1, 3), rng.randint(1, 40), rng.randint(1, 23), rng.randint(1, 23), k,
+               rng.choice([1, 1, 2, 3]), scale, rng.choice(['mul', 'add']),
+               rng.choice([torch.float64, torch.float32, torch.float16]))
+
+
+@pytest.mark.parametrize('chunk', range(3))
+def test_random_shapes_against_oracle(chunk):
+    """60 seeded random problems, forward and every gradient."""
+    for i, (N, C, H, W, k, d, scale, combine, dtype) in enumerate(_random_up_cases(20, 500 + chunk)):
+        check_up(N, C, H, W, k, d, scale, combine, dtype, seed=chunk * 100 + i)
+
+
+def test_up_forward_replays_in_a_hip_graph():
+    """The fused launch enqueues one kernel and allocates only its result, so
+    it can be captured; every replay, with eager work in between, reproduces
+    the eager result bit for bit."""
+    N, C, H, W, k, scale = 2, 24, 12, 10, 3, 2
+    cases = [up_case(N, C, H, W, k, scale, torch.float32, seed=s) for s in (31, 32, 33)]
+    x = cases[0][0].cuda()
+    cfs = [t.cuda() for t in cases[0][1]]
+    sfs = [t.cuda() for t in cases[0][2]]
+
+    def step():
+        with torch.no_grad():
+            return ddf_up(x, cfs, sfs, k, 1, scale, 'mul')
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    for cx, ccfs, csfs, _ in cases:
+        x.copy_(cx.cuda())
+        for dst, src in zip(cfs + sfs, ccfs + csfs):
+            dst.copy_(src.cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        got = captured.clone()
+        want = step()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want)
+        assert rel_err(got, oracle.up_forward(cx, ccfs, csfs, k, 1, scale, 'mul')) <= 1e-5
