@@ -32,6 +32,8 @@ SYMBOLS = {
     'ddf_hip_filter_norm_backward': (_i, [_vp] * 4 + [_i64] * 2 + [_i, _i64, ctypes.c_double, _vp,
                                           _i, _vp]),
     'ddf_hip_up_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 5 + [_vp]),
+    'ddf_hip_up_backward_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u]),
+    'ddf_hip_up_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _vp]),
 }
 
 _lib = None
@@ -168,6 +170,31 @@ def up_forward(features, channel_filters, spatial_filters, output, k, d, scale, 
     check(lib().ddf_hip_up_forward(
         _ptr(features), cf, sf, _ptr(output), N, C, H, W, k, d, scale, COMBINE[combine],
         DTYPE[features.dtype], _stream()))
+
+
+def up_backward(grad_output, features, channel_filters, spatial_filters, grad_features,
+                grad_channel_filters, grad_spatial_filters, k, d, scale, combine):
+    """Gradients of ``up_forward``; a gradient tensor given as None is not
+    computed.  Allocates the library's workspace from torch's allocator."""
+    N, C, H, W = features.shape
+    branches = scale * scale
+    need = ((NEED_DX if grad_features is not None else 0) |
+            (NEED_DCF if any(t is not None for t in grad_channel_filters) else 0) |
+            (NEED_DSF if any(t is not None for t in grad_spatial_filters) else 0))
+    if need == 0:
+        return
+
+    def ptrs(tensors):
+        return (ctypes.c_void_p * branches)(*[None if t is None else t.data_ptr() for t in tensors])
+
+    dt = DTYPE[features.dtype]
+    nbytes = int(lib().ddf_hip_up_backward_workspace_bytes(N, C, H, W, k, d, scale,
+                                                           COMBINE[combine], dt, need))
+    workspace = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=features.device)
+    check(lib().ddf_hip_up_backward(
+        _ptr(grad_output), _ptr(features), ptrs(channel_filters), ptrs(spatial_filters),
+        _ptr(grad_features), ptrs(grad_channel_filters), ptrs(grad_spatial_filters),
+        _ptr(workspace), nbytes, N, C, H, W, k, d, scale, COMBINE[combine], dt, need, _stream()))
 
 
 def up_forward_covers(k, scale):

@@ -96,6 +96,58 @@ int backward_typed(const ddf::Problem &p, const void *go, const void *x, const v
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_backward launch");
 }
 
+size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+// Workspace of the up-sampling backward: the lattices of dO, the per-branch
+// feature gradients (when dX is wanted) and one branch's own workspace.
+struct UpWorkspace {
+    size_t lattices, dx_parts, branch, total;
+};
+
+UpWorkspace up_workspace(const ddf::Problem &p, int scale, int dtype, unsigned need) {
+    const size_t esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
+    const size_t n_x = (size_t)(p.N * p.C * p.H * p.W);
+    UpWorkspace w;
+    w.lattices = align256(n_x * esz * scale * scale);
+    w.dx_parts = (need & DDF_NEED_DX) ? align256(n_x * esz * scale * scale) : 0;
+    w.branch = ddf::tiled_backward_supported(p, dtype)
+                   ? align256(ddf::tiled_backward_workspace(p, dtype, need))
+                   : 0;
+    w.total = w.lattices + w.dx_parts + w.branch;
+    return w;
+}
+
+template <typename T>
+int up_backward_typed(const ddf::Problem &p, int scale, const void *go, const void *x,
+                      const void *const *cfs, const void *const *sfs, void *dx, void *const *dcfs,
+                      void *const *dsfs, void *ws, int dtype, unsigned need, hipStream_t stream) {
+    const UpWorkspace w = up_workspace(p, scale, dtype, need);
+    unsigned char *base = static_cast<unsigned char *>(ws);
+    T *lat = reinterpret_cast<T *>(base);
+    T *parts = reinterpret_cast<T *>(base + w.lattices);
+    void *branch_ws = w.branch ? base + w.lattices + w.dx_parts : nullptr;
+    const int64_t n_x = p.N * p.C * p.H * p.W;
+    hipError_t err = ddf::up_split_lattices<T>((const T *)go, lat, p.N * p.C, p.H, p.W, scale, stream);
+    if (err != hipSuccess) return fail_hip(err, "ddf_hip_up_backward split launch");
+    for (int b = 0; b < scale * scale; ++b) {
+        unsigned bneed = need & DDF_NEED_DX;
+        if ((need & DDF_NEED_DCF) && dcfs && dcfs[b]) bneed |= DDF_NEED_DCF;
+        if ((need & DDF_NEED_DSF) && dsfs && dsfs[b]) bneed |= DDF_NEED_DSF;
+        if (bneed == 0) continue;
+        const int rc = backward_typed<T>(p, lat + b * n_x, x, cfs[b], sfs[b],
+                                         (need & DDF_NEED_DX) ? parts + b * n_x : nullptr,
+                                         dcfs ? dcfs[b] : nullptr, dsfs ? dsfs[b] : nullptr,
+                                         branch_ws, w.branch, dtype, bneed, DDF_VARIANT_AUTO,
+                                         stream);
+        if (rc != DDF_OK) return rc;
+    }
+    if (need & DDF_NEED_DX) {
+        err = ddf::up_sum_parts<T>(parts, (T *)dx, n_x, scale * scale, stream);
+        if (err != hipSuccess) return fail_hip(err, "ddf_hip_up_backward sum launch");
+    }
+    return DDF_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -294,6 +346,59 @@ int ddf_hip_up_forward(const void *features, const void *const *channel_filters,
                                           spatial_filters, (double *)output, st);
     }
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_up_forward launch");
+}
+
+size_t ddf_hip_up_backward_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W,
+                                           int kernel_size, int dilation, int scale, int combine,
+                                           int dtype, unsigned need_mask) {
+    if (check_problem(N, C, H, W, kernel_size, dilation, 1, combine, dtype, DDF_VARIANT_AUTO) !=
+            DDF_OK || scale < 2 || scale * scale > DDF_UP_MAX_BRANCHES)
+        return 0;
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, 1, combine);
+    return up_workspace(p, scale, dtype, need_mask & DDF_NEED_ALL).total;
+}
+
+int ddf_hip_up_backward(const void *grad_output, const void *features,
+                        const void *const *channel_filters, const void *const *spatial_filters,
+                        void *grad_features, void *const *grad_channel_filters,
+                        void *const *grad_spatial_filters, void *workspace, size_t workspace_bytes,
+                        int64_t N, int64_t C, int64_t H, int64_t W, int kernel_size, int dilation,
+                        int scale, int combine, int dtype, unsigned need_mask, void *stream) {
+    int rc = check_problem(N, C, H, W, kernel_size, dilation, 1, combine, dtype, DDF_VARIANT_AUTO);
+    if (rc != DDF_OK) return rc;
+    if (scale < 2 || scale * scale > DDF_UP_MAX_BRANCHES)
+        return fail(DDF_ERR_BAD_ARG, "scale must be 2..4 (got %d)", scale);
+    const unsigned need = need_mask & DDF_NEED_ALL;
+    if (need == 0 || N * C * H * W == 0) return DDF_OK;
+    if (!grad_output || !features || !channel_filters || !spatial_filters)
+        return fail(DDF_ERR_BAD_ARG, "null input tensor pointer");
+    for (int b = 0; b < scale * scale; ++b)
+        if (!channel_filters[b] || !spatial_filters[b])
+            return fail(DDF_ERR_BAD_ARG, "null filter pointer for branch %d", b);
+    if ((need & DDF_NEED_DX) && !grad_features)
+        return fail(DDF_ERR_BAD_ARG, "null pointer for a requested gradient");
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, 1, combine);
+    const size_t want = up_workspace(p, scale, dtype, need).total;
+    if (!workspace || workspace_bytes < want)
+        return fail(DDF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", want,
+                    workspace ? workspace_bytes : (size_t)0);
+    if (((uintptr_t)workspace & 255u) != 0)
+        return fail(DDF_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+        case DDF_F16:
+            return up_backward_typed<__half>(p, scale, grad_output, features, channel_filters,
+                                             spatial_filters, grad_features, grad_channel_filters,
+                                             grad_spatial_filters, workspace, dtype, need, st);
+        case DDF_F32:
+            return up_backward_typed<float>(p, scale, grad_output, features, channel_filters,
+                                            spatial_filters, grad_features, grad_channel_filters,
+                                            grad_spatial_filters, workspace, dtype, need, st);
+        default:
+            return up_backward_typed<double>(p, scale, grad_output, features, channel_filters,
+                                             spatial_filters, grad_features, grad_channel_filters,
+                                             grad_spatial_filters, workspace, dtype, need, st);
+    }
 }
 
 }  // extern "C"

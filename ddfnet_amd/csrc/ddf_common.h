@@ -79,6 +79,15 @@ hipError_t up_forward(int64_t N, int64_t C, int64_t H, int64_t W, int k, int d, 
                       bool mul, const T *x, const void *const *cf, const void *const *sf, T *out,
                       hipStream_t st);
 
+// Helpers of the up-sampling backward: the gradient of the pixel shuffle (dO
+// split into its scale*scale sub-pixel lattices, stored back to back) and the
+// sum of `parts` equally sized tensors stored back to back.
+template <typename T>
+hipError_t up_split_lattices(const T *go, T *lat, int64_t planes, int64_t H, int64_t W, int scale,
+                             hipStream_t st);
+template <typename T>
+hipError_t up_sum_parts(const T *in, T *out, int64_t count, int parts, hipStream_t st);
+
 bool tiled_forward_supported(const Problem &p, int dtype);
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,

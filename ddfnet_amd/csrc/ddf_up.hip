@@ -208,8 +208,6 @@ hipError_t launch(bool mul, const UpFilters<T> &f, const T *x, T *out, int64_t N
     using A = typename Acc<T>::type;
     const int64_t pblocks = cdiv((int64_t)H * W, kThreads);
     const int per_channel = R * R * K * K * (int)sizeof(A);
-    // Split the channels only as far as it takes to fill the chip: every chunk
-    // re-reads the R*R*K*K spatial taps of its pixels.
     // Split the channels over blocks until the chip is full once: as many
     // blocks as can be resident together (a second round of blocks would start
     // late and finish alone), and no further, because every chunk re-reads the
@@ -248,7 +246,62 @@ hipError_t launch(bool mul, const UpFilters<T> &f, const T *x, T *out, int64_t N
     return hipGetLastError();
 }
 
+// Gradient of the pixel shuffle: lat[b][nc][y][x] = dO[nc][y*R + i][x*R + j],
+// b = i*R + j.  One thread per (nc, y, x): it reads R runs of R neighbouring
+// elements and writes one element to each of the R*R lattices (neighbouring
+// lanes write neighbouring elements).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void k_up_split(const T *__restrict__ go,
+                                                       T *__restrict__ lat, int64_t planes, int H,
+                                                       int W, int R) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t plane = (int64_t)H * W;
+    if (idx >= planes * plane) return;
+    const int64_t nc = idx / plane;
+    const int pix = (int)(idx - nc * plane);
+    const int y = pix / W, x = pix - y * W;
+    const T *src = go + (nc * H * R + (int64_t)y * R) * W * R + (int64_t)x * R;
+    for (int i = 0; i < R; ++i)
+        for (int j = 0; j < R; ++j)
+            lat[(int64_t)(i * R + j) * planes * plane + idx] = src[(int64_t)i * W * R + j];
+}
+
+// out[e] = sum over `parts` tensors of `count` elements stored back to back.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void k_up_sum(const T *__restrict__ in,
+                                                     T *__restrict__ out, int64_t count,
+                                                     int parts) {
+    using A = typename Acc<T>::type;
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= count) return;
+    A acc = 0;
+    for (int b = 0; b < parts; ++b) acc += (A)ld(in + (int64_t)b * count + idx);
+    st(out + idx, acc);
+}
+
 }  // namespace
+
+template <typename T>
+hipError_t up_split_lattices(const T *go, T *lat, int64_t planes, int64_t H, int64_t W, int scale,
+                             hipStream_t stream) {
+    const int64_t total = planes * H * W;
+    if (total == 0) return hipSuccess;
+    const int64_t grid = cdiv(total, kThreads);
+    if (grid > 2147483647) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((k_up_split<T>), dim3((unsigned)grid), dim3(kThreads), 0, stream, go, lat,
+                       planes, (int)H, (int)W, scale);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t up_sum_parts(const T *in, T *out, int64_t count, int parts, hipStream_t stream) {
+    if (count == 0) return hipSuccess;
+    const int64_t grid = cdiv(count, kThreads);
+    if (grid > 2147483647) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((k_up_sum<T>), dim3((unsigned)grid), dim3(kThreads), 0, stream, in, out,
+                       count, parts);
+    return hipGetLastError();
+}
 
 bool up_forward_supported(int64_t H, int64_t W, int k, int d, int scale) {
     if (H * W > (int64_t)1 << 30) return false;   // 32-bit offsets inside a plane
@@ -282,7 +335,10 @@ hipError_t up_forward(int64_t N, int64_t C, int64_t H, int64_t W, int k, int d, 
 #define DDF_UP_INSTANCE(T)                                                                      \
     template hipError_t up_forward<T>(int64_t, int64_t, int64_t, int64_t, int, int, int, bool,  \
                                       const T *, const void *const *, const void *const *, T *, \
-                                      hipStream_t);
+                                      hipStream_t);                                             \
+    template hipError_t up_split_lattices<T>(const T *, T *, int64_t, int64_t, int64_t, int,    \
+                                             hipStream_t);                                      \
+    template hipError_t up_sum_parts<T>(const T *, T *, int64_t, int, hipStream_t);
 DDF_UP_INSTANCE(__half)
 DDF_UP_INSTANCE(float)
 DDF_UP_INSTANCE(double)

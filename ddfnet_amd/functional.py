@@ -189,9 +189,9 @@ class DDFUpFunction(Function):
     of ``DDFUpPack.forward`` (``ddf/ddf.py:264-272``) as one operator.
 
     The forward is one launch that reads the features once and writes the
-    (N, C, H*scale, W*scale) result in place.  The backward splits the incoming
-    gradient into its ``scale*scale`` sub-pixel lattices with one copy and runs
-    the ``ddf`` backward kernels per branch; dX is their sum.
+    (N, C, H*scale, W*scale) result in place.  The backward is one library call
+    that splits the incoming gradient into its ``scale*scale`` sub-pixel
+    lattices, runs the ``ddf`` backward kernels per branch and sums their dX.
     """
 
     @staticmethod
@@ -235,31 +235,18 @@ class DDFUpFunction(Function):
     def backward(ctx, grad_output):
         saved = ctx.saved_tensors
         features, filters = saved[0], saved[1:]
-        r, k = ctx.scale, ctx.kernel_size
+        r = ctx.scale
         branches = r * r
-        b, c, h, w = features.size()
-        # (b, c, h, r, w, r) -> (r, r, b, c, h, w): lattice (i, j) becomes contiguous
-        lattices = grad_output.to(features.dtype).reshape(b, c, h, r, w, r) \
-            .permute(3, 5, 0, 1, 2, 4).contiguous()
-        want_x = ctx.needs_input_grad[0]
+        cfs, sfs = filters[:branches], filters[branches:]
+        grad_output = grad_output.to(features.dtype).contiguous()
         want_f = ctx.needs_input_grad[5:]
-        op = OP_DICT[ctx.op_type]
-        grad_x = None
-        grad_filters = [None] * (2 * branches)
-        for br in range(branches):
-            want_cf, want_sf = want_f[br], want_f[branches + br]
-            if not (want_x or want_cf or want_sf):
-                continue
-            cf, sf = filters[br], filters[branches + br]
-            dx = torch.empty_like(features) if want_x else None
-            dcf = torch.empty_like(cf) if want_cf else None
-            dsf = torch.empty_like(sf) if want_sf else None
-            op.backward(lattices[br // r, br % r], features, cf, sf, k, ctx.dilation, 1,
-                        None, None, None, dx, dcf, dsf)
-            grad_filters[br], grad_filters[branches + br] = dcf, dsf
-            if want_x:
-                grad_x = dx if grad_x is None else grad_x.add_(dx)
-        return (grad_x, None, None, None, None) + tuple(grad_filters)
+        grad_x = torch.empty_like(features) if ctx.needs_input_grad[0] else None
+        grad_cfs = [torch.empty_like(t) if w else None for t, w in zip(cfs, want_f[:branches])]
+        grad_sfs = [torch.empty_like(t) if w else None for t, w in zip(sfs, want_f[branches:])]
+        with _lib.on_device_of(features):
+            _lib.up_backward(grad_output, features, cfs, sfs, grad_x, grad_cfs, grad_sfs,
+                             ctx.kernel_size, ctx.dilation, r, ctx.op_type)
+        return (grad_x, None, None, None, None) + tuple(grad_cfs) + tuple(grad_sfs)
 
 
 def ddf_up(features, channel_filters, spatial_filters, kernel_size=3, dilation=1,

@@ -171,7 +171,7 @@ int ddf_hip_filter_norm_backward(const void *grad_y, const void *x,
  * pointers, each a dense (N, C, k, k) resp. (N, k*k, H, W) tensor; `output`
  * is dense (N, C, H*scale, W*scale).  Covered: k = 1 or 3 with scale 2..4 and
  * k = 5 with scale 2; anything else returns DDF_ERR_UNSUPPORTED and the caller
- * composes the result from ddf_hip_forward.  Forward only.
+ * composes the result from ddf_hip_forward.
  */
 #define DDF_UP_MAX_BRANCHES 16
 int ddf_hip_up_forward(const void *features,
@@ -180,6 +180,35 @@ int ddf_hip_up_forward(const void *features,
                        int64_t N, int64_t C, int64_t H, int64_t W,
                        int kernel_size, int dilation, int scale, int combine,
                        int dtype, void *stream);
+
+/*
+ * Backward of ddf_hip_up_forward: what autograd derives in the reference from
+ * F.pixel_shuffle, torch.stack and the scale*scale `ddf` calls of
+ * DDFUpPack.forward (ddf/ddf.py:264-272), done inside the library: the
+ * gradient is split into its sub-pixel lattices (one launch), every branch
+ * runs the kernels of ddf_hip_backward on its lattice, and the branches'
+ * feature gradients are summed (one launch).  `grad_output` is dense
+ * (N, C, H*scale, W*scale); `grad_channel_filters` / `grad_spatial_filters`
+ * are host arrays of scale*scale device pointers (an array, or single
+ * entries of it, may be NULL: that gradient is not computed); `need_mask` as
+ * in ddf_hip_backward.  Any odd kernel_size; scale 2..4.  `workspace` must
+ * hold ddf_hip_up_backward_workspace_bytes(...) bytes, 256-byte aligned.
+ */
+size_t ddf_hip_up_backward_workspace_bytes(int64_t N, int64_t C, int64_t H,
+                                           int64_t W, int kernel_size,
+                                           int dilation, int scale,
+                                           int combine, int dtype,
+                                           unsigned need_mask);
+int ddf_hip_up_backward(const void *grad_output, const void *features,
+                        const void *const *channel_filters,
+                        const void *const *spatial_filters,
+                        void *grad_features,
+                        void *const *grad_channel_filters,
+                        void *const *grad_spatial_filters, void *workspace,
+                        size_t workspace_bytes, int64_t N, int64_t C,
+                        int64_t H, int64_t W, int kernel_size, int dilation,
+                        int scale, int combine, int dtype, unsigned need_mask,
+                        void *stream);
 
 #ifdef __cplusplus
 }

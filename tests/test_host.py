@@ -206,6 +206,28 @@ def test_up_forward_argument_validation_needs_no_gpu():
     assert _lib.up_forward_covers(3, 2) and not _lib.up_forward_covers(7, 2)
 
 
+def test_up_backward_validation_and_workspace_need_no_gpu():
+    import ctypes
+    lib = _lib.lib()
+    none = (ctypes.c_void_p * 16)()
+    bwd, size = lib.ddf_hip_up_backward, lib.ddf_hip_up_backward_workspace_bytes
+    args = (1, 1, 4, 4, 3, 1)
+    assert bwd(None, None, none, none, None, none, none, None, 0, *args, 1, 0, 1, 7, None) == 1
+    assert b'scale' in lib.ddf_hip_last_error()
+    assert bwd(None, None, none, none, None, none, none, None, 0, *args, 2, 0, 1, 0, None) == 0
+    assert bwd(None, None, none, none, None, none, none, None, 0, *args, 2, 0, 1, 7, None) == 1
+    assert b'null' in lib.ddf_hip_last_error()
+    # lattices and per-branch dX of 4 branches, each padded to 256 bytes, plus
+    # the workspace of one 3x3 stride-1 branch (none at this size)
+    n_x = 2 * 8 * 6 * 6 * 4
+    pad = lambda v: (v + 255) // 256 * 256
+    branch = lib.ddf_hip_backward_workspace_bytes(2, 8, 6, 6, 3, 1, 1, 0, 1, 7, 0)
+    assert size(2, 8, 6, 6, 3, 1, 2, 0, 1, 7) == 2 * pad(4 * n_x) + pad(branch)
+    assert size(2, 8, 6, 6, 3, 1, 2, 0, 1, 6) == pad(4 * n_x) + pad(
+        lib.ddf_hip_backward_workspace_bytes(2, 8, 6, 6, 3, 1, 1, 0, 1, 6, 0))
+    assert size(2, 8, 6, 6, 3, 1, 1, 0, 1, 7) == 0
+
+
 def _load_bench():
     import importlib.util
     spec = importlib.util.spec_from_file_location('ddf_bench', os.path.join(ROOT, 'bench.py'))
