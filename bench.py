@@ -58,6 +58,8 @@ STEP_PHASES = ('fwd', 'bwd')
 # writes the feature gradient); otherwise bwd = the dx call + the dfilters call.
 PHASE_KERNELS = {
     'fwd': 'ddf::wave::k_forward',
+    # one fused launch where a plane fits one 16-byte vector per lane (3x3,
+    # stride 1, up to about 16x16), else feature and filter gradients apart
     'bwd': 'ddf::wave::k_backward_filters<DX=true> + ddf::wave::k_sum_partials',
     'dx': 'ddf::wave::k_backward_features',
     'dfilters': 'ddf::wave::k_backward_filters<DX=false> + ddf::wave::k_sum_partials',
@@ -179,7 +181,12 @@ def timed(fn, count):
 # reports null.
 MEASURED_TRAFFIC = {
     'r50_stage3_mul_fp32': {'fwd': 27760539, 'bwd': 49286424, 'dx': 27762539, 'dfilters': 35535013},
+    'r50_stage1_add_fp16': {'fwd': 56477696, 'bwd': 116746240, 'dx': 56538112, 'dfilters': 60208128},
 }
+# kernels behind the backward call where the fused kernel does not apply
+UNFUSED_BWD = ('ddf::wave::k_backward_features + ddf::wave::k_backward_filters<DX=false> + '
+               'ddf::wave::k_sum_partials')
+FUSED_BWD_WORKLOADS = ('r50_stage3_mul_fp32',)
 
 
 def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
@@ -417,6 +424,9 @@ def main():
     dom_bytes = res['bytes'][dominant]
     dom_s = res['phase_ms'][dominant] * 1e-3
     achieved = dom_bytes / dom_s / 1e9
+    kernel_label = PHASE_KERNELS[dominant]
+    if dominant == 'bwd' and res['workload'] not in FUSED_BWD_WORKLOADS:
+        kernel_label = UNFUSED_BWD
     line = {
         'metric': 'ddf_fwd_bwd_hbm_gbps', 'value': round(res['gbps'], 2), 'unit': 'GB/s',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -429,7 +439,7 @@ def main():
             'buffer_sets': res['buffer_sets']},
         'pct_of_hbm_peak': round(100 * res['gbps'] / HBM_PEAK_GBPS, 2),
         'images_per_s': round(res['images_per_s'], 1),
-        'roofline': {'bound': 'hbm', 'phase': dominant, 'kernel': PHASE_KERNELS[dominant], 'achieved': round(achieved, 2),
+        'roofline': {'bound': 'hbm', 'phase': dominant, 'kernel': kernel_label, 'achieved': round(achieved, 2),
                      'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
                      'frac': round(achieved / HBM_PEAK_GBPS, 4),
                      'traffic': MEASURED_TRAFFIC.get(res['workload'], {}).get(dominant),
