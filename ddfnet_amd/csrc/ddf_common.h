@@ -88,6 +88,14 @@ hipError_t up_split_lattices(const T *go, T *lat, int64_t planes, int64_t H, int
 template <typename T>
 hipError_t up_sum_parts(const T *in, T *out, int64_t count, int parts, hipStream_t st);
 
+// Tiny planes (H*W <= 64), 3x3, stride 1: forward (backward = false: x -> out)
+// and feature gradient (backward = true: dO -> dX), G = 256 / (H*W) channel
+// planes per workgroup pass.
+bool small_supported(const Problem &p);
+template <typename T>
+hipError_t small_launch(const Problem &p, bool backward, const T *x, const T *cf, const T *sf,
+                        T *out, hipStream_t st);
+
 bool tiled_forward_supported(const Problem &p, int dtype);
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,

@@ -153,6 +153,7 @@ bool wave_plan(const Problem &p, int kind, std::initializer_list<const void *> p
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf, T *out,
                          hipStream_t st) {
+    if (small_supported(p)) return small_launch<T>(p, false, x, cf, sf, out, st);
     WaveGeom g; int ps, nv;
     if (!wave_plan<T>(p, kWaveForward, {x, sf, out}, &g, &ps, &nv))
         return generic_forward<T>(p, x, cf, sf, out, st);   // e.g. pointers not 16-byte aligned
@@ -178,7 +179,9 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
                gp.csplit == g.csplit;
     }
     if ((need & DDF_NEED_DX) && !fuse) {
-        if (!wave_plan<T>(p, kWaveFeatures, {go, sf, dx}, &g, &ps, &nv)) {
+        if (small_supported(p)) {
+            err = small_launch<T>(p, true, go, cf, sf, dx, st);
+        } else if (!wave_plan<T>(p, kWaveFeatures, {go, sf, dx}, &g, &ps, &nv)) {
             err = generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, DDF_NEED_DX, st);
         } else {
             DDF_DISPATCH_KDS(p, err = tiled::launch_features<T, KK_, DD_, SS_>(p, g, ps, nv, go, cf, sf, dx, st));

@@ -510,3 +510,19 @@ def test_tensors_beyond_2_31_elements():
     want = oracle.forward(xs[:, sl].detach().cpu(), cfs[:, sl].detach().cpu(), sfs.detach().cpu(),
                           3, 1, 1, 'mul')
     assert rel_err(outs[:, sl], want) <= TOL[torch.float16]
+
+
+@pytest.mark.parametrize('dtype', [torch.float64, torch.float32, torch.float16])
+@pytest.mark.parametrize('N,C,H,W,d,combine', [
+    (3, 37, 7, 7, 1, 'mul'),     # 5 channel planes per workgroup pass, ragged channel count
+    (2, 130, 7, 7, 2, 'add'),    # taps staged in two rounds
+    (1, 3, 8, 8, 1, 'mul'),      # fewer channels than plane slots
+    (2, 19, 3, 20, 2, 'mul'), (2, 19, 20, 3, 1, 'add'),
+    (1, 300, 1, 1, 1, 'mul'), (2, 9, 1, 64, 1, 'mul'), (4, 64, 4, 4, 1, 'mul'),
+])
+def test_tiny_planes(N, C, H, W, d, combine, dtype):
+    """Planes of at most 64 pixels take the kernels that pack several channel
+    planes into one workgroup pass (forward and feature gradient)."""
+    case = random_case(N, C, H, W, 3, 1, dtype, seed=N + C)
+    check_against_oracle(*case, 3, d, 1, combine, '', what='tiny plane')
+    check_against_oracle(*case, 3, d, 1, combine, 'f', what='tiny plane, tiled forced')
