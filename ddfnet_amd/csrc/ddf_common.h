@@ -96,6 +96,22 @@ template <typename T>
 hipError_t small_launch(const Problem &p, bool backward, const T *x, const T *cf, const T *sf,
                         T *out, hipStream_t st);
 
+// Row-register kernels (stride 1; rows that are a whole number of vectors):
+// forward (backward = false: x -> out) or feature gradient (backward = true:
+// dO -> dX).  hipErrorNotSupported when the family does not cover the problem
+// or a pointer is not aligned to its vectors; nothing was launched then.
+template <typename T>
+hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf, const T *sf,
+                       T *out, hipStream_t st);
+
+// Filter gradients (dCF, dSF) on the row-register kernel; same conventions.
+// The workspace (rows_filters_workspace bytes, 256-byte aligned) holds the
+// partial sums over channel splits and strips.
+size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);
+template <typename T>
+hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
+                               T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st);
+
 bool tiled_forward_supported(const Problem &p, int dtype);
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,

@@ -1,0 +1,453 @@
+// Row-register DDF kernels for gfx950 (stride 1): forward and feature gradient.
+//
+// A lane owns R consecutive rows of VX neighbouring pixels (one 16-, 8- or 4-byte
+// vector per row) of one sample and walks a range of channels.  Nothing of the
+// feature map goes through LDS:
+//   * the R + 2*HY rows a lane needs per channel (its own and the HY = (K/2)*D
+//     rows above and below) come straight from global memory as whole vectors,
+//     a few channels ahead of use; the rows shared with the lanes above and
+//     below are served by the cache;
+//   * every plane is addressed through a buffer descriptor that covers exactly
+//     that plane, so a row above or below the image, the vector of an idle lane
+//     and the channels past a wave's last one are simply given an offset
+//     outside the descriptor: such loads return zero and such stores are
+//     dropped by the memory unit - the zero padding of the operator costs no
+//     instruction and the kernels contain no bounds branch;
+//   * the HX = (K/2)*D pixels left and right of a vector are the edge words of
+//     the neighbouring lanes' vectors, fetched with one wavefront shift (DPP)
+//     per word.  Lanes are laid out over a strip as (row group, vector) with
+//     lpr = W / VX lanes per image row; where it costs no row group, an idle
+//     lane (whose loads return zero) separates consecutive image rows, and the
+//     shift brings in the zero padding by itself; otherwise the lanes at the
+//     ends of an image row select zero;
+//   * the K*K spatial-filter taps of the lane's R*VX pixels stay in registers
+//     for the whole channel walk, in storage format (fp16 stays packed);
+//   * the K*K channel-filter taps of a channel come in through the scalar unit
+//     (fp32, fp64) or are loaded by lanes 0..K*K-1 and broadcast (fp16).
+//
+// The feature gradient is the same walk over dO with flipped taps,
+//   dX[p] = sum_t dO[p - o_t] * comb(CF[t], SF[t, p - o_t]),
+// so the only difference is the prologue: the spatial taps a lane keeps are
+// those of the pixels its dO values come from (rows fetched at the tap's row
+// offset, columns shifted by the same wavefront shifts, zero outside the
+// image).  Reference kernels computing the same sums:
+// ddf/src/cuda/ddf_mul_cuda_kernel.cu:85-165 (forward), :198-290 (feature
+// gradient), ddf_mul_faster_cuda_kernel.cu:47-163.
+#pragma once
+
+#include <type_traits>
+
+#include "ddf_common.h"
+
+namespace ddf {
+
+struct RowsGeom {
+    int C, H, W;              // per sample (stride 1: the result plane has the same shape)
+    int lpr, rg;              // lanes per image row, row groups per wave
+    int lp;                   // lane pitch of a row group: lpr, or lpr + 1 (an idle lane after each row)
+    unsigned lp_magic;        // ceil(2^32 / lp), 0 when lp == 1
+    int rps, nstrips;         // rows per strip (= rg * R), strips per plane
+    int cpw, cpb, csplit;     // channels per wave and per work item; channel ranges per plane
+    int wpb;                  // work items (independent waves) per workgroup
+    int nwork;                // N * nstrips * csplit wave-sized work items
+    unsigned csplit_magic, nstrips_magic, xcd_per;
+};
+
+namespace rows {
+
+constexpr int kXcd = 8;
+constexpr int kMaxWpb = 4;
+
+// q = n / d through the host's magic number m = ceil(2^32 / d) (0: d == 1);
+// exact while n * d < 2^32.
+__host__ __device__ __forceinline__ int magic_div(int n, unsigned m) {
+    return m ? (int)(((unsigned long long)(unsigned)n * m) >> 32) : n;
+}
+
+// Which strip of which sample and which channel range a wave works on.
+// Workgroups are handed to the 8 XCDs round-robin; they are renumbered so that
+// consecutive work items (same sample, neighbouring channel ranges and strips)
+// share an XCD and its L2.
+struct Work {
+    int cs, strip, c_begin, c_end;
+    int64_t n;
+    __host__ __device__ __forceinline__ bool init(const RowsGeom &g, int block, int wave) {
+        const int wg = (block % kXcd) * (int)g.xcd_per + block / kXcd;
+        const int b = wg * g.wpb + wave;
+        if (wave >= g.wpb || b >= g.nwork) return false;
+        const int rest = magic_div(b, g.csplit_magic);
+        cs = b - rest * g.csplit;
+        const int smp = magic_div(rest, g.nstrips_magic);
+        strip = rest - smp * g.nstrips;
+        n = smp;
+        c_begin = cs * g.cpb;
+        c_end = c_begin + g.cpb < g.C ? c_begin + g.cpb : g.C;
+        return true;
+    }
+};
+
+// Where a lane's rows are.  Shared by the kernels and by the host-side bounds
+// model, which replays it for every lane.
+//   xoff[rr]: element offset inside a plane of the lane's vector in window row
+//             rr (rr = 0 is HY rows above the lane's first row), or -1 when the
+//             row lies outside the image or the lane is idle;
+//   ooff[r]:  the same for the R result rows.
+template <int R, int HY, int VX>
+struct Lane {
+    static constexpr int ROWS = R + 2 * HY;
+    bool first, last;         // at the ends of an image row
+    int xoff[ROWS];
+    int ooff[R];
+    __host__ __device__ __forceinline__ void init(const RowsGeom &g, int strip, int lane) {
+        const int grp = magic_div(lane, g.lp_magic);
+        const int v = lane - grp * g.lp;
+        const bool live = grp < g.rg && v < g.lpr;
+        const int x0 = v * VX;
+        const int y0 = strip * g.rps + grp * R;
+        first = v == 0;
+        last = v == g.lpr - 1;
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) {
+            const int yy = y0 - HY + rr;
+            xoff[rr] = (live && yy >= 0 && yy < g.H) ? yy * g.W + x0 : -1;
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) ooff[r] = xoff[HY + r];
+    }
+};
+
+#ifdef __HIPCC__
+
+// Byte offset no plane reaches (planes are below 2^31 bytes): a buffer access
+// at this offset is out of range whatever it is added to.
+constexpr uint32_t kOutside = 0x80000000u;
+
+// Buffer descriptor over `bytes` bytes at p (raw buffer, no stride): accesses at
+// offsets >= bytes read as zero and are not written.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t plane_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+
+template <int N>
+__device__ __forceinline__ void load_words(__amdgpu_buffer_rsrc_t rsrc, uint32_t off, uint32_t (&w)[N]) {
+    if constexpr (N == 1) {
+        w[0] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)off, 0, 0);
+    } else if constexpr (N == 2) {
+        const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)off, 0, 0);
+        w[0] = v[0]; w[1] = v[1];
+    } else {
+        static_assert(N == 4, "vectors of 4, 8 or 16 bytes");
+        const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) w[k] = v[k];
+    }
+}
+
+// Nontemporal: results are not read again by this kernel.
+template <int N>
+__device__ __forceinline__ void store_words_nt(__amdgpu_buffer_rsrc_t rsrc, uint32_t off, const uint32_t (&w)[N]) {
+    if constexpr (N == 1) {
+        __builtin_amdgcn_raw_buffer_store_b32(w[0], rsrc, (int)off, 0, 2);
+    } else if constexpr (N == 2) {
+        typedef uint32_t v2 __attribute__((ext_vector_type(2)));
+        v2 v = {w[0], w[1]};
+        __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, (int)off, 0, 2);
+    } else {
+        static_assert(N == 4, "vectors of 4, 8 or 16 bytes");
+        typedef uint32_t v4 __attribute__((ext_vector_type(4)));
+        v4 v = {w[0], w[1], w[2], w[3]};
+        __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)off, 0, 2);
+    }
+}
+
+// Element e of a run of storage-type values held in 32-bit words, widened to
+// the accumulator type.  (e is a constant wherever this is called: every loop
+// around it is unrolled.)
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+template <typename T>
+__device__ __forceinline__ typename Acc<T>::type elem(const uint32_t *w, int e) {
+    if constexpr (sizeof(T) == 2) {
+        const half2_t h = __builtin_bit_cast(half2_t, w[e / 2]);
+        return (float)((e & 1) ? h[1] : h[0]);
+    } else if constexpr (sizeof(T) == 4) {
+        return __uint_as_float(w[e]);
+    } else {
+        return __hiloint2double((int)w[2 * e + 1], (int)w[2 * e]);
+    }
+}
+
+// VX accumulator-type values -> storage-type words (round to nearest even).
+template <typename T, int VX, typename A>
+__device__ __forceinline__ void pack(const A (&v)[VX], uint32_t (&w)[VX * sizeof(T) / 4]) {
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+        for (int k = 0; k < VX / 2; ++k) {
+            half2_t h;
+            h[0] = (_Float16)v[2 * k];
+            h[1] = (_Float16)v[2 * k + 1];
+            w[k] = __builtin_bit_cast(uint32_t, h);
+        }
+    } else if constexpr (sizeof(T) == 4) {
+#pragma unroll
+        for (int k = 0; k < VX; ++k) w[k] = __float_as_uint(v[k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < VX; ++k) {
+            w[2 * k] = (uint32_t)__double2loint(v[k]);
+            w[2 * k + 1] = (uint32_t)__double2hiint(v[k]);
+        }
+    }
+}
+
+// Whole-wavefront shifts of one register: lane l receives lane l-1's (from_left)
+// or lane l+1's value; the lane without a source receives 0.
+__device__ __forceinline__ uint32_t from_left(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x138 /* wave_shr:1 */, 0xf, 0xf, true);
+}
+__device__ __forceinline__ uint32_t from_right(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x130 /* wave_shl:1 */, 0xf, 0xf, true);
+}
+
+__device__ __forceinline__ float fma_(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+// One image row as a lane sees it: its own VX elements plus HX elements of the
+// lanes to its left and right (zero beyond the ends of the image row).
+// PAD: an idle lane holding zeros follows every image row, so the shifted-in
+// words are already right; otherwise the lanes at the row ends select zero.
+template <typename T, int VX, int HX, bool PAD>
+struct ExtRow {
+    using A = typename Acc<T>::type;
+    static constexpr int NW = VX * sizeof(T) / 4;
+    static constexpr int SW = HX == 0 ? 1 : (HX * sizeof(T) + 3) / 4;   // words taken from each neighbour
+    static constexpr int kLeftFirst = (NW - SW) * 4 / (int)sizeof(T);   // neighbour element in left[0]
+    static_assert(HX <= VX, "taps reach beyond the neighbouring lane");
+    uint32_t own[NW], left[SW], right[SW];
+    __device__ __forceinline__ void sides(bool first, bool last) {
+        if constexpr (HX > 0) {
+#pragma unroll
+            for (int k = 0; k < SW; ++k) {
+                const uint32_t l = from_left(own[NW - SW + k]);
+                const uint32_t r = from_right(own[k]);
+                left[k] = PAD ? l : (first ? 0u : l);
+                right[k] = PAD ? r : (last ? 0u : r);
+            }
+        }
+    }
+    // element at column e relative to the lane's first pixel, e in [-HX, VX + HX)
+    __device__ __forceinline__ A at(int e) const {
+        if (e < 0) return elem<T>(left, VX + e - kLeftFirst);
+        if (e >= VX) return elem<T>(right, e - VX);
+        return elem<T>(own, e);
+    }
+};
+
+template <typename A>
+__device__ __forceinline__ A lane_broadcast(A v, int src_lane);
+template <>
+__device__ __forceinline__ float lane_broadcast<float>(float v, int src_lane) {
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), src_lane));
+}
+template <>
+__device__ __forceinline__ double lane_broadcast<double>(double v, int src_lane) {
+    const int lo = __builtin_amdgcn_readlane(__double2loint(v), src_lane);
+    const int hi = __builtin_amdgcn_readlane(__double2hiint(v), src_lane);
+    return __hiloint2double(hi, lo);
+}
+
+// BWD = false: out = forward(x, cf, sf).  BWD = true: x is dO and out is dX.
+// WPE: waves per SIMD the register allocation must leave room for.
+template <typename T, int K, int D, bool MUL, bool BWD, int VX, int R, bool PAD, int NST, int WPE>
+__global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const T *__restrict__ x,
+                                                         const T *__restrict__ cf,
+                                                         const T *__restrict__ sf,
+                                                         T *__restrict__ out) {
+    using A = typename Acc<T>::type;
+    constexpr int KK = K * K, RAD = K / 2, HX = RAD * D, HY = RAD * D;
+    constexpr int ROWS = R + 2 * HY;
+    constexpr int NW = VX * sizeof(T) / 4;
+    using Row = ExtRow<T, VX, HX, PAD>;
+    static_assert(KK <= kWave, "one lane per channel-filter tap");
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    Work wk;
+    if (!wk.init(g, blockIdx.x, wave) || wk.c_end <= wk.c_begin) return;
+    const int nch = wk.c_end - wk.c_begin;
+    const int64_t plane = (int64_t)g.H * g.W;
+    const uint32_t plane_bytes = (uint32_t)plane * (uint32_t)sizeof(T);
+    Lane<R, HY, VX> ln;
+    ln.init(g, wk.strip, lane);
+
+    const T *xs = x + (wk.n * g.C + wk.c_begin) * plane;
+    T *os = out + (wk.n * g.C + wk.c_begin) * plane;
+    // byte offsets of the lane's vectors inside a plane; kOutside: reads as zero, is not written
+    uint32_t xb[ROWS], ob[R];
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr)
+        xb[rr] = ln.xoff[rr] < 0 ? kOutside : (uint32_t)ln.xoff[rr] * (uint32_t)sizeof(T);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        ob[r] = ln.ooff[r] < 0 ? kOutside : (uint32_t)ln.ooff[r] * (uint32_t)sizeof(T);
+    const T *cfs = cf + (wk.n * g.C + wk.c_begin) * KK;
+    constexpr bool kScalarTaps = sizeof(T) >= 4;
+    const int tl = lane < KK ? lane : KK - 1;   // lane t holds tap t of a channel (flipped for the gradient)
+    const int tsel = BWD ? KK - 1 - tl : tl;
+
+    // feature rows and channel taps of channel ci, stage ST; a channel past the
+    // wave's last one reads zeros (empty descriptor)
+    uint32_t xw[NST][ROWS][NW];
+    T cfl[NST];
+    A cfu[NST][kScalarTaps ? KK : 1];
+    auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * plane, ci < nch ? plane_bytes : 0u);
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) load_words<NW>(pr, xb[rr], xw[ST][rr]);
+        const int cc = ci < nch ? ci : nch - 1;   // (the taps are read through plain pointers: stay inside)
+        if constexpr (kScalarTaps) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) cfu[ST][t] = cfs[(int64_t)cc * KK + (BWD ? KK - 1 - t : t)];
+        } else {
+            cfl[ST] = cfs[(int64_t)cc * KK + tsel];
+        }
+    };
+    issue(std::integral_constant<int, 0>{}, 0);
+    if constexpr (NST > 2) issue(std::integral_constant<int, 1>{}, 1);
+    if constexpr (NST > 3) issue(std::integral_constant<int, 2>{}, 2);
+
+    // Spatial taps of the lane's pixels, in storage format.  Forward: tap t at
+    // the pixel itself.  Gradient: slot (i, j) holds tap (K-1-i, K-1-j) at the
+    // pixel (i-RAD)*D rows and (j-RAD)*D columns away - the pixel whose result
+    // that dO value belongs to - and zero where that pixel does not exist.
+    uint32_t sfw[R][KK][NW];
+    {
+        const T *sfn = sf + wk.n * KK * plane;
+        if constexpr (!BWD) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) {
+                const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
+#pragma unroll
+                for (int r = 0; r < R; ++r) load_words<NW>(sr, ob[r], sfw[r][t]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const __amdgpu_buffer_rsrc_t sr =
+                        plane_rsrc(sfn + ((K - 1 - i) * K + (K - 1 - j)) * plane, plane_bytes);
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        Row row;
+                        load_words<NW>(sr, xb[r + i * D], row.own);
+                        row.sides(ln.first, ln.last);
+                        A v[VX];
+#pragma unroll
+                        for (int e = 0; e < VX; ++e) v[e] = row.at(e + j * D - HX);
+                        pack<T, VX, A>(v, sfw[r][i * K + j]);
+                    }
+                }
+        }
+    }
+
+    auto compute = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        if constexpr (sizeof(T) == 2) {
+            // Keeps the packed taps packed: without this the compiler widens all
+            // of them to fp32 ahead of the channel loop, twice the registers.
+            // Widened at their one use per channel they fold into the
+            // mixed-precision multiply-add at no cost.
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < KK; ++t)
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfw[r][t][k]));
+        }
+        Row row[ROWS];
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) {
+#pragma unroll
+            for (int k = 0; k < NW; ++k) row[rr].own[k] = xw[ST][rr][k];
+            row[rr].sides(ln.first, ln.last);
+        }
+        A w[KK];
+        if constexpr (kScalarTaps) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) w[t] = cfu[ST][t];
+        } else {
+            const A cfa = (A)ld(&cfl[ST]);
+#pragma unroll
+            for (int t = 0; t < KK; ++t) w[t] = lane_broadcast<A>(cfa, t);
+        }
+        A acc[R][VX];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int e = 0; e < VX; ++e) acc[r][e] = 0;
+        // mul: x * sf is exact in the accumulator type for fp16 storage and goes
+        // into one mixed-precision multiply; add: two multiply-adds
+#pragma unroll
+        for (int i = 0; i < K; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j)
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) {
+                        const A xv = row[r + i * D].at(e + j * D - HX);
+                        const A sv = elem<T>(sfw[r][i * K + j], e);
+                        if constexpr (MUL) {
+                            acc[r][e] = fma_(w[i * K + j], fma_(xv, sv, A(0)), acc[r][e]);
+                        } else {
+                            acc[r][e] = fma_(xv, w[i * K + j], acc[r][e]);
+                            acc[r][e] = fma_(xv, sv, acc[r][e]);
+                        }
+                    }
+        const __amdgpu_buffer_rsrc_t orr = plane_rsrc(os + (int64_t)ci * plane, ci < nch ? plane_bytes : 0u);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            if constexpr (sizeof(T) == 2) {
+                // The sum is complete in fp32 before it is rounded to fp16.  Left
+                // alone, the compiler fuses the last multiply-add with the rounding
+                // in some unrolled copies of this code and not in others, and a
+                // result would then depend on which copy its channel falls to.
+#pragma unroll
+                for (int e = 0; e < VX; ++e) asm volatile("" : "+v"(acc[r][e]));
+            }
+            uint32_t ow[NW];
+            pack<T, VX, A>(acc[r], ow);
+            store_words_nt<NW>(orr, ob[r], ow);
+        }
+    };
+
+    // Channel ci is computed from stage ci % NST while the loads of channel
+    // ci + NST - 1 go out.  The walk is unrolled NST times so that stages are
+    // compile-time register sets; it always runs whole rounds of NST channels
+    // (one basic block, no tail code): a channel past the wave's last one is
+    // computed from zeros and its stores are dropped.
+    auto step = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        issue(std::integral_constant<int, (ST + NST - 1) % NST>{}, ci + NST - 1);
+        compute(st_tag, ci);
+    };
+    for (int ci = 0; ci < nch; ci += NST) {
+        step(std::integral_constant<int, 0>{}, ci);
+        if constexpr (NST > 1) step(std::integral_constant<int, 1>{}, ci + 1);
+        if constexpr (NST > 2) step(std::integral_constant<int, 2>{}, ci + 2);
+        if constexpr (NST > 3) step(std::integral_constant<int, 3>{}, ci + 3);
+    }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace rows
+
+// Host-side geometry (ddf_rows_host.hip).  Fills *g and names the kernel
+// instantiation (*vx elements per lane and row, *r rows per lane; g->lp >
+// g->lpr selects the PAD kernels); false when the family does not cover the
+// problem.
+bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx, int *r);
+
+}  // namespace ddf

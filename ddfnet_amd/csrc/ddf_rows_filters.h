@@ -1,0 +1,320 @@
+// Row-register filter-gradient kernel for gfx950 (stride 1): dCF and dSF in one
+// walk, same lane layout and feature-row handling as ddf_rows.h.
+//
+// The kFilterWaves waves of a workgroup work on the same strip of the same
+// sample and walk consecutive channel ranges of g.cpw channels each.  Per
+// channel a lane forms gx[t] = dO * X_t for its R*VX pixels once and feeds it
+// to both sums:
+//   dSF[t, pixel] += gx[t] * CF[c, t]      register accumulators over the walk
+//   dCF[c, t]      = sum over pixels of gx[t] * SF[t, pixel]
+// ('add' combine: both are sums of gx[t] itself.)  The per-lane dCF partials
+// of kFlushChannels channels are parked in LDS, lane-contiguous per (channel,
+// tap); then one lane per (channel, tap) adds up the 64 lane values with
+// 16-byte reads.  That costs a quarter of the vector instructions of a
+// cross-lane butterfly per channel, and the LDS pipe is otherwise idle here.
+// After the walk the waves add their dSF accumulators through LDS (the only
+// workgroup barriers).  Partial sums over channel splits (dSF) and strips
+// (dCF) go to the workspace; no atomics, so results are reproducible.
+// Reference kernels computing the same sums:
+// ddf/src/cuda/ddf_mul_cuda_kernel.cu:293-355 (spatial filter), :358-420
+// (channel filter).
+#pragma once
+
+#include "ddf_rows.h"
+
+namespace ddf {
+namespace rows {
+
+constexpr int kFilterWaves = 4;
+constexpr int kFlushChannels = 4;   // power of two
+constexpr int kRedPitch = 68;       // accumulator values per (channel, tap) row: 64 lanes + pad, 16-byte rows
+constexpr int kTapChunk = 3;        // taps per round of the final dSF sum
+
+// LDS of one workgroup of k_rows_filters, bytes.
+template <int KK>
+constexpr int filters_lds_bytes(int asz, int r, int vx) {
+    const int flush = kFilterWaves * kFlushChannels * KK * kRedPitch * asz;
+    const int final_sum = kFilterWaves * kTapChunk * r * vx * kWave * asz;
+    return flush > final_sum ? flush : final_sum;
+}
+
+#ifdef __HIPCC__
+
+// Compiler-level ordering point between LDS writes and the reads of other
+// lanes of the same wavefront.  The LDS unit executes one wave's instructions
+// in order, so no hardware wait is needed.
+__device__ __forceinline__ void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <typename T, int K, int D, bool MUL, int VX, int R, bool PAD, int NST, int WPE>
+__global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
+    RowsGeom g, const T *__restrict__ go, const T *__restrict__ x, const T *__restrict__ cf,
+    const T *__restrict__ sf, T *__restrict__ dcf, T *__restrict__ dsf,
+    typename Acc<T>::type *__restrict__ ws_sf, typename Acc<T>::type *__restrict__ ws_cf,
+    unsigned need) {
+    using A = typename Acc<T>::type;
+    constexpr int KK = K * K, RAD = K / 2, HX = RAD * D, HY = RAD * D;
+    constexpr int ROWS = R + 2 * HY;
+    constexpr int NW = VX * sizeof(T) / 4;
+    constexpr int G = kFlushChannels;
+    using Row = ExtRow<T, VX, HX, PAD>;
+    static_assert(G * KK <= kWave, "one lane per (channel, tap) of a flush group");
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    Work wk;
+    if (!wk.init(g, blockIdx.x, 0)) return;   // whole workgroup leaves together
+    const bool want_cf = need & DDF_NEED_DCF, want_sf = need & DDF_NEED_DSF;
+    // this wave's channels inside the workgroup's range
+    const int c0 = min(wk.c_begin + wave * g.cpw, wk.c_end);
+    const int nch = min(g.cpw, wk.c_end - c0);
+    const int c_first = min(c0, g.C - 1);   // (pointers of a wave without channels stay inside)
+    const int64_t plane = (int64_t)g.H * g.W;
+    const uint32_t plane_bytes = (uint32_t)plane * (uint32_t)sizeof(T);
+    Lane<R, HY, VX> ln;
+    ln.init(g, wk.strip, lane);
+
+    const T *xs = x + (wk.n * g.C + c_first) * plane;
+    const T *gs = go + (wk.n * g.C + c_first) * plane;
+    uint32_t xb[ROWS], ob[R];
+#pragma unroll
+    for (int rr = 0; rr < ROWS; ++rr)
+        xb[rr] = ln.xoff[rr] < 0 ? kOutside : (uint32_t)ln.xoff[rr] * (uint32_t)sizeof(T);
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        ob[r] = ln.ooff[r] < 0 ? kOutside : (uint32_t)ln.ooff[r] * (uint32_t)sizeof(T);
+    const int tl = lane < KK ? lane : KK - 1;
+    const T *cfs = cf + (wk.n * g.C + c_first) * KK;
+
+    // Feature rows, dO rows and channel taps of channel ci, stage ST.  A channel
+    // past the wave's last one reads zeros (empty descriptors) and so adds nothing;
+    // idle lanes and rows outside the image read zeros as well.
+    constexpr bool kScalarTaps = sizeof(T) >= 4;   // (see k_rows)
+    uint32_t xw[NST][ROWS][NW], gw[NST][R][NW];
+    T cfl[NST];
+    A cfu[NST][kScalarTaps && MUL ? KK : 1];
+    auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        const uint32_t bytes = ci < nch ? plane_bytes : 0u;
+        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * plane, bytes);
+        const __amdgpu_buffer_rsrc_t gr = plane_rsrc(gs + (int64_t)ci * plane, bytes);
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) load_words<NW>(pr, xb[rr], xw[ST][rr]);
+#pragma unroll
+        for (int r = 0; r < R; ++r) load_words<NW>(gr, ob[r], gw[ST][r]);
+        if constexpr (MUL) {
+            const int cc = ci < nch ? ci : (nch > 0 ? nch - 1 : 0);
+            if constexpr (kScalarTaps) {
+#pragma unroll
+                for (int t = 0; t < KK; ++t) cfu[ST][t] = cfs[(int64_t)cc * KK + t];
+            } else {
+                cfl[ST] = cfs[(int64_t)cc * KK + tl];
+            }
+        }
+    };
+    issue(std::integral_constant<int, 0>{}, 0);
+    if constexpr (NST > 2) issue(std::integral_constant<int, 1>{}, 1);
+    if constexpr (NST > 3) issue(std::integral_constant<int, 2>{}, 2);
+
+    // spatial taps of the lane's pixels (needed for dCF under 'mul' only)
+    uint32_t sfw[MUL ? R : 1][KK][NW];
+    if constexpr (MUL) {
+        const T *sfn = sf + wk.n * KK * plane;
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
+#pragma unroll
+            for (int r = 0; r < R; ++r) load_words<NW>(sr, ob[r], sfw[r][t]);
+        }
+    }
+    A acc_sf[R][KK][VX];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < KK; ++t)
+#pragma unroll
+            for (int e = 0; e < VX; ++e) acc_sf[r][t][e] = 0;
+    A *red = reinterpret_cast<A *>(smem) + (size_t)wave * (G * KK * kRedPitch);
+
+    // Adds up the 64 lane partials of each (channel, tap) of a flush group of
+    // `cnt` channels starting at channel `cbase` of the wave, and stores them.
+    auto flush = [&](int cbase, int cnt) __attribute__((always_inline)) {
+        wave_sync();
+        if (lane < cnt * KK) {
+            const A *rowp = red + lane * kRedPitch;
+            A tot[4] = {0, 0, 0, 0};
+            // (four 16-byte reads in flight at a time: more would cost registers the walk needs)
+#pragma nounroll
+            for (int k0 = 0; k0 < kWave / 4; k0 += 4) {
+                typedef A vec4 __attribute__((ext_vector_type(4)));
+                vec4 v[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) v[k] = *reinterpret_cast<const vec4 *>(rowp + 4 * (k0 + k));
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) tot[q] += v[k][q];
+            }
+            const A sum = (tot[0] + tot[1]) + (tot[2] + tot[3]);
+            // lane = slot * KK + tap: consecutive lanes are consecutive elements of dCF
+            const int slot = lane / KK, tap = lane - slot * KK;
+            const int64_t nc = wk.n * g.C + c0 + cbase + slot;
+            if (g.nstrips == 1) st(dcf + nc * KK + tap, sum);
+            else ws_cf[(nc * g.nstrips + wk.strip) * KK + tap] = sum;
+        }
+        wave_sync();
+    };
+
+    auto compute = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        if constexpr (sizeof(T) == 2 && MUL) {
+            // keep the packed taps packed (see k_rows)
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int t = 0; t < KK; ++t)
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfw[r][t][k]));
+        }
+        Row row[ROWS];
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) {
+#pragma unroll
+            for (int k = 0; k < NW; ++k) row[rr].own[k] = xw[ST][rr][k];
+            row[rr].sides(ln.first, ln.last);
+        }
+        A gval[R][VX];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int e = 0; e < VX; ++e) gval[r][e] = elem<T>(gw[ST][r], e);
+        A w[KK];
+        if constexpr (MUL) {
+            if constexpr (kScalarTaps) {
+#pragma unroll
+                for (int t = 0; t < KK; ++t) w[t] = cfu[ST][t];
+            } else {
+                const A cfa = (A)ld(&cfl[ST]);
+#pragma unroll
+                for (int t = 0; t < KK; ++t) w[t] = lane_broadcast<A>(cfa, t);
+            }
+        }
+        A pcf[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) pcf[t] = 0;
+#pragma unroll
+        for (int i = 0; i < K; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j)
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) {
+                        const int t = i * K + j;
+                        const A gx = gval[r][e] * row[r + i * D].at(e + j * D - HX);
+                        if constexpr (MUL) {
+                            acc_sf[r][t][e] = fma_(gx, w[t], acc_sf[r][t][e]);
+                            pcf[t] = fma_(gx, elem<T>(sfw[r][t], e), pcf[t]);
+                        } else {
+                            acc_sf[r][t][e] += gx;
+                            pcf[t] += gx;
+                        }
+                    }
+        if (want_cf && ci < nch) {
+            const int slot = ci & (G - 1);
+#pragma unroll
+            for (int t = 0; t < KK; ++t) red[(slot * KK + t) * kRedPitch + lane] = pcf[t];
+            if (slot == G - 1 || ci == nch - 1) flush(ci - slot, slot + 1);
+        }
+    };
+
+    // whole rounds of NST channels (see k_rows)
+    auto step = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        issue(std::integral_constant<int, (ST + NST - 1) % NST>{}, ci + NST - 1);
+        compute(st_tag, ci);
+    };
+    for (int ci = 0; ci < nch; ci += NST) {
+        step(std::integral_constant<int, 0>{}, ci);
+        if constexpr (NST > 1) step(std::integral_constant<int, 1>{}, ci + 1);
+        if constexpr (NST > 2) step(std::integral_constant<int, 2>{}, ci + 2);
+        if constexpr (NST > 3) step(std::integral_constant<int, 3>{}, ci + 3);
+    }
+
+    if (!want_sf) return;   // (uniform over the workgroup)
+    // Add the waves' dSF accumulators: kTapChunk taps per round through LDS.
+    A *all = reinterpret_cast<A *>(smem);
+#pragma unroll
+    for (int t0 = 0; t0 < KK; t0 += kTapChunk) {
+        __syncthreads();
+#pragma unroll
+        for (int tt = 0; tt < kTapChunk; ++tt)
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int e = 0; e < VX; ++e) {
+                    const int t = t0 + tt < KK ? t0 + tt : KK - 1;   // (past the last tap: unused filler)
+                    all[(((wave * kTapChunk + tt) * R + r) * VX + e) * kWave + lane] = acc_sf[r][t][e];
+                }
+        __syncthreads();
+        // (tap, row) pairs of this round are dealt out to the waves
+        for (int idx = wave; idx < kTapChunk * R; idx += kFilterWaves) {
+            const int tt = idx / R, r = idx - tt * R;
+            const int t = t0 + tt;
+            if (t >= KK) break;
+            A tot[VX];
+#pragma unroll
+            for (int e = 0; e < VX; ++e) {
+                tot[e] = 0;
+#pragma unroll
+                for (int wv = 0; wv < kFilterWaves; ++wv)
+                    tot[e] += all[(((wv * kTapChunk + tt) * R + r) * VX + e) * kWave + lane];
+            }
+            uint32_t off_r = kOutside;   // (by run-time row index, without a register array lookup)
+#pragma unroll
+            for (int q = 0; q < R; ++q)
+                if (q == r) off_r = ob[q];
+            if (g.csplit == 1) {
+                uint32_t ow[NW];
+                pack<T, VX, A>(tot, ow);
+                store_words_nt<NW>(plane_rsrc(dsf + (wk.n * KK + t) * plane, plane_bytes), off_r, ow);
+            } else {
+                // partial sums in the accumulator type, same plane shape
+                constexpr int AW = VX * sizeof(A) / 4;
+                constexpr int CH = AW < 4 ? AW : 4;
+                const __amdgpu_buffer_rsrc_t wr =
+                    plane_rsrc(ws_sf + ((wk.n * g.csplit + wk.cs) * KK + t) * plane,
+                               (uint32_t)plane * (uint32_t)sizeof(A));
+                const uint32_t off_a = off_r == kOutside ? kOutside
+                                                         : off_r / (uint32_t)sizeof(T) * (uint32_t)sizeof(A);
+                uint32_t aw[AW];
+                pack<A, VX, A>(tot, aw);
+#pragma unroll
+                for (int h = 0; h < AW; h += CH) {
+                    uint32_t part[CH];
+#pragma unroll
+                    for (int q = 0; q < CH; ++q) part[q] = aw[h + q];
+                    store_words_nt<CH>(wr, off_a + h * 4, part);
+                }
+            }
+        }
+    }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace rows
+
+// Host-side geometry of k_rows_filters (ddf_rows_host.hip): a work item is a
+// workgroup of rows::kFilterWaves waves (g->wpb = 1) that covers g->cpb =
+// g->cpw * rows::kFilterWaves channels; g->csplit counts those ranges.
+bool rows_filters_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx, int *r);
+// Workspace the kernel needs (layout as the tile kernels': dSF partials over
+// channel splits, then dCF partials over strips, each 256-byte aligned).
+size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);
+
+}  // namespace ddf

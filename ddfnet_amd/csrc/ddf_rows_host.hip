@@ -1,0 +1,190 @@
+// Host-side geometry of the row-register kernels: elements per lane and row,
+// rows per lane, how lanes are laid over a strip and how many channels a wave
+// walks.
+#include <algorithm>
+
+#include "ddf_rows_filters.h"
+
+namespace ddf {
+
+int tune_int(const char *name, int fallback);
+
+namespace {
+
+constexpr int kRowsStages = 3;   // channels in flight per wave of k_rows (rows::kStages)
+
+unsigned magic_of(int d) { return d == 1 ? 0u : (unsigned)((0x100000000ull + d - 1) / d); }
+
+// Lanes over a strip: lpr = W / vx lanes per image row, rg row groups of R rows
+// per wave, strips of even height.  Where it costs no row group, every image
+// row is followed by an idle lane (lane pitch lpr + 1): its loads return zero,
+// which is exactly what the neighbour shift must bring in at the row ends.
+void lay_out_lanes(RowsGeom *t, int H, int W, int vx, int R) {
+    t->lpr = W / vx;
+    const int row_units = (H + R - 1) / R;                  // lane-sized row groups of the plane
+    const int fit_plain = std::min(kWave / t->lpr, row_units);
+    const int fit_padded = std::min((kWave + 1) / (t->lpr + 1), row_units);
+    auto strips_with = [&](int fit) { return fit > 0 ? (row_units + fit - 1) / fit : 1 << 30; };
+    const bool pad = fit_padded > 0 && strips_with(fit_padded) <= strips_with(fit_plain) &&
+                     tune_int("DDF_TUNE_ROWS_PAD", 1) != 0;
+    t->lp = t->lpr + (pad ? 1 : 0);
+    t->lp_magic = magic_of(t->lp);
+    const int rg_max = pad ? fit_padded : fit_plain;
+    t->nstrips = (row_units + rg_max - 1) / rg_max;
+    t->rg = (row_units + t->nstrips - 1) / t->nstrips;      // even strips
+    t->rps = t->rg * R;
+}
+
+}  // namespace
+
+// Instantiated (elements per lane and row, rows per lane) per element size.
+bool rows_variant_built(int esz, int vx, int r) {
+    if (r != 2 && r != 1) return false;
+    if (esz == 2) return vx == 8 || vx == 4 || vx == 2;
+    if (esz == 4) return vx == 4 || vx == 2;
+    return false;
+}
+
+bool rows_shape_built(int k, int d, int s) { return s == 1 && k == 3 && (d == 1 || d == 2); }
+
+bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx_out, int *r_out) {
+    if (!rows_shape_built(p.k, p.d, p.s)) return false;
+    if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
+    if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
+    const int esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
+    const int H = (int)p.H, W = (int)p.W, C = (int)p.C;
+    const int hx = p.r * p.d;
+    if ((int64_t)H * W * esz >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
+    // widest vector the row length allows, at most 32 lanes per image row
+    int vx = 0;
+    for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
+        if (max_vx > 0 && cand > max_vx) continue;
+        if (cand > tune_int("DDF_TUNE_ROWS_VX", 16)) continue;
+        if (W % cand != 0 || cand < hx) continue;
+        if (W / cand > tune_int("DDF_TUNE_ROWS_LPR", 32)) continue;
+        vx = cand;
+        break;
+    }
+    if (vx == 0) return false;
+    // One row per lane keeps the registers low enough for 4-5 waves per SIMD,
+    // which is what the larger planes want.  Small fp32 planes whose rows are
+    // not a multiple of four pixels (14 x 14) take two rows per lane: the plane
+    // is then one strip, and the shorter prologue matters more there.
+    int R = (esz == 4 && vx == 2 && H % 2 == 0 && H * W <= 1024) ? 2 : 1;
+    R = tune_int("DDF_TUNE_ROWS_R", R);
+    if (!rows_variant_built(esz, vx, R)) return false;
+
+    RowsGeom t{};
+    t.C = C; t.H = H; t.W = W;
+    lay_out_lanes(&t, H, W, vx, R);
+
+    // Channels per wave: enough waves to fill the machine (and to even out its
+    // SIMDs), walks long enough to amortise the spatial-filter registers.  The
+    // kernels walk whole rounds of kRowsStages channels, so the count is a
+    // multiple of that.
+    const int64_t base = p.N * t.nstrips;
+    const int target = tune_int("DDF_TUNE_ROWS_WAVES", 8192);
+    const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
+    int cpw = (int)(C / want_split);
+    const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", 2 * kRowsStages);
+    cpw = std::max(cpw / kRowsStages * kRowsStages, min_cpw);
+    const int forced = tune_int("DDF_TUNE_ROWS_CPW", 0);
+    if (forced) cpw = forced;
+    t.cpw = std::max(1, std::min(cpw, C));
+    t.cpb = t.cpw;
+    t.csplit = (C + t.cpw - 1) / t.cpw;
+    t.wpb = std::max(1, std::min(tune_int("DDF_TUNE_ROWS_WPB", 2), rows::kMaxWpb));
+    const int64_t nwork = base * t.csplit;
+    if (nwork > (1 << 30)) return false;
+    // magic-number division of the work id is exact while id * divisor < 2^32
+    if (nwork * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
+    t.csplit_magic = magic_of(t.csplit);
+    t.nstrips_magic = magic_of(t.nstrips);
+    const int64_t ngroups = (nwork + t.wpb - 1) / t.wpb;
+    t.xcd_per = (unsigned)((ngroups + rows::kXcd - 1) / rows::kXcd);
+    t.nwork = (int)nwork;
+    *g = t;
+    *vx_out = vx;
+    *r_out = R;
+    return true;
+}
+
+// Instantiated (elements per lane and row, rows per lane) of k_rows_filters.
+bool rows_filters_variant_built(int esz, int vx, int r) {
+    if (r != 1) return false;
+    if (esz == 2) return vx == 4 || vx == 2;
+    if (esz == 4) return vx == 4 || vx == 2;
+    return false;
+}
+
+bool rows_filters_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx_out,
+                           int *r_out) {
+    if (!(p.s == 1 && p.k == 3 && p.d == 1)) return false;
+    if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
+    if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
+    const int esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
+    const int H = (int)p.H, W = (int)p.W, C = (int)p.C;
+    const int hx = p.r * p.d;
+    if ((int64_t)H * W * 8 >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
+    const int R = 1;
+    int vx = 0;
+    for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
+        if (max_vx > 0 && cand > max_vx) continue;
+        if (cand > tune_int("DDF_TUNE_ROWSF_VX", 16)) continue;
+        if (!rows_filters_variant_built(esz, cand, R)) continue;
+        if (W % cand != 0 || cand < hx) continue;
+        if (W / cand > 32) continue;
+        vx = cand;
+        break;
+    }
+    if (vx == 0) return false;
+
+    RowsGeom t{};
+    t.C = C; t.H = H; t.W = W;
+    lay_out_lanes(&t, H, W, vx, R);
+
+    // Channels per wave: the four waves of a workgroup cover cpb = 4 * cpw
+    // channels; enough workgroups to fill the machine, as few channel splits
+    // (dSF partial sums through the workspace) as that allows.
+    const int64_t base = p.N * t.nstrips;
+    const int target = tune_int("DDF_TUNE_ROWSF_WAVES", 2048);
+    const int64_t want_split = std::max<int64_t>(1, (target + base * rows::kFilterWaves - 1) /
+                                                        (base * rows::kFilterWaves));
+    int cpb = (int)((C + want_split - 1) / want_split);
+    int cpw = (cpb + rows::kFilterWaves - 1) / rows::kFilterWaves;
+    // whole rounds of the kernel's channel pipeline and whole dCF flush groups
+    cpw = (cpw + rows::kFlushChannels - 1) / rows::kFlushChannels * rows::kFlushChannels;
+    cpw = std::max(cpw, tune_int("DDF_TUNE_ROWSF_MIN_CPW", 2 * rows::kFlushChannels));
+    const int forced = tune_int("DDF_TUNE_ROWSF_CPW", 0);
+    if (forced) cpw = std::min(forced, C);
+    t.cpw = std::max(1, cpw);
+    t.cpb = t.cpw * rows::kFilterWaves;
+    t.csplit = (C + t.cpb - 1) / t.cpb;
+    t.wpb = 1;
+    const int64_t nwork = base * t.csplit;
+    if (nwork > (1 << 30)) return false;
+    if (nwork * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
+    t.csplit_magic = magic_of(t.csplit);
+    t.nstrips_magic = magic_of(t.nstrips);
+    t.xcd_per = (unsigned)((nwork + rows::kXcd - 1) / rows::kXcd);
+    t.nwork = (int)nwork;
+    *g = t;
+    *vx_out = vx;
+    *r_out = R;
+    return true;
+}
+
+size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need) {
+    if (!(need & (DDF_NEED_DCF | DDF_NEED_DSF))) return 0;
+    RowsGeom g; int vx, r;
+    if (!rows_filters_geometry(p, dtype, 0, &g, &vx, &r)) return 0;
+    const size_t asz = dtype == DDF_F64 ? 8 : 4;
+    size_t bytes = 0;
+    if ((need & DDF_NEED_DSF) && g.csplit > 1)
+        bytes += ((size_t)p.N * g.csplit * p.kk * p.H * p.W * asz + 255) / 256 * 256;
+    if ((need & DDF_NEED_DCF) && g.nstrips > 1)
+        bytes += ((size_t)p.N * p.C * g.nstrips * p.kk * asz + 255) / 256 * 256;
+    return bytes;
+}
+
+}  // namespace ddf

@@ -1,0 +1,160 @@
+// Launch code of the row-register kernels, instantiated once per element type.
+#pragma once
+
+#include "ddf_rows_filters.h"
+#include "ddf_wave.h"
+
+namespace ddf {
+namespace rows {
+
+constexpr int kStages = 3;   // channels in flight per wave (one computed, two loading)
+// waves per SIMD the registers are budgeted for (fp16 with 16 pixels per lane needs the room)
+template <typename T, int VX, int R>
+constexpr int waves_per_simd() { return sizeof(T) == 2 && VX * R >= 16 ? 2 : 3; }
+
+template <typename T, int K, int D, int VX, int R>
+hipError_t launch_kdv(const Problem &p, const RowsGeom &g, bool backward, const T *x, const T *cf,
+                      const T *sf, T *out, hipStream_t st) {
+    const dim3 grid(g.xcd_per * kXcd), block(kWave * g.wpb);
+    const bool pad = g.lp > g.lpr;
+#define DDF_ROWS_CASE(MUL_, BWD_)                                                               \
+    do {                                                                                        \
+        if (pad)                                                                                \
+            hipLaunchKernelGGL((k_rows<T, K, D, MUL_, BWD_, VX, R, true, kStages,               \
+                                       waves_per_simd<T, VX, R>()>),                            \
+                               grid, block, 0, st, g, x, cf, sf, out);                          \
+        else                                                                                    \
+            hipLaunchKernelGGL((k_rows<T, K, D, MUL_, BWD_, VX, R, false, kStages,              \
+                                       waves_per_simd<T, VX, R>()>),                            \
+                               grid, block, 0, st, g, x, cf, sf, out);                          \
+    } while (0)
+    if (p.mul) {
+        if (backward) DDF_ROWS_CASE(true, true);
+        else DDF_ROWS_CASE(true, false);
+    } else {
+        if (backward) DDF_ROWS_CASE(false, true);
+        else DDF_ROWS_CASE(false, false);
+    }
+#undef DDF_ROWS_CASE
+    return hipGetLastError();
+}
+
+template <typename T, int VX, int R>
+hipError_t launch_v(const Problem &p, const RowsGeom &g, bool backward, const T *x, const T *cf,
+                    const T *sf, T *out, hipStream_t st) {
+    if (p.k == 3 && p.d == 1) return launch_kdv<T, 3, 1, VX, R>(p, g, backward, x, cf, sf, out, st);
+    if constexpr (VX >= 2) {
+        if (p.k == 3 && p.d == 2)
+            return launch_kdv<T, 3, 2, VX, R>(p, g, backward, x, cf, sf, out, st);
+    }
+    return hipErrorNotSupported;
+}
+
+}  // namespace rows
+
+// Forward (backward = false: x -> out) or feature gradient (backward = true:
+// dO -> dX) on the row-register kernels.  hipErrorNotSupported: not covered
+// (shape, or pointers not aligned to the vector the geometry wants); nothing
+// was launched then.
+template <typename T>
+hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf, const T *sf,
+                       T *out, hipStream_t st) {
+    const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
+    RowsGeom g;
+    int vx, r;
+    if (!rows_geometry(p, dtype, 0, &g, &vx, &r)) return hipErrorNotSupported;
+    const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
+    if ((((uintptr_t)x | (uintptr_t)sf | (uintptr_t)out) & mask) != 0) return hipErrorNotSupported;
+    if constexpr (sizeof(T) == 2) {
+        if (vx == 8 && r == 2) return rows::launch_v<T, 8, 2>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 2 && r == 2) return rows::launch_v<T, 2, 2>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 8 && r == 1) return rows::launch_v<T, 8, 1>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
+    } else if constexpr (sizeof(T) == 4) {
+        if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 2 && r == 2) return rows::launch_v<T, 2, 2>(p, g, backward, x, cf, sf, out, st);
+    }
+    return hipErrorNotSupported;
+}
+
+namespace rows {
+
+template <typename T, int VX, int R>
+hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, const T *x,
+                            const T *cf, const T *sf, T *dcf, T *dsf,
+                            typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
+                            unsigned need, hipStream_t st) {
+    using A = typename Acc<T>::type;
+    // waves per SIMD the registers are budgeted for: 'mul' keeps the spatial taps as well
+    constexpr int WPE_MUL = VX * R >= 4 ? 2 : 3, WPE_ADD = 3;
+    constexpr int kFilterStages = 2;   // channels in flight per wave
+    const dim3 grid(g.xcd_per * kXcd), block(kWave * kFilterWaves);
+    const int lds = filters_lds_bytes<9>((int)sizeof(A), R, VX);
+    if (p.k != 3 || p.d != 1) return hipErrorNotSupported;
+    const bool pad = g.lp > g.lpr;
+#define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
+    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, R, PAD_, kFilterStages,                \
+                                       MUL_ ? WPE_MUL : WPE_ADD>),                               \
+                       grid, block, lds, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need)
+    if (p.mul) {
+        if (pad) DDF_ROWSF_CASE(true, true);
+        else DDF_ROWSF_CASE(true, false);
+    } else {
+        if (pad) DDF_ROWSF_CASE(false, true);
+        else DDF_ROWSF_CASE(false, false);
+    }
+#undef DDF_ROWSF_CASE
+    return hipGetLastError();
+}
+
+}  // namespace rows
+
+// Filter gradients on the row-register kernel, partial sums included.
+// hipErrorNotSupported: not covered (nothing was launched).  `ws` must hold
+// rows_filters_workspace() bytes.
+template <typename T>
+hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
+                               T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st) {
+    using A = typename Acc<T>::type;
+    const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
+    RowsGeom g;
+    int vx, r;
+    if (!rows_filters_geometry(p, dtype, 0, &g, &vx, &r)) return hipErrorNotSupported;
+    const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
+    if ((((uintptr_t)x | (uintptr_t)go | (uintptr_t)sf | (uintptr_t)dsf) & mask) != 0)
+        return hipErrorNotSupported;
+    unsigned char *wp = static_cast<unsigned char *>(ws);
+    A *ws_sf = nullptr, *ws_cf = nullptr;
+    const int64_t n_sf = p.N * p.kk * p.H * p.W;
+    if ((need & DDF_NEED_DSF) && g.csplit > 1) {
+        ws_sf = reinterpret_cast<A *>(wp);
+        wp += ((size_t)n_sf * g.csplit * sizeof(A) + 255) / 256 * 256;
+    }
+    if ((need & DDF_NEED_DCF) && g.nstrips > 1) ws_cf = reinterpret_cast<A *>(wp);
+    hipError_t err = hipErrorNotSupported;
+    if constexpr (sizeof(T) != 8) {
+        if (vx == 4 && r == 1)
+            err = rows::launch_filters_v<T, 4, 1>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+        else if (vx == 2 && r == 1)
+            err = rows::launch_filters_v<T, 2, 1>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+    }
+    if (err != hipSuccess) return err;
+    if (ws_sf) {
+        err = wave::sum_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.H * p.W, st);
+        if (err != hipSuccess) return err;
+    }
+    if (ws_cf) err = wave::sum_partials<T>(ws_cf, dcf, p.N * p.C, g.nstrips, (int64_t)p.kk, st);
+    return err;
+}
+
+#define DDF_INSTANTIATE_ROWS(T)                                                              \
+    template hipError_t rows_filters_launch<T>(const Problem &, const T *, const T *, const T *, \
+                                               const T *, T *, T *, void *, unsigned, hipStream_t); \
+    template hipError_t rows_launch<T>(const Problem &, bool, const T *, const T *, const T *, \
+                                       T *, hipStream_t);
+
+}  // namespace ddf

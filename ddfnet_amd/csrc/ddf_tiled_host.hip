@@ -10,9 +10,18 @@ namespace ddf {
 namespace {
 
 
+// Launch-geometry knobs.  A release build compiles them to their defaults: no
+// environment lookups on the launch path, and a geometry that depends on the
+// problem alone.  Built with -DDDF_TUNING they are read from the environment
+// at every call, for experiments and for the host-side bounds model.
 int env_int(const char *name, int fallback) {
+#ifdef DDF_TUNING
     const char *v = std::getenv(name);
     return (v && *v) ? std::atoi(v) : fallback;
+#else
+    (void)name;
+    return fallback;
+#endif
 }
 
 int elem_size(int dtype) { return dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8; }
@@ -22,6 +31,8 @@ int round_up(int v, int m) { return (v + m - 1) / m * m; }
 }  // namespace
 
 int tune_int(const char *name, int fallback) { return env_int(name, fallback); }
+
+size_t wave_backward_workspace(const Problem &p, int dtype, unsigned need);
 
 bool tiled_shape_instantiated(int k, int d, int s) {
     return (k == 3 || k == 5) && (d == 1 || d == 2) && (s == 1 || s == 2);
@@ -248,6 +259,11 @@ bool tiled_backward_supported(const Problem &p, int dtype) {
 // each in the accumulator type and starting on a 256-byte boundary.
 size_t tiled_backward_workspace(const Problem &p, int dtype, unsigned need) {
     if (!(need & (DDF_NEED_DCF | DDF_NEED_DSF))) return 0;
+    // whichever family runs (it depends on pointer alignment too) finds room
+    return std::max(wave_backward_workspace(p, dtype, need), rows_filters_workspace(p, dtype, need));
+}
+
+size_t wave_backward_workspace(const Problem &p, int dtype, unsigned need) {
     // csplit and nstrips do not depend on the access width, so the scalar
     // fallback for misaligned pointers needs the same workspace
     WaveGeom g; int ps, nv;

@@ -154,6 +154,12 @@ template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf, T *out,
                          hipStream_t st) {
     if (small_supported(p)) return small_launch<T>(p, false, x, cf, sf, out, st);
+    if constexpr (sizeof(T) != 8) {
+        if (tune_int("DDF_TUNE_ROWS", 1) != 0) {
+            const hipError_t err = rows_launch<T>(p, false, x, cf, sf, out, st);
+            if (err != hipErrorNotSupported) return err;
+        }
+    }
     WaveGeom g; int ps, nv;
     if (!wave_plan<T>(p, kWaveForward, {x, sf, out}, &g, &ps, &nv))
         return generic_forward<T>(p, x, cf, sf, out, st);   // e.g. pointers not 16-byte aligned
@@ -179,7 +185,15 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
                gp.csplit == g.csplit;
     }
     if ((need & DDF_NEED_DX) && !fuse) {
-        if (small_supported(p)) {
+        bool done = false;
+        if constexpr (sizeof(T) != 8) {
+            if (!small_supported(p) && tune_int("DDF_TUNE_ROWS", 1) != 0) {
+                err = rows_launch<T>(p, true, go, cf, sf, dx, st);
+                done = err != hipErrorNotSupported;
+            }
+        }
+        if (done) {
+        } else if (small_supported(p)) {
             err = small_launch<T>(p, true, go, cf, sf, dx, st);
         } else if (!wave_plan<T>(p, kWaveFeatures, {go, sf, dx}, &g, &ps, &nv)) {
             err = generic_backward<T>(p, go, x, cf, sf, dx, dcf, dsf, DDF_NEED_DX, st);
@@ -187,6 +201,15 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
             DDF_DISPATCH_KDS(p, err = tiled::launch_features<T, KK_, DD_, SS_>(p, g, ps, nv, go, cf, sf, dx, st));
         }
         if (err != hipSuccess) return err;
+    }
+    if (fneed && !fuse) {
+        if constexpr (sizeof(T) != 8) {
+            if (tune_int("DDF_TUNE_ROWSF", 1) != 0) {
+                err = rows_filters_launch<T>(p, go, x, cf, sf, dcf, dsf, ws, fneed, st);
+                if (err != hipErrorNotSupported) return err;
+                err = hipSuccess;
+            }
+        }
     }
     if (fneed) {
         if (!fuse && !wave_plan<T>(p, kWaveFilters, {go, x, sf}, &g, &ps, &nv))

@@ -1158,7 +1158,7 @@ inline hipError_t sum_partials(const typename Acc<T>::type *part, T *out, int64_
 
 }  // namespace wave
 
-// Integer tuning knob from the environment (for experiments), else `fallback`.
+// Integer tuning knob: `fallback`, or the environment's value in a -DDDF_TUNING build.
 int tune_int(const char *name, int fallback);
 
 enum WaveKind { kWaveForward = 0, kWaveFeatures = 1, kWaveFilters = 2, kWaveFused = 3 };

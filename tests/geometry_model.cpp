@@ -8,8 +8,10 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <vector>
 
 #include "ddf_tiled_host.hip"
+#include "ddf_rows_host.hip"
 
 using namespace ddf;
 
@@ -176,6 +178,99 @@ static void check_geometry(int kind, long N, long C, long H, long W, int k, int 
     g_fails = 0;
 }
 
+// Row-register kernels (ddf_rows.h, ddf_rows_filters.h): the kernels ask rows::Lane and
+// rows::Work - the very code compiled here - where a lane's vectors are, so the model runs
+// that code for every lane of every strip and checks what the kernels rely on: offsets
+// inside the plane and aligned to the vector (or -1: the access is given an offset outside
+// the buffer descriptor), every pixel of the plane owned by exactly one lane, an idle lane
+// after every image row in the padded layout, all lanes within the wavefront, every work
+// item mapped to its own (sample, strip, channel range), the channel ranges covering C.
+template <int R, int HY, int VX>
+static void replay_rows(const RowsGeom &g, long N, long C, bool filters) {
+    const long plane = (long)g.H * g.W;
+    std::vector<int> owner(plane, 0);
+    CHECK(g.lp == g.lpr || g.lp == g.lpr + 1, "lane pitch %d for %d lanes per row", g.lp, g.lpr);
+    CHECK((long)(g.rg - 1) * g.lp + g.lpr <= 64, "row groups do not fit the wavefront");
+    CHECK(g.lpr * VX == g.W, "lanes per row");
+    for (int strip = 0; strip < g.nstrips; ++strip)
+        for (int lane = 0; lane < 64; ++lane) {
+            rows::Lane<R, HY, VX> ln;
+            ln.init(g, strip, lane);
+            const int grp = lane / g.lp, v = lane % g.lp;
+            for (int rr = 0; rr < R + 2 * HY; ++rr) {
+                const int off = ln.xoff[rr];
+                if (off < 0) continue;
+                CHECK(grp < g.rg && v < g.lpr, "idle lane %d with a live offset", lane);
+                CHECK(off % VX == 0 && off + VX <= plane, "offset %d outside the plane or misaligned", off);
+                const int yy = strip * g.rps + grp * R - HY + rr;
+                CHECK(off == yy * g.W + v * VX, "offset %d is not row %d vector %d", off, yy, v);
+            }
+            for (int r = 0; r < R; ++r)
+                if (ln.ooff[r] >= 0)
+                    for (int e = 0; e < VX; ++e) ++owner[ln.ooff[r] + e];
+            if (g.lp > g.lpr && v == g.lpr)
+                for (int rr = 0; rr < R + 2 * HY; ++rr) CHECK(ln.xoff[rr] < 0, "padding lane %d is live", lane);
+            CHECK(ln.first == (v == 0) && ln.last == (v == g.lpr - 1), "row ends");
+        }
+    for (long i = 0; i < plane; ++i)
+        if (owner[i] != 1) { CHECK(false, "pixel %ld owned %d times", i, owner[i]); break; }
+    // work items
+    const long items = (long)N * g.nstrips * g.csplit;
+    CHECK(items == g.nwork, "work items %d", g.nwork);
+    CHECK((long)g.csplit * g.cpb >= C && (long)(g.csplit - 1) * g.cpb < C, "channel ranges");
+    if (filters) CHECK(g.cpb == g.cpw * rows::kFilterWaves && g.wpb == 1, "filter workgroup shape");
+    else CHECK(g.cpb == g.cpw && g.wpb >= 1 && g.wpb <= rows::kMaxWpb, "waves per workgroup");
+    const long groups = (items + g.wpb - 1) / g.wpb;
+    CHECK((long)g.xcd_per * 8 >= groups && (long)(g.xcd_per - 1) * 8 < groups, "workgroups per XCD");
+    const long nblk = (long)g.xcd_per * 8;
+    std::vector<char> seen(items, 0);
+    const long stepb = nblk > 100000 ? 53 : 1;
+    for (long blk = 0; blk < nblk; blk += stepb)
+        for (int w = 0; w < g.wpb; ++w) {
+            rows::Work wk;
+            if (!wk.init(g, (int)blk, w)) continue;
+            const long id = ((long)wk.n * g.nstrips + wk.strip) * g.csplit + wk.cs;
+            CHECK(wk.n < N && wk.strip < g.nstrips && wk.cs < g.csplit && id < items, "work item out of range");
+            if (id < items) { CHECK(!seen[id], "work item %ld handed out twice", id); seen[id] = 1; }
+            CHECK(wk.c_begin == wk.cs * g.cpb && wk.c_end <= C && wk.c_end > wk.c_begin, "channel range");
+        }
+    if (stepb == 1)
+        for (long i = 0; i < items; ++i)
+            if (!seen[i]) { CHECK(false, "work item %ld never handed out", i); break; }
+}
+
+static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, bool filters) {
+    const Problem p = make_problem(N, C, H, W, k, d, 1, 0);
+    RowsGeom g;
+    int vx, r;
+    const bool ok = filters ? rows_filters_geometry(p, dtype, 0, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r);
+    if (!ok) {
+        printf("kind rows%s %ldx%ldx%ldx%ld k%d d%d dt%d: unsupported\n", filters ? "-filters" : "", N, C, H, W, k, d, dtype);
+        return;
+    }
+    printf("kind rows%s %ldx%ldx%ldx%ld k%d d%d dt%d: vx=%d r=%d lpr=%d lp=%d rg=%d rps=%d nstrips=%d cpw=%d cpb=%d "
+           "csplit=%d wpb=%d nwork=%d\n", filters ? "-filters" : "", N, C, H, W, k, d, dtype, vx, r, g.lpr, g.lp,
+           g.rg, g.rps, g.nstrips, g.cpw, g.cpb, g.csplit, g.wpb, g.nwork);
+    const int esz = dtype == 0 ? 2 : dtype == 1 ? 4 : 8;
+    CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4, "vector of %d bytes", vx * esz);
+    CHECK((k / 2) * d <= vx, "taps reach beyond the neighbouring lane");
+    CHECK((long)H * W * 8 < (1l << 31), "plane beyond 32-bit byte offsets");
+    if (filters) {
+        const int lds = rows::filters_lds_bytes<9>(dtype == 2 ? 8 : 4, r, vx);
+        CHECK(lds <= 64 * 1024, "filter kernel LDS %d", lds);
+        CHECK(g.cpw % rows::kFlushChannels == 0, "channels per wave %d not whole flush groups", g.cpw);
+    }
+    const int hy = (k / 2) * d;
+#define ROWS_CASE(R_, HY_, VX_) if (r == R_ && hy == HY_ && vx == VX_) { replay_rows<R_, HY_, VX_>(g, N, C, filters); done = true; }
+    bool done = false;
+    ROWS_CASE(1, 1, 2) ROWS_CASE(1, 1, 4) ROWS_CASE(1, 1, 8) ROWS_CASE(2, 1, 2) ROWS_CASE(2, 1, 4) ROWS_CASE(2, 1, 8)
+    ROWS_CASE(1, 2, 2) ROWS_CASE(1, 2, 4) ROWS_CASE(1, 2, 8) ROWS_CASE(2, 2, 2) ROWS_CASE(2, 2, 4) ROWS_CASE(2, 2, 8)
+#undef ROWS_CASE
+    CHECK(done, "no replay for r=%d hy=%d vx=%d", r, hy, vx);
+    if (g_fails) printf("  -> %d violations\n", g_fails);
+    g_fails = 0;
+}
+
 int main() {
     const long shapes[][4] = {
         {96, 64, 56, 56},   {64, 256, 14, 14}, {64, 128, 28, 28},  {64, 512, 7, 7},   {64, 64, 56, 56},
@@ -192,6 +287,11 @@ int main() {
                         if (sh[2] / q[2] == 0 || sh[3] / q[2] == 0) continue;
                         check_geometry(kind, sh[0], sh[1], sh[2], sh[3], q[0], q[1], q[2], dtype, max_vec);
                     }
+    for (auto &sh : shapes)
+        for (int d = 1; d <= 2; ++d)
+            for (int dtype = 0; dtype < 3; ++dtype)
+                for (int filters = 0; filters < 2; ++filters)
+                    check_rows(sh[0], sh[1], sh[2], sh[3], 3, d, dtype, filters != 0);
     // seeded random shapes on top of the fixed list
     unsigned long long state = 0x9E3779B97F4A7C15ull;
     auto next = [&](int lo, int hi) {
@@ -204,6 +304,8 @@ int main() {
         if (H / q[2] == 0 || W / q[2] == 0) continue;
         for (int kind = 0; kind < 4; ++kind)
             check_geometry(kind, N, C, H, W, q[0], q[1], q[2], next(0, 2), next(0, 1));
+        check_rows(N, C, H, W / 2 * 2 + 2, 3, next(1, 2), next(0, 1), next(0, 1) != 0);
+        check_rows(N, C, H, (W / 8 + 1) * 8, 3, next(1, 2), next(0, 1), next(0, 1) != 0);
     }
     return 0;
 }

@@ -253,7 +253,9 @@ def test_needs_input_grad_subsets():
         part = run_ddf(x, cf, sf, go, 3, 1, 1, 'mul', need=need)
         for g_full, g_part, n in zip(full[1:], part[1:], need):
             if n:
-                assert torch.equal(g_full, g_part)
+                # a subset may run other kernels than the full backward (other
+                # summation order): equal to rounding, not bit for bit
+                assert rel_err(g_part, g_full.cpu()) <= 1e-6
             else:
                 assert g_part is None
 
@@ -261,41 +263,26 @@ def test_needs_input_grad_subsets():
 @pytest.mark.parametrize('dtype', [torch.float32, torch.float16], ids=_ids)
 @pytest.mark.parametrize('combine', ['mul', 'add'])
 @pytest.mark.parametrize('shape,d', [((3, 40, 14, 14), 1), ((2, 24, 14, 14), 2), ((2, 9, 12, 16), 1),
-                                     ((1, 130, 8, 8), 1)])
-def test_one_launch_backward_equals_two_launches(shape, d, combine, dtype, monkeypatch):
-    """All three gradients requested together come from one fused kernel where
-    it exists (3x3, stride 1, short strips); switched off, the feature gradient
-    and the filter gradients come from their own kernels.  Same sums in the same
-    order: the results must be identical, and both must match the oracle."""
+                                     ((1, 130, 8, 8), 1), ((2, 20, 28, 28), 1), ((2, 12, 56, 56), 1)])
+def test_one_launch_backward_equals_separate_requests(shape, d, combine, dtype):
+    """All three gradients requested together may come from one fused kernel
+    (3x3, stride 1, short strips); requested one at a time - what autograd does
+    when only some inputs need gradients - the feature gradient and the filter
+    gradients come from kernels of their own.  The routes may order their sums
+    differently: they must agree to rounding, and both must match the oracle."""
     N, C, H, W = shape
     x, cf, sf, go = random_case(N, C, H, W, 3, 1, dtype, seed=11)
-    fused = run_ddf(x, cf, sf, go, 3, d, 1, combine)
-    monkeypatch.setenv('DDF_TUNE_FUSED', '0')
-    split = run_ddf(x, cf, sf, go, 3, d, 1, combine)
-    for a, b in zip(fused, split):
-        assert torch.equal(a, b)
+    together = run_ddf(x, cf, sf, go, 3, d, 1, combine)
+    only_dx = run_ddf(x, cf, sf, go, 3, d, 1, combine, need=(True, False, False))
+    only_filters = run_ddf(x, cf, sf, go, 3, d, 1, combine, need=(False, True, True))
+    tol = 1e-6 if dtype == torch.float32 else 2e-3
+    assert rel_err(only_dx[0], together[0].cpu()) == 0.0
+    assert rel_err(only_dx[1], together[1].cpu()) <= tol
+    assert rel_err(only_filters[2], together[2].cpu()) <= tol
+    assert rel_err(only_filters[3], together[3].cpu()) <= tol
     want = oracle.backward(go, x, cf, sf, 3, d, 1, combine)
-    for got, w in zip(fused[1:], want):
+    for got, w in zip(together[1:], want):
         assert rel_err(got, w) <= TOL[dtype]
-
-
-@pytest.mark.parametrize('knob,value', [('DDF_TUNE_WPB', '2'), ('DDF_TUNE_WPB', '4'),
-                                        ('DDF_TUNE_WIDE', '0'), ('DDF_TUNE_WAVES', '512'),
-                                        ('DDF_TUNE_CPW', '3'), ('DDF_TUNE_VEC', '1')])
-def test_tuning_knobs_do_not_change_results(knob, value, monkeypatch):
-    """The launch geometry has experiment knobs (waves per workgroup, aligned
-    tile writes, wave count, channels per wave, access width).  Whatever they
-    are set to, the kernels must produce the same bits: the knobs change how
-    the work is cut, not the order of any sum."""
-    cases = [((3, 40, 14, 14), 3, 1, 1, torch.float32), ((2, 24, 28, 28), 3, 2, 1, torch.float16),
-             ((2, 16, 20, 24), 5, 1, 2, torch.float32)]
-    for (N, C, H, W), k, d, s, dtype in cases:
-        x, cf, sf, go = random_case(N, C, H, W, k, s, dtype, seed=31)
-        base = run_ddf(x, cf, sf, go, k, d, s, 'mul', need=(True, False, False))
-        monkeypatch.setenv(knob, value)
-        tuned = run_ddf(x, cf, sf, go, k, d, s, 'mul', need=(True, False, False))
-        monkeypatch.delenv(knob)
-        assert torch.equal(base[0], tuned[0]) and torch.equal(base[1], tuned[1])
 
 
 def test_mixed_dtypes_are_promoted():

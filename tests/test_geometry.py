@@ -25,7 +25,7 @@ def _hipcc():
 @pytest.mark.skipif(_hipcc() is None, reason='hipcc not available')
 def test_every_launch_geometry_stays_in_bounds(tmp_path):
     exe = str(tmp_path / 'geometry_model')
-    cmd = [_hipcc(), '-O1', '-x', 'hip', '--cuda-host-only', '-w',
+    cmd = [_hipcc(), '-O1', '-x', 'hip', '--cuda-host-only', '-w', '-DDDF_TUNING',
            '-I' + os.path.join(ROOT, 'include'), '-I' + os.path.join(ROOT, 'ddfnet_amd', 'csrc'),
            os.path.join(ROOT, 'tests', 'geometry_model.cpp'), '-o', exe]
     build = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
@@ -34,8 +34,12 @@ def test_every_launch_geometry_stays_in_bounds(tmp_path):
     for key in list(env):
         if key.startswith('DDF_TUNE_'):
             del env[key]
+    # (the model is built with the geometry knobs switched on, so that other cuts of the
+    # same problems are replayed as well; the shipped library compiles them to defaults)
     for extra in ({}, {'DDF_TUNE_WPB': '4'}, {'DDF_TUNE_WIDE': '0'}, {'DDF_TUNE_WAVES': '512'},
-                  {'DDF_TUNE_CPW': '3', 'DDF_TUNE_CPW_FILTERS': '3'}, {'DDF_TUNE_VEC': '1'}):
+                  {'DDF_TUNE_CPW': '3', 'DDF_TUNE_CPW_FILTERS': '3'}, {'DDF_TUNE_VEC': '1'},
+                  {'DDF_TUNE_ROWS_R': '2'}, {'DDF_TUNE_ROWS_R': '1', 'DDF_TUNE_ROWS_PAD': '0'},
+                  {'DDF_TUNE_ROWS_WAVES': '512', 'DDF_TUNE_ROWS_WPB': '4', 'DDF_TUNE_ROWS_LPR': '64'}):
         run = subprocess.run([exe], capture_output=True, text=True, timeout=600,
                              env=dict(env, **extra))
         assert run.returncode == 0
