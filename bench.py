@@ -7,17 +7,26 @@ operator over one batch of synthetic input, called through the C ABI of
 workload is the ResNet-50 stage-3 shape the headline metric is quoted on:
 N=64, C=256, 14x14, k=3 d=1 s=1, 'mul', fp32, filters standardised per tap set.
 
-Timing: W warm-up steps, then K steps between two events on the launch stream,
-bracketed by device synchronisation.  Inputs and outputs rotate over enough
-distinct buffer sets to exceed the 256 MB last-level cache, so the figure is an
-HBM figure.  ``value`` = algorithmic bytes of forward+backward / time per step.
+Timing: W warm-up steps, then exactly K steps between two events on the launch
+stream, bracketed by device synchronisation.  Inputs and outputs rotate over
+enough distinct buffer sets to exceed the 256 MB last-level cache, so the
+figure is an HBM figure.  ``value`` = algorithmic bytes of forward+backward /
+time per step.  Four more blocks of K steps follow; ``ms_per_step_median`` is
+the median of the five.
 
-After the timed region each library call of a step (forward / feature gradient
-/ filter gradients) is timed on its own: K back-to-back launches between one
-event pair, same buffers.  The ``roofline`` object reports the slowest of them.
+After the timed region each library call of a step (forward / backward / the
+two halves of the backward requested separately) is timed on its own: five
+blocks of K back-to-back launches, median reported, same buffers.  The
+``roofline`` object describes the slower call of the step; its ``traffic`` is
+looked up in ``profiles/`` (hardware counters of the same kernels) and is null
+when no profile covers the kernels the library reports for that call.
 
-``--model`` additionally times ddf_mul_resnet50 inference (fp16, batch 128,
-224x224, random weights) and reports images/s with the DDF share of the time.
+The same line carries the other benchmark configurations
+(``other_workloads``: the fp16 'add' stage-1 shape, the strided and the
+dilated 5x5 shapes, two more ResNet stages), ddf_mul_resnet50 inference
+(``model_inference``: fp16, batch 128, 224x224, random weights: images/s and
+per-layer GB/s of the DDF layers) and the CPU baseline; ``--only-headline``
+leaves the first two out.
 
 Prints ONE JSON line on stdout; everything else goes to stderr.
 """
@@ -53,18 +62,6 @@ DTYPE_NAME = {torch.float32: 'f32', torch.float16: 'f16', torch.float64: 'f64'}
 # (autograd does that when only some inputs need gradients).
 PHASES = ('fwd', 'bwd', 'dx', 'dfilters')
 STEP_PHASES = ('fwd', 'bwd')
-# kernels behind each call.  At 3x3 / stride 1 with short strips the whole
-# backward pass is one launch of k_backward_filters<..., DX=true> (it also
-# writes the feature gradient); otherwise bwd = the dx call + the dfilters call.
-PHASE_KERNELS = {
-    'fwd': 'ddf::wave::k_forward',
-    # one fused launch where a plane fits one 16-byte vector per lane (3x3,
-    # stride 1, up to about 16x16), else feature and filter gradients apart
-    'bwd': 'ddf::wave::k_backward_filters<DX=true> + ddf::wave::k_sum_partials',
-    'dx': 'ddf::wave::k_backward_features',
-    'dfilters': 'ddf::wave::k_backward_filters<DX=false> + ddf::wave::k_sum_partials',
-}
-
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -172,21 +169,31 @@ def timed(fn, count):
     return start.elapsed_time(stop) / count
 
 
-# HBM bytes per library call of a phase, from hardware counters: two
-# `rocprofv3 --pmc` runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per
-# dispatch, summed over the kernels of the call), each scaled by what the same
-# counter reads for the 256 MiB device copy of --copy-probe (fetch x2.000,
-# write x1.000 on MI355X).  Counters cannot be read from inside a timed run, so
-# the figures are recorded here; a workload or phase that was not profiled
-# reports null.
-MEASURED_TRAFFIC = {
-    'r50_stage3_mul_fp32': {'fwd': 27760539, 'bwd': 49286424, 'dx': 27762539, 'dfilters': 35535013},
-    'r50_stage1_add_fp16': {'fwd': 56477696, 'bwd': 116746240, 'dx': 56538112, 'dfilters': 60208128},
-}
-# kernels behind the backward call where the fused kernel does not apply
-UNFUSED_BWD = ('ddf::wave::k_backward_features + ddf::wave::k_backward_filters<DX=false> + '
-               'ddf::wave::k_sum_partials')
-FUSED_BWD_WORKLOADS = ('r50_stage3_mul_fp32',)
+def timed_blocks(fn, count, blocks=5):
+    """`blocks` timed blocks of `count` calls each; (first, median) in ms per call."""
+    t = [timed(fn, count) for _ in range(blocks)]
+    return t[0], sorted(t)[len(t) // 2]
+
+
+def profiled_traffic(workload, phase, kernels):
+    """HBM bytes per call from hardware counters, as recorded in profiles/*.md
+    by lines of the form
+        TRAFFIC workload=<name> phase=<fwd|bwd|dx|dfilters> kernels="<names>" bytes=<n>
+    (FETCH_SIZE and WRITE_SIZE runs of rocprofv3, scaled as the file says).
+    Returns (bytes, file name), or (None, None) when no line matches the kernels
+    the library reports for this call."""
+    import glob
+    import re
+    pat = re.compile(r'TRAFFIC workload=(\S+) phase=(\S+) kernels="([^"]*)" bytes=(\d+)')
+    for path in sorted(glob.glob(os.path.join(ROOT, 'profiles', '*.md'))):
+        try:
+            text = open(path).read()
+        except OSError:
+            continue
+        for m in pat.finditer(text):
+            if m.group(1) == workload and m.group(2) == phase and m.group(3) == kernels:
+                return int(m.group(4)), os.path.relpath(path, ROOT)
+    return None, None
 
 
 def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
@@ -208,14 +215,16 @@ def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
 
     for i in range(warmup):
         step(i)
-    ms_per_step = timed(step, steps)
+    ms_per_step, ms_median = timed_blocks(step, steps)
 
     # each library call on its own: back-to-back launches, same buffers
     phase_ms = {}
     for ph in PHASES:
         for i in range(min(warmup, 10)):
             run.phase(ph, i)
-        phase_ms[ph] = timed(lambda i, ph=ph: run.phase(ph, i), steps)
+        phase_ms[ph] = timed_blocks(lambda i, ph=ph: run.phase(ph, i), steps)[1]
+    need_of = {'fwd': 0, 'bwd': 7, 'dx': 1, 'dfilters': 6}
+    kernels = {ph: lib.describe((N, C, H, W), k, d, s, combine, dtype, need_of[ph]) for ph in PHASES}
 
     if copy_probe:
         # a plain device copy of known size: the yardstick the hardware
@@ -231,7 +240,7 @@ def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
     res = {
         'workload': name, 'N': N, 'C': C, 'H': H, 'W': W, 'k': k, 'd': d, 's': s,
         'combine': combine, 'dtype': DTYPE_NAME[dtype],
-        'ms_per_step': ms_per_step,
+        'ms_per_step': ms_per_step, 'ms_per_step_median': ms_median, 'kernels': kernels,
         'gbps': total / (ms_per_step * 1e-3) / 1e9,
         'images_per_s': N / (ms_per_step * 1e-3),
         'bytes': ab, 'phase_ms': phase_ms, 'buffer_sets': nsets,
@@ -293,12 +302,16 @@ def model_inference(batch=128, steps=10, warmup=3):
     with torch.no_grad():
         for _ in range(warmup):
             model(x)
-        ms = timed(lambda i: model(x), steps)
+        ms = timed_blocks(lambda i: model(x), steps)[1]
         layers = ddf_resnet.time_ddf_layers(model, x)
     ddf_ms = sum(l['ms'] for l in layers)
-    return {'model': 'ddf_mul_resnet50', 'batch': batch, 'dtype': 'f16',
+    ddf_bytes = sum(l['bytes'] for l in layers)
+    return {'model': 'ddf_mul_resnet50', 'batch': batch, 'dtype': 'f16', 'input': [batch, 3, 224, 224],
+            'weights': 'random (Kaiming normal, BatchNorm at default init)',
             'images_per_s': round(batch / (ms * 1e-3), 1), 'ms_per_batch': round(ms, 3),
-            'ddf_ms_per_batch': round(ddf_ms, 3), 'ddf_layers': layers}
+            'ddf_ms_per_batch': round(ddf_ms, 3),
+            'ddf_gbps': round(ddf_bytes / (ddf_ms * 1e-3) / 1e9, 1) if ddf_ms else None,
+            'ddf_layers': layers}
 
 
 def test_time_table(iters=20, warmup=5):
@@ -387,14 +400,46 @@ def up_forward_table(lib, iters=50, warmup=10):
     return rows
 
 
+def roofline_of(res):
+    """Roofline object of a workload: the slower call of its step (forward or
+    backward), algorithmic bytes of that call / its median launch time."""
+    dominant = max(STEP_PHASES, key=lambda p: res['phase_ms'][p])
+    nbytes = res['bytes'][dominant]
+    sec = res['phase_ms'][dominant] * 1e-3
+    achieved = nbytes / sec / 1e9
+    traffic, source = profiled_traffic(res['workload'], dominant, res['kernels'][dominant])
+    return {'bound': 'hbm', 'phase': dominant, 'kernel': res['kernels'][dominant],
+            'achieved': round(achieved, 2), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+            'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': traffic,
+            'traffic_source': source, 'bytes_per_launch': nbytes,
+            'avg_launch_us': round(sec * 1e6, 3)}
+
+
+def workload_summary(r):
+    """What the JSON line carries for a workload other than the headline one."""
+    return {
+        'config': '%s: N=%d C=%d H=W=%d k=%d d=%d s=%d %s %s' % (
+            r['workload'], r['N'], r['C'], r['H'], r['k'], r['d'], r['s'], r['combine'], r['dtype']),
+        'gbps': round(r['gbps'], 1), 'pct_of_hbm_peak': round(100 * r['gbps'] / HBM_PEAK_GBPS, 2),
+        'us_per_step': round(r['ms_per_step'] * 1e3, 2),
+        'us_per_step_median': round(r['ms_per_step_median'] * 1e3, 2),
+        'images_per_s': round(r['images_per_s'], 1),
+        'bytes_per_step': r['bytes']['fwd'] + r['bytes']['bwd'],
+        'phases_us': {p: round(r['phase_ms'][p] * 1e3, 2) for p in PHASES},
+        'phases_pct_of_hbm_peak': {p: round(100 * r['phase_gbps'][p] / HBM_PEAK_GBPS, 1) for p in PHASES},
+        'kernels': r['kernels'], 'roofline': roofline_of(r)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=200)
+    ap.add_argument('--steps', type=int, default=100)
     ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--workload', default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
-    ap.add_argument('--all', action='store_true', help='also time the other workloads')
-    ap.add_argument('--model', action='store_true', help='also time ddf_mul_resnet50 inference')
+    ap.add_argument('--only-headline', action='store_true',
+                    help='time the headline workload only (no other workloads, no model)')
+    ap.add_argument('--all', action='store_true', help='(default now; kept for old command lines)')
+    ap.add_argument('--model', action='store_true', help='(default now; kept for old command lines)')
     ap.add_argument('--test-time', action='store_true',
                     help="also run the reference's micro-benchmark table (conv, depthwise conv, "
                          "DDFPack, ddf at seven 256-channel shapes)")
@@ -413,20 +458,13 @@ def main():
     from ddfnet_amd import _lib as lib
     lib.lib()
 
+    res = run_workload(args.workload, args.steps, args.warmup, lib, copy_probe=args.copy_probe)
     extra = {}
-    if args.all:
+    if not args.only_headline:
         for name in WORKLOADS:
             if name != args.workload:
                 extra[name] = run_workload(name, args.steps, args.warmup, lib)
-    res = run_workload(args.workload, args.steps, args.warmup, lib, copy_probe=args.copy_probe)
 
-    dominant = max(STEP_PHASES, key=lambda p: res['phase_ms'][p])
-    dom_bytes = res['bytes'][dominant]
-    dom_s = res['phase_ms'][dominant] * 1e-3
-    achieved = dom_bytes / dom_s / 1e9
-    kernel_label = PHASE_KERNELS[dominant]
-    if dominant == 'bwd' and res['workload'] not in FUSED_BWD_WORKLOADS:
-        kernel_label = UNFUSED_BWD
     line = {
         'metric': 'ddf_fwd_bwd_hbm_gbps', 'value': round(res['gbps'], 2), 'unit': 'GB/s',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
@@ -437,23 +475,16 @@ def main():
             res['combine'], res['dtype']),
             'bytes_per_step': res['bytes']['fwd'] + res['bytes']['bwd'],
             'buffer_sets': res['buffer_sets']},
+        'ms_per_step_median': round(res['ms_per_step_median'], 6),
         'pct_of_hbm_peak': round(100 * res['gbps'] / HBM_PEAK_GBPS, 2),
         'images_per_s': round(res['images_per_s'], 1),
-        'roofline': {'bound': 'hbm', 'phase': dominant, 'kernel': kernel_label, 'achieved': round(achieved, 2),
-                     'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-                     'frac': round(achieved / HBM_PEAK_GBPS, 4),
-                     'traffic': MEASURED_TRAFFIC.get(res['workload'], {}).get(dominant),
-                     'bytes_per_launch': dom_bytes,
-                     'avg_launch_us': round(dom_s * 1e6, 3)},
+        'roofline': roofline_of(res),
         'phases_us': {p: round(res['phase_ms'][p] * 1e3, 3) for p in PHASES},
+        'kernels': res['kernels'],
     }
     if extra:
-        line['other_workloads'] = {
-            n: {'gbps': round(r['gbps'], 1), 'us_per_step': round(r['ms_per_step'] * 1e3, 2),
-                'images_per_s': round(r['images_per_s'], 1),
-                'phases_us': {p: round(r['phase_ms'][p] * 1e3, 2) for p in PHASES}}
-            for n, r in extra.items()}
-    if args.model:
+        line['other_workloads'] = {n: workload_summary(r) for n, r in extra.items()}
+    if not args.only_headline:
         line['model_inference'] = model_inference()
         mi = line['model_inference']
         log('[model] %s bs%d %s: %.1f images/s (%.2f ms/batch, DDF layers %.2f ms)' % (

@@ -24,6 +24,7 @@ SYMBOLS = {
     'ddf_hip_version': (_i, []),
     'ddf_hip_status_string': (ctypes.c_char_p, [_i]),
     'ddf_hip_last_error': (ctypes.c_char_p, []),
+    'ddf_hip_describe': (_i, [_i64] * 4 + [_i] * 5 + [_u, _i, ctypes.c_char_p, _i]),
     'ddf_hip_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 6 + [_vp]),
     'ddf_hip_backward_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u, _i]),
     'ddf_hip_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
@@ -100,6 +101,15 @@ class on_device_of(object):
         if self.guard is not None:
             self.guard.__exit__(*exc)
         return False
+
+
+def describe(shape, k, d, s, combine, dtype, need=0, variant=''):
+    """Names of the kernels a forward (need = 0) or backward call launches."""
+    N, C, H, W = shape
+    buf = ctypes.create_string_buffer(256)
+    check(lib().ddf_hip_describe(N, C, H, W, k, d, s, COMBINE[combine], DTYPE[dtype], need,
+                                 VARIANT[variant], buf, len(buf)))
+    return buf.value.decode()
 
 
 def forward(features, channel_filter, spatial_filter, output, k, d, s, combine, variant=''):

@@ -167,6 +167,30 @@ const char *ddf_hip_status_string(int status) {
 
 const char *ddf_hip_last_error(void) { return g_last_error; }
 
+int ddf_hip_describe(int64_t N, int64_t C, int64_t H, int64_t W, int kernel_size, int dilation,
+                     int stride, int combine, int dtype, unsigned need_mask, int variant,
+                     char *buffer, int buffer_len) {
+    if (!buffer || buffer_len <= 0) return fail(DDF_ERR_BAD_ARG, "no buffer for the description");
+    buffer[0] = 0;
+    int rc = check_problem(N, C, H, W, kernel_size, dilation, stride, combine, dtype, variant);
+    if (rc != DDF_OK) return rc;
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
+    if (N * C * p.Ho * p.Wo == 0) { snprintf(buffer, buffer_len, "nothing"); return DDF_OK; }
+    const unsigned need = need_mask & DDF_NEED_ALL;
+    if (need == 0) {
+        if (variant == DDF_VARIANT_GENERIC || !ddf::tiled_forward_supported(p, dtype))
+            snprintf(buffer, buffer_len, "generic_forward");
+        else
+            ddf::describe_forward(p, dtype, buffer, buffer_len);
+    } else {
+        if (variant == DDF_VARIANT_GENERIC || !ddf::tiled_backward_supported(p, dtype))
+            snprintf(buffer, buffer_len, "generic_backward");
+        else
+            ddf::describe_backward(p, dtype, need, buffer, buffer_len);
+    }
+    return DDF_OK;
+}
+
 int ddf_hip_forward(const void *features, const void *channel_filter,
                     const void *spatial_filter, void *output, int64_t N, int64_t C,
                     int64_t H, int64_t W, int kernel_size, int dilation, int stride,

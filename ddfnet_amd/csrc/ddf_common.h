@@ -112,6 +112,11 @@ template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
                                T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st);
 
+// Names of the kernels a forward / backward call on the tiled families would
+// launch, written into buf (at most len bytes); returns snprintf's count.
+int describe_forward(const Problem &p, int dtype, char *buf, int len);
+int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int len);
+
 bool tiled_forward_supported(const Problem &p, int dtype);
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,

@@ -150,6 +150,7 @@ def time_ddf_layers(model, x, iters=20):
             n, c, h, w = feat.shape
             esz = feat.element_size()
             nbytes = esz * (feat.numel() + n * c * (h // s) * (w // s) + cf.numel() + sf.numel())
-            out.append({'shape': [n, c, h, w], 'stride': s, 'ms': round(ms, 4),
-                        'gbps': round(nbytes / (ms * 1e-3) / 1e9, 1)})
+            out.append({'shape': [n, c, h, w], 'stride': s, 'ms': round(ms, 4), 'bytes': nbytes,
+                        'gbps': round(nbytes / (ms * 1e-3) / 1e9, 1),
+                        'pct_of_hbm_peak': round(nbytes / (ms * 1e-3) / 8e12 * 100, 1)})
     return out

@@ -81,6 +81,18 @@ const char *ddf_hip_status_string(int status);
 const char *ddf_hip_last_error(void);
 
 /*
+ * Names of the kernels a call with these arguments launches, as text in
+ * `buffer` (diagnostics for benchmarks and profiles; no counterpart in the
+ * reference).  need_mask 0 describes ddf_hip_forward, anything else
+ * ddf_hip_backward with that mask.  Pointer alignment, which can send a call
+ * to the scalar-access kernels, is assumed to be 16 bytes.
+ */
+int ddf_hip_describe(int64_t N, int64_t C, int64_t H, int64_t W,
+                     int kernel_size, int dilation, int stride, int combine,
+                     int dtype, unsigned need_mask, int variant, char *buffer,
+                     int buffer_len);
+
+/*
  * Forward pass.  Replaces `forward(features, channel_filter, spatial_filter,
  * kernel_size, dilation, stride, output)` of ddf_{mul,add}{,_faster}_ext
  * (ddf/src/ddf_mul_ext.cpp:21-34, ddf/src/ddf_mul_faster_ext.cpp:13-26).

@@ -148,6 +148,27 @@ def test_resnet50_forward_matches_cpu_reference(monkeypatch):
     assert (out.cpu().double() - out_r).abs().max().item() <= 1e-3 * scale
 
 
+def test_resnet50_fp16_forward_matches_cpu_reference(monkeypatch):
+    """The same network in fp16 on the GPU (the dtype of the batch-128 inference
+    configuration; every DDF layer then runs the fp16 kernels) against the CPU
+    fp64 model holding the same fp16-rounded weights and input.  Tolerance 2e-2
+    of the largest logit: 50+ layers of fp16 activations and BatchNorm, of which
+    the DDF layers are held to 1e-2 each at operator level."""
+    from ddfnet_amd import ddf_resnet
+    torch.manual_seed(5)
+    model = ddf_resnet.ddf_mul_resnet50(num_classes=10).cuda().half().eval()
+    x = torch.randn(2, 3, 64, 64, device='cuda').half()
+    with torch.no_grad():
+        out = model(x)
+        assert out.dtype == torch.float16 and out.shape == (2, 10)
+        ref = copy.deepcopy(model).cpu().double()
+        monkeypatch.setattr(ddf_modules, 'ddf', _OracleOp())
+        out_r = ref(x.cpu().double())
+    assert torch.isfinite(out).all()
+    scale = out_r.abs().max().item()
+    assert (out.cpu().double() - out_r).abs().max().item() <= 2e-2 * scale
+
+
 def test_resnet50_fp16_inference_and_layer_timing():
     from ddfnet_amd import ddf_resnet
     torch.manual_seed(4)
