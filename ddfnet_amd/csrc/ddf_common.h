@@ -105,12 +105,14 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
                        T *out, hipStream_t st);
 
 // Filter gradients (dCF, dSF) on the row-register kernel; same conventions.
-// The workspace (rows_filters_workspace bytes, 256-byte aligned) holds the
-// partial sums over channel splits and strips.
+// With dx != nullptr the launch also writes the feature gradient (small planes:
+// the whole backward pass in one kernel).  The workspace
+// (rows_filters_workspace bytes, 256-byte aligned) holds the partial sums over
+// channel splits and strips.
 size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);
 template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
-                               T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st);
+                               T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st);
 
 // Names of the kernels a forward / backward call on the tiled families would
 // launch, written into buf (at most len bytes); returns snprintf's count.

@@ -49,15 +49,23 @@ __device__ __forceinline__ void wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <typename T, int K, int D, bool MUL, int VX, int R, bool PAD, int NST, int WPE>
+// DX: the same walk also produces the feature gradient (as k_rows<BWD> does):
+// dO then comes in with its rows above and below as well, the lane keeps a
+// second set of spatial taps (those of the pixels its dO values come from),
+// and every channel ends with the store of its dX rows.  One launch for the
+// whole backward pass; dO, CF and SF are read once.
+template <typename T, int K, int D, bool MUL, int VX, int R, bool PAD, bool DX, int NST, int WPE>
 __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     RowsGeom g, const T *__restrict__ go, const T *__restrict__ x, const T *__restrict__ cf,
-    const T *__restrict__ sf, T *__restrict__ dcf, T *__restrict__ dsf,
+    const T *__restrict__ sf, T *__restrict__ dx, T *__restrict__ dcf, T *__restrict__ dsf,
     typename Acc<T>::type *__restrict__ ws_sf, typename Acc<T>::type *__restrict__ ws_cf,
     unsigned need) {
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RAD = K / 2, HX = RAD * D, HY = RAD * D;
     constexpr int ROWS = R + 2 * HY;
+    constexpr int GROWS = DX ? ROWS : R;       // dO rows a lane loads per channel
+    constexpr int GOWN = DX ? HY : 0;          // its own first row among them
+    constexpr bool kFilters = MUL || DX;       // CF and SF values are needed at all
     constexpr int NW = VX * sizeof(T) / 4;
     constexpr int G = kFlushChannels;
     using Row = ExtRow<T, VX, HX, PAD>;
@@ -80,6 +88,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 
     const T *xs = x + (wk.n * g.C + c_first) * plane;
     const T *gs = go + (wk.n * g.C + c_first) * plane;
+    T *ds = DX ? dx + (wk.n * g.C + c_first) * plane : nullptr;
     uint32_t xb[ROWS], ob[R];
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr)
@@ -94,9 +103,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     // past the wave's last one reads zeros (empty descriptors) and so adds nothing;
     // idle lanes and rows outside the image read zeros as well.
     constexpr bool kScalarTaps = sizeof(T) >= 4;   // (see k_rows)
-    uint32_t xw[NST][ROWS][NW], gw[NST][R][NW];
+    uint32_t xw[NST][ROWS][NW], gw[NST][GROWS][NW];
     T cfl[NST];
-    A cfu[NST][kScalarTaps && MUL ? KK : 1];
+    A cfu[NST][kScalarTaps && kFilters ? KK : 1];
     auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         const uint32_t bytes = ci < nch ? plane_bytes : 0u;
@@ -105,8 +114,8 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr) load_words<NW>(pr, xb[rr], xw[ST][rr]);
 #pragma unroll
-        for (int r = 0; r < R; ++r) load_words<NW>(gr, ob[r], gw[ST][r]);
-        if constexpr (MUL) {
+        for (int r = 0; r < GROWS; ++r) load_words<NW>(gr, DX ? xb[r] : ob[r], gw[ST][r]);
+        if constexpr (kFilters) {
             const int cc = ci < nch ? ci : (nch > 0 ? nch - 1 : 0);
             if constexpr (kScalarTaps) {
 #pragma unroll
@@ -130,6 +139,30 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
             for (int r = 0; r < R; ++r) load_words<NW>(sr, ob[r], sfw[r][t]);
         }
+    }
+    // (DX) spatial taps at the pixels the lane's dO values come from: slot (i, j)
+    // holds tap (K-1-i, K-1-j) of the pixel (i-RAD)*D rows and (j-RAD)*D columns
+    // away, zero where that pixel does not exist (see k_rows)
+    uint32_t sfg[DX ? R : 1][KK][NW];
+    if constexpr (DX) {
+        const T *sfn = sf + wk.n * KK * plane;
+#pragma unroll
+        for (int i = 0; i < K; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                const __amdgpu_buffer_rsrc_t sr =
+                    plane_rsrc(sfn + ((K - 1 - i) * K + (K - 1 - j)) * plane, plane_bytes);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    Row row;
+                    load_words<NW>(sr, xb[r + i * D], row.own);
+                    row.sides(ln.first, ln.last);
+                    A v[VX];
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) v[e] = row.at(e + j * D - HX);
+                    pack<T, VX, A>(v, sfg[r][i * K + j]);
+                }
+            }
     }
     A acc_sf[R][KK][VX];
 #pragma unroll
@@ -171,14 +204,17 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 
     auto compute = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
-        if constexpr (sizeof(T) == 2 && MUL) {
+        if constexpr (sizeof(T) == 2) {
             // keep the packed taps packed (see k_rows)
 #pragma unroll
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int t = 0; t < KK; ++t)
 #pragma unroll
-                    for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfw[r][t][k]));
+                    for (int k = 0; k < NW; ++k) {
+                        if constexpr (MUL) asm volatile("" : "+v"(sfw[r][t][k]));
+                        if constexpr (DX) asm volatile("" : "+v"(sfg[r][t][k]));
+                    }
         }
         Row row[ROWS];
 #pragma unroll
@@ -191,9 +227,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int e = 0; e < VX; ++e) gval[r][e] = elem<T>(gw[ST][r], e);
+            for (int e = 0; e < VX; ++e) gval[r][e] = elem<T>(gw[ST][GOWN + r], e);
         A w[KK];
-        if constexpr (MUL) {
+        if constexpr (kFilters) {
             if constexpr (kScalarTaps) {
 #pragma unroll
                 for (int t = 0; t < KK; ++t) w[t] = cfu[ST][t];
@@ -224,6 +260,47 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                             pcf[t] += gx;
                         }
                     }
+        if constexpr (DX) {
+            // feature gradient of the lane's pixels: dO at the flipped tap offsets
+            Row grow[ROWS];
+#pragma unroll
+            for (int rr = 0; rr < ROWS; ++rr) {
+#pragma unroll
+                for (int k = 0; k < NW; ++k) grow[rr].own[k] = gw[ST][rr][k];
+                grow[rr].sides(ln.first, ln.last);
+            }
+            const __amdgpu_buffer_rsrc_t dr = plane_rsrc(ds + (int64_t)ci * plane, ci < nch ? plane_bytes : 0u);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                A accx[VX];
+#pragma unroll
+                for (int e = 0; e < VX; ++e) accx[e] = 0;
+#pragma unroll
+                for (int i = 0; i < K; ++i)
+#pragma unroll
+                    for (int j = 0; j < K; ++j)
+#pragma unroll
+                        for (int e = 0; e < VX; ++e) {
+                            const int t = i * K + j;
+                            const A gv = grow[r + i * D].at(e + j * D - HX);
+                            const A sv = elem<T>(sfg[r][t], e);
+                            if constexpr (MUL) {
+                                accx[e] = fma_(w[KK - 1 - t], fma_(gv, sv, A(0)), accx[e]);
+                            } else {
+                                accx[e] = fma_(gv, w[KK - 1 - t], accx[e]);
+                                accx[e] = fma_(gv, sv, accx[e]);
+                            }
+                        }
+                if constexpr (sizeof(T) == 2) {
+                    // round the complete fp32 sum, the same way in every unrolled copy (see k_rows)
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) asm volatile("" : "+v"(accx[e]));
+                }
+                uint32_t ow[NW];
+                pack<T, VX, A>(accx, ow);
+                store_words_nt<NW>(dr, ob[r], ow);
+            }
+        }
         if (want_cf && ci < nch) {
             const int slot = ci & (G - 1);
 #pragma unroll
@@ -312,7 +389,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 // Host-side geometry of k_rows_filters (ddf_rows_host.hip): a work item is a
 // workgroup of rows::kFilterWaves waves (g->wpb = 1) that covers g->cpb =
 // g->cpw * rows::kFilterWaves channels; g->csplit counts those ranges.
-bool rows_filters_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx, int *r);
+// fused: the geometry of the launch that also writes the feature gradient
+// (covers small planes only).
+bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g, int *vx, int *r);
 // Workspace the kernel needs (layout as the tile kernels': dSF partials over
 // channel splits, then dCF partials over strips, each 256-byte aligned).
 size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);

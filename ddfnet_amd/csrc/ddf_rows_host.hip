@@ -109,15 +109,15 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     return true;
 }
 
-// Instantiated (elements per lane and row, rows per lane) of k_rows_filters.
-bool rows_filters_variant_built(int esz, int vx, int r) {
-    if (r != 1) return false;
-    if (esz == 2) return vx == 4 || vx == 2;
-    if (esz == 4) return vx == 4 || vx == 2;
-    return false;
+// Instantiated (elements per lane and row, rows per lane) of k_rows_filters;
+// fused: of the variant that also writes the feature gradient.
+bool rows_filters_variant_built(int esz, int vx, int r, bool fused) {
+    if (esz != 2 && esz != 4) return false;
+    if (fused) return (vx == 2 && r == 2) || (vx == 4 && r == 1);
+    return r == 1 && (vx == 4 || vx == 2);
 }
 
-bool rows_filters_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx_out,
+bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g, int *vx_out,
                            int *r_out) {
     if (!(p.s == 1 && p.k == 3 && p.d == 1)) return false;
     if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
@@ -126,15 +126,21 @@ bool rows_filters_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g,
     const int H = (int)p.H, W = (int)p.W, C = (int)p.C;
     const int hx = p.r * p.d;
     if ((int64_t)H * W * 8 >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
-    const int R = 1;
-    int vx = 0;
-    for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
-        if (max_vx > 0 && cand > max_vx) continue;
+    // One launch for the whole backward pass pays where the plane is small: the
+    // launches are then bound by ramp and latency, not by bytes or arithmetic.
+    if (fused && (H * W > tune_int("DDF_TUNE_ROWSF_FUSED_PLANE", 400) ||
+                  tune_int("DDF_TUNE_ROWSF_FUSED", 1) == 0))
+        return false;
+    int vx = 0, R = 1;
+    for (int cand = std::min(16 / esz, 4); cand * esz >= 4; cand /= 2) {
         if (cand > tune_int("DDF_TUNE_ROWSF_VX", 16)) continue;
-        if (!rows_filters_variant_built(esz, cand, R)) continue;
         if (W % cand != 0 || cand < hx) continue;
         if (W / cand > 32) continue;
+        // two rows per lane where a row is a few 2-pixel vectors (14 x 14: one strip per plane)
+        const int r = (fused && cand == 2 && H % 2 == 0) ? 2 : 1;
+        if (!rows_filters_variant_built(esz, cand, r, fused)) continue;
         vx = cand;
+        R = r;
         break;
     }
     if (vx == 0) return false;
@@ -176,15 +182,21 @@ bool rows_filters_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g,
 
 size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need) {
     if (!(need & (DDF_NEED_DCF | DDF_NEED_DSF))) return 0;
-    RowsGeom g; int vx, r;
-    if (!rows_filters_geometry(p, dtype, 0, &g, &vx, &r)) return 0;
     const size_t asz = dtype == DDF_F64 ? 8 : 4;
-    size_t bytes = 0;
-    if ((need & DDF_NEED_DSF) && g.csplit > 1)
-        bytes += ((size_t)p.N * g.csplit * p.kk * p.H * p.W * asz + 255) / 256 * 256;
-    if ((need & DDF_NEED_DCF) && g.nstrips > 1)
-        bytes += ((size_t)p.N * p.C * g.nstrips * p.kk * asz + 255) / 256 * 256;
-    return bytes;
+    size_t most = 0;
+    // (room for either cut of the problem: which one runs also depends on pointer alignment)
+    for (int fused = 0; fused < 2; ++fused) {
+        RowsGeom g; int vx, r;
+        if (fused && !(need & DDF_NEED_DX)) continue;
+        if (!rows_filters_geometry(p, dtype, fused != 0, &g, &vx, &r)) continue;
+        size_t bytes = 0;
+        if ((need & DDF_NEED_DSF) && g.csplit > 1)
+            bytes += ((size_t)p.N * g.csplit * p.kk * p.H * p.W * asz + 255) / 256 * 256;
+        if ((need & DDF_NEED_DCF) && g.nstrips > 1)
+            bytes += ((size_t)p.N * p.C * g.nstrips * p.kk * asz + 255) / 256 * 256;
+        most = std::max(most, bytes);
+    }
+    return most;
 }
 
 }  // namespace ddf

@@ -83,23 +83,24 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
 
 namespace rows {
 
-template <typename T, int VX, int R>
+template <typename T, int VX, int R, bool DX>
 hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, const T *x,
-                            const T *cf, const T *sf, T *dcf, T *dsf,
+                            const T *cf, const T *sf, T *dx, T *dcf, T *dsf,
                             typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                             unsigned need, hipStream_t st) {
     using A = typename Acc<T>::type;
-    // waves per SIMD the registers are budgeted for: 'mul' keeps the spatial taps as well
-    constexpr int WPE_MUL = VX * R >= 4 ? 2 : 3, WPE_ADD = 3;
+    // waves per SIMD the registers are budgeted for: 'mul' keeps the spatial taps
+    // as well, the fused feature gradient a second set of them
+    constexpr int WPE_MUL = (DX || VX * R >= 4) ? 2 : 3, WPE_ADD = DX ? 2 : 3;
     constexpr int kFilterStages = 2;   // channels in flight per wave
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kFilterWaves);
     const int lds = filters_lds_bytes<9>((int)sizeof(A), R, VX);
     if (p.k != 3 || p.d != 1) return hipErrorNotSupported;
     const bool pad = g.lp > g.lpr;
 #define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
-    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, R, PAD_, kFilterStages,                \
+    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, R, PAD_, DX, kFilterStages,            \
                                        MUL_ ? WPE_MUL : WPE_ADD>),                               \
-                       grid, block, lds, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need)
+                       grid, block, lds, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need)
     if (p.mul) {
         if (pad) DDF_ROWSF_CASE(true, true);
         else DDF_ROWSF_CASE(true, false);
@@ -113,19 +114,22 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
 
 }  // namespace rows
 
-// Filter gradients on the row-register kernel, partial sums included.
+// Filter gradients on the row-register kernel, partial sums included; with
+// dx != nullptr the same launch also writes the feature gradient (small planes
+// only: rows_filters_geometry(..., fused = true) must cover the problem).
 // hipErrorNotSupported: not covered (nothing was launched).  `ws` must hold
 // rows_filters_workspace() bytes.
 template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
-                               T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st) {
+                               T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st) {
     using A = typename Acc<T>::type;
     const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
+    const bool fused = dx != nullptr;
     RowsGeom g;
     int vx, r;
-    if (!rows_filters_geometry(p, dtype, 0, &g, &vx, &r)) return hipErrorNotSupported;
+    if (!rows_filters_geometry(p, dtype, fused, &g, &vx, &r)) return hipErrorNotSupported;
     const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
-    if ((((uintptr_t)x | (uintptr_t)go | (uintptr_t)sf | (uintptr_t)dsf) & mask) != 0)
+    if ((((uintptr_t)x | (uintptr_t)go | (uintptr_t)sf | (uintptr_t)dsf | (uintptr_t)dx) & mask) != 0)
         return hipErrorNotSupported;
     unsigned char *wp = static_cast<unsigned char *>(ws);
     A *ws_sf = nullptr, *ws_cf = nullptr;
@@ -137,10 +141,17 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     if ((need & DDF_NEED_DCF) && g.nstrips > 1) ws_cf = reinterpret_cast<A *>(wp);
     hipError_t err = hipErrorNotSupported;
     if constexpr (sizeof(T) != 8) {
-        if (vx == 4 && r == 1)
-            err = rows::launch_filters_v<T, 4, 1>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
-        else if (vx == 2 && r == 1)
-            err = rows::launch_filters_v<T, 2, 1>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+        if (fused) {
+            if (vx == 2 && r == 2)
+                err = rows::launch_filters_v<T, 2, 2, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+            else if (vx == 4 && r == 1)
+                err = rows::launch_filters_v<T, 4, 1, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+        } else {
+            if (vx == 4 && r == 1)
+                err = rows::launch_filters_v<T, 4, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+            else if (vx == 2 && r == 1)
+                err = rows::launch_filters_v<T, 2, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+        }
     }
     if (err != hipSuccess) return err;
     if (ws_sf) {
@@ -153,7 +164,8 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
 
 #define DDF_INSTANTIATE_ROWS(T)                                                              \
     template hipError_t rows_filters_launch<T>(const Problem &, const T *, const T *, const T *, \
-                                               const T *, T *, T *, void *, unsigned, hipStream_t); \
+                                               const T *, T *, T *, T *, void *, unsigned,   \
+                                               hipStream_t);                                  \
     template hipError_t rows_launch<T>(const Problem &, bool, const T *, const T *, const T *, \
                                        T *, hipStream_t);
 

@@ -3,8 +3,6 @@
 #include <algorithm>
 #include <cstdlib>
 
-#include <cstdio>
-
 #include "ddf_rows_filters.h"
 #include "ddf_wave.h"
 
@@ -278,65 +276,6 @@ size_t wave_backward_workspace(const Problem &p, int dtype, unsigned need) {
     if ((need & DDF_NEED_DCF) && g.nstrips > 1)
         bytes += ((size_t)p.N * p.C * g.nstrips * p.kk * asz + 255) / 256 * 256;
     return bytes;
-}
-
-// Which kernels a call would launch, in words (pointer alignment assumed).
-// Mirrors the choices of tiled_forward / tiled_backward in ddf_tiled_launch.h.
-int describe_forward(const Problem &p, int dtype, char *buf, int len) {
-    RowsGeom rg; int vx, r;
-    WaveGeom wg; int ps, nv;
-    if (small_supported(p)) return snprintf(buf, len, "k_small");
-    if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 && rows_geometry(p, dtype, 0, &rg, &vx, &r))
-        return snprintf(buf, len, "k_rows<VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
-    if (wave_geometry(p, dtype, kWaveForward, 0, &wg, &ps, &nv))
-        return snprintf(buf, len, "k_forward<PS=%d,NV=%d,V=%d>", ps, nv, wg.vec);
-    return snprintf(buf, len, "generic_forward");
-}
-
-int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int len) {
-    RowsGeom rg; int vx, r;
-    WaveGeom wg, gp; int ps, nv, pps, pnv;
-    const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
-    int n = 0;
-    auto add = [&](const char *fmt, auto... args) {
-        if (n < len) n += snprintf(buf + n, len - n, fmt, args...);
-    };
-    if (len > 0) buf[0] = 0;
-    const bool tiled = wave_geometry(p, dtype, kWaveFeatures, 0, &wg, &ps, &nv) &&
-                       wave_geometry(p, dtype, kWaveFilters, 0, &wg, &ps, &nv);
-    if (!tiled) { add("%s", "generic_backward"); return n; }
-    const bool fuse = (need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_FUSED", 1) != 0 &&
-                      wave_geometry(p, dtype, kWaveFused, 0, &wg, &ps, &nv) &&
-                      wave_geometry(p, dtype, kWaveFilters, 0, &gp, &pps, &pnv) && gp.TH == wg.TH &&
-                      gp.csplit == wg.csplit;
-    if (fuse) {
-        add("%s", "k_backward_filters<DX>");
-        if ((fneed & DDF_NEED_DSF) && wg.csplit > 1) add("%s", " + k_sum_partials");
-        if ((fneed & DDF_NEED_DCF) && wg.nstrips > 1) add("%s", " + k_sum_partials");
-        return n;
-    }
-    if (need & DDF_NEED_DX) {
-        if (!small_supported(p) && dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
-            rows_geometry(p, dtype, 0, &rg, &vx, &r))
-            add("k_rows<dX,VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
-        else if (small_supported(p)) add("%s", "k_small<dX>");
-        else add("%s", "k_backward_features");
-    }
-    if (fneed) {
-        if (n) add("%s", " + ");
-        if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
-            rows_filters_geometry(p, dtype, 0, &rg, &vx, &r)) {
-            add("k_rows_filters<VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
-            if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
-            if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
-        } else {
-            wave_geometry(p, dtype, kWaveFilters, 0, &wg, &ps, &nv);
-            add("%s", "k_backward_filters");
-            if ((fneed & DDF_NEED_DSF) && wg.csplit > 1) add("%s", " + k_sum_partials");
-            if ((fneed & DDF_NEED_DCF) && wg.nstrips > 1) add("%s", " + k_sum_partials");
-        }
-    }
-    return n;
 }
 
 }  // namespace ddf

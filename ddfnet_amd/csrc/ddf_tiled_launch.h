@@ -176,6 +176,14 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
     // One launch for all gradients where the fused kernel exists and cuts the
     // problem exactly as the workspace was sized for.
+    if constexpr (sizeof(T) != 8) {
+        // small planes: the row-register kernel does the whole backward pass in one launch
+        if ((need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_ROWSF", 1) != 0) {
+            err = rows_filters_launch<T>(p, go, x, cf, sf, dx, dcf, dsf, ws, fneed, st);
+            if (err != hipErrorNotSupported) return err;
+            err = hipSuccess;
+        }
+    }
     WaveGeom g; int ps, nv;
     bool fuse = false;
     if ((need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_FUSED", 1) != 0) {
@@ -205,7 +213,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     if (fneed && !fuse) {
         if constexpr (sizeof(T) != 8) {
             if (tune_int("DDF_TUNE_ROWSF", 1) != 0) {
-                err = rows_filters_launch<T>(p, go, x, cf, sf, dcf, dsf, ws, fneed, st);
+                err = rows_filters_launch<T>(p, go, x, cf, sf, (T *)nullptr, dcf, dsf, ws, fneed, st);
                 if (err != hipErrorNotSupported) return err;
                 err = hipSuccess;
             }

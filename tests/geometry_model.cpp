@@ -239,11 +239,11 @@ static void replay_rows(const RowsGeom &g, long N, long C, bool filters) {
             if (!seen[i]) { CHECK(false, "work item %ld never handed out", i); break; }
 }
 
-static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, bool filters) {
+static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, bool filters, bool fused = false) {
     const Problem p = make_problem(N, C, H, W, k, d, 1, 0);
     RowsGeom g;
     int vx, r;
-    const bool ok = filters ? rows_filters_geometry(p, dtype, 0, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r);
+    const bool ok = filters ? rows_filters_geometry(p, dtype, fused, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r);
     if (!ok) {
         printf("kind rows%s %ldx%ldx%ldx%ld k%d d%d dt%d: unsupported\n", filters ? "-filters" : "", N, C, H, W, k, d, dtype);
         return;
@@ -290,8 +290,8 @@ int main() {
     for (auto &sh : shapes)
         for (int d = 1; d <= 2; ++d)
             for (int dtype = 0; dtype < 3; ++dtype)
-                for (int filters = 0; filters < 2; ++filters)
-                    check_rows(sh[0], sh[1], sh[2], sh[3], 3, d, dtype, filters != 0);
+                for (int filters = 0; filters < 3; ++filters)
+                    check_rows(sh[0], sh[1], sh[2], sh[3], 3, d, dtype, filters != 0, filters == 2);
     // seeded random shapes on top of the fixed list
     unsigned long long state = 0x9E3779B97F4A7C15ull;
     auto next = [&](int lo, int hi) {
