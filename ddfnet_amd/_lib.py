@@ -28,6 +28,7 @@ SYMBOLS = {
     'ddf_hip_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 6 + [_vp]),
     'ddf_hip_backward_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u, _i]),
     'ddf_hip_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
+    'ddf_hip_backward_static': (_i, [_vp] * 7 + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
     'ddf_hip_filter_norm': (_i, [_vp] * 2 + [_i64] * 2 + [_i, _i64, ctypes.c_double] + [_vp] * 2 +
                             [_i, _vp]),
     'ddf_hip_filter_norm_backward': (_i, [_vp] * 4 + [_i64] * 2 + [_i, _i64, ctypes.c_double, _vp,

@@ -1,11 +1,19 @@
 // C ABI of the DDF HIP library: argument validation and kernel-family choice.
 // Declarations and the reference entry points each call replaces are in
 // include/ddf_hip.h.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "ddf_common.h"
+
+// Scratch of ddf_hip_backward_static: device memory that belongs to the library's
+// code object, so that entry point never allocates.  Every GPU the library runs on
+// holds its own copy at its own address until the process ends.  (In host code
+// the name below is only a handle for hipGetSymbolAddress, not a device address.)
+static __device__ __align__(256) unsigned char scratch[DDF_HIP_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -97,6 +105,34 @@ int backward_typed(const ddf::Problem &p, const void *go, const void *x, const v
 }
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+
+// Address of `scratch` on the current device, looked up once per device (with
+// that device current) and kept.
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+int scratch_of_current_device(void **out) {
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return fail_hip(err, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(DDF_ERR_UNSUPPORTED, "device index %d beyond the %d this entry point keeps scratch for",
+                    dev, kMaxDevices);
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+        if (p == nullptr) {
+            err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (err != hipSuccess || p == nullptr)
+                return fail_hip(err, "hipGetSymbolAddress(scratch)");
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return DDF_OK;
+}
 
 // Workspace of the up-sampling backward: the lattices of dO, the per-branch
 // feature gradients (when dX is wanted) and one branch's own workspace.
@@ -269,6 +305,33 @@ int ddf_hip_backward(const void *grad_output, const void *features,
                                           grad_spatial_filter, workspace, workspace_bytes,
                                           dtype, need, variant, st);
     }
+}
+
+int ddf_hip_backward_static(const void *grad_output, const void *features,
+                            const void *channel_filter, const void *spatial_filter,
+                            void *grad_features, void *grad_channel_filter,
+                            void *grad_spatial_filter, int64_t N, int64_t C, int64_t H, int64_t W,
+                            int kernel_size, int dilation, int stride, int combine, int dtype,
+                            unsigned need_mask, int variant, void *stream) {
+    // the device's copy of the scratch array (first call on a device: looked up, no allocation)
+    void *ws = nullptr;
+    int rc = scratch_of_current_device(&ws);
+    if (rc != DDF_OK) return rc;
+    rc = check_problem(N, C, H, W, kernel_size, dilation, stride, combine, dtype, variant);
+    if (rc != DDF_OK) return rc;
+    const size_t want = ddf_hip_backward_workspace_bytes(N, C, H, W, kernel_size, dilation, stride,
+                                                         combine, dtype, need_mask, variant);
+    if (want > (size_t)DDF_HIP_STATIC_SCRATCH_BYTES)
+        return fail(DDF_ERR_WORKSPACE,
+                    "this problem needs %zu bytes of scratch; ddf_hip_backward_static holds %zu "
+                    "(use ddf_hip_backward with a workspace of your own)",
+                    want, (size_t)DDF_HIP_STATIC_SCRATCH_BYTES);
+    // Every partial sum the kernels read back from the scratch they have written in
+    // the same call, so what an earlier call left there needs no clearing.
+    return ddf_hip_backward(grad_output, features, channel_filter, spatial_filter, grad_features,
+                            grad_channel_filter, grad_spatial_filter, ws,
+                            (size_t)DDF_HIP_STATIC_SCRATCH_BYTES, N, C, H, W, kernel_size, dilation,
+                            stride, combine, dtype, need_mask, variant, stream);
 }
 
 int ddf_hip_filter_norm(const void *x, void *y, int64_t outer, int64_t groups, int taps,

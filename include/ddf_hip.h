@@ -137,6 +137,31 @@ int ddf_hip_backward(const void *grad_output, const void *features,
                      void *stream);
 
 /*
+ * ddf_hip_backward for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
+ * has no counterpart in the reference (whose backward takes caller-allocated
+ * scratch tensors, ddf/src/ddf_mul_ext.cpp:36-42).  Same arguments as
+ * ddf_hip_backward without the workspace: the partial sums go to a buffer of
+ * DDF_HIP_STATIC_SCRATCH_BYTES bytes that is part of the library's device
+ * image (every GPU the library runs on holds it until the process ends), and
+ * the call allocates and frees nothing.  A problem whose
+ * ddf_hip_backward_workspace_bytes() exceeds that size is rejected with
+ * DDF_ERR_WORKSPACE.  All calls on one GPU share the buffer: calls that
+ * overlap in time on the same GPU (different streams, different threads) race
+ * and must be serialised by the caller.  The first call on a device looks the
+ * buffer's address up (no allocation); make it outside a graph capture.
+ */
+#define DDF_HIP_STATIC_SCRATCH_BYTES (16u * 1024u * 1024u)
+int ddf_hip_backward_static(const void *grad_output, const void *features,
+                            const void *channel_filter,
+                            const void *spatial_filter, void *grad_features,
+                            void *grad_channel_filter,
+                            void *grad_spatial_filter, int64_t N, int64_t C,
+                            int64_t H, int64_t W, int kernel_size,
+                            int dilation, int stride, int combine, int dtype,
+                            unsigned need_mask, int variant, void *stream);
+
+/*
  * Filter normalisation of the two filter branches, one launch.  Restates
  * FilterNorm.forward of the reference (ddf/ddf.py:145-173), which is a chain
  * of elementwise and reduction ops there.  `x` and `y` are dense
