@@ -110,6 +110,9 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
 // (rows_filters_workspace bytes, 256-byte aligned) holds the partial sums over
 // channel splits and strips.
 size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);
+// The row-register kernels cover the feature gradient and, in a launch of its
+// own, the filter gradients of this problem (pointer alignment assumed).
+bool rows_cover_backward(const Problem &p, int dtype);
 template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
                                T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st);

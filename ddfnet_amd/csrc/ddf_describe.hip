@@ -2,7 +2,7 @@
 // tiled_forward / tiled_backward in ddf_tiled_launch.h, from the geometry alone.
 #include <cstdio>
 
-#include "ddf_rows_filters.h"
+#include "ddf_rows_taprow.h"
 #include "ddf_wave.h"
 
 namespace ddf {
@@ -32,7 +32,10 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
     const bool tiled = wave_geometry(p, dtype, kWaveFeatures, 0, &wg, &ps, &nv) &&
                        wave_geometry(p, dtype, kWaveFilters, 0, &wg, &ps, &nv);
     if (!tiled) { add("%s", "generic_backward"); return n; }
-    const bool fuse = (need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_FUSED", 1) != 0 &&
+    const bool rows_both = dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
+                           tune_int("DDF_TUNE_ROWSF", 1) != 0 && !small_supported(p) &&
+                           rows_cover_backward(p, dtype);
+    const bool fuse = (need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0 &&
                       wave_geometry(p, dtype, kWaveFused, 0, &wg, &ps, &nv) &&
                       wave_geometry(p, dtype, kWaveFilters, 0, &gp, &pps, &pnv) && gp.TH == wg.TH &&
                       gp.csplit == wg.csplit;
@@ -59,6 +62,11 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
     if (fneed) {
         if (n) add("%s", " + ");
         if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
+            rows_taprow_geometry(p, dtype, &rg, &vx, &r)) {
+            add("k_rows_taprow_filters<VX=%d,%s>", vx, rg.lp > rg.lpr ? "padded" : "plain");
+            if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
+            if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
+        } else if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
             rows_filters_geometry(p, dtype, false, &rg, &vx, &r)) {
             add("k_rows_filters<VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
             if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");

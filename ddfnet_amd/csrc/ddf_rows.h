@@ -71,10 +71,20 @@ __host__ __device__ __forceinline__ int magic_div(int n, unsigned m) {
 struct Work {
     int cs, strip, c_begin, c_end;
     int64_t n;
-    __host__ __device__ __forceinline__ bool init(const RowsGeom &g, int block, int wave) {
+    // Number of the work item of wave `wave` of workgroup `block`, -1: none.
+    __host__ __device__ static __forceinline__ int item_of(const RowsGeom &g, int block, int wave) {
         const int wg = (block % kXcd) * (int)g.xcd_per + block / kXcd;
         const int b = wg * g.wpb + wave;
-        if (wave >= g.wpb || b >= g.nwork) return false;
+        return (wave >= g.wpb || b >= g.nwork) ? -1 : b;
+    }
+    __host__ __device__ __forceinline__ bool init(const RowsGeom &g, int block, int wave) {
+        const int b = item_of(g, block, wave);
+        if (b < 0) return false;
+        decode(g, b);
+        return true;
+    }
+    // b: (sample, strip, channel range) number, channel range fastest
+    __host__ __device__ __forceinline__ void decode(const RowsGeom &g, int b) {
         const int rest = magic_div(b, g.csplit_magic);
         cs = b - rest * g.csplit;
         const int smp = magic_div(rest, g.nstrips_magic);
@@ -82,7 +92,6 @@ struct Work {
         n = smp;
         c_begin = cs * g.cpb;
         c_end = c_begin + g.cpb < g.C ? c_begin + g.cpb : g.C;
-        return true;
     }
 };
 
@@ -98,7 +107,8 @@ struct Lane {
     bool first, last;         // at the ends of an image row
     int xoff[ROWS];
     int ooff[R];
-    __host__ __device__ __forceinline__ void init(const RowsGeom &g, int strip, int lane) {
+    // dy: the window rows (xoff) are taken dy image rows further down
+    __host__ __device__ __forceinline__ void init(const RowsGeom &g, int strip, int lane, int dy = 0) {
         const int grp = magic_div(lane, g.lp_magic);
         const int v = lane - grp * g.lp;
         const bool live = grp < g.rg && v < g.lpr;
@@ -108,13 +118,24 @@ struct Lane {
         last = v == g.lpr - 1;
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr) {
-            const int yy = y0 - HY + rr;
+            const int yy = y0 - HY + rr + dy;
             xoff[rr] = (live && yy >= 0 && yy < g.H) ? yy * g.W + x0 : -1;
         }
 #pragma unroll
-        for (int r = 0; r < R; ++r) ooff[r] = xoff[HY + r];
+        for (int r = 0; r < R; ++r) ooff[r] = (live && y0 + r < g.H) ? (y0 + r) * g.W + x0 : -1;
     }
 };
+
+// Window row rr (0 = HY rows above the lane's first row) is touched by some tap
+// of some of the lane's R rows: rr = r + i*D.  With dilation the window has
+// rows no tap lands on; they are neither loaded nor shifted.
+template <int R, int K, int D>
+__host__ __device__ constexpr bool row_needed(int rr) {
+    for (int r = 0; r < R; ++r)
+        for (int i = 0; i < K; ++i)
+            if (r + i * D == rr) return true;
+    return false;
+}
 
 #ifdef __HIPCC__
 
@@ -143,6 +164,15 @@ __device__ __forceinline__ void load_words(__amdgpu_buffer_rsrc_t rsrc, uint32_t
     }
 }
 
+// f(integral_constant<int, I>) for I = 0 .. N-1, unrolled.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
 // Nontemporal: results are not read again by this kernel.
 template <int N>
 __device__ __forceinline__ void store_words_nt(__amdgpu_buffer_rsrc_t rsrc, uint32_t off, const uint32_t (&w)[N]) {
@@ -157,6 +187,23 @@ __device__ __forceinline__ void store_words_nt(__amdgpu_buffer_rsrc_t rsrc, uint
         typedef uint32_t v4 __attribute__((ext_vector_type(4)));
         v4 v = {w[0], w[1], w[2], w[3]};
         __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)off, 0, 2);
+    }
+}
+
+// One accumulator-type value, rounded to the storage type, to byte offset off
+// of the buffer.
+template <typename T>
+__device__ __forceinline__ void store_value(__amdgpu_buffer_rsrc_t rsrc, uint32_t off,
+                                            typename Acc<T>::type v) {
+    if constexpr (sizeof(T) == 2) {
+        const _Float16 h = (_Float16)v;
+        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, h), rsrc, (int)off, 0, 0);
+    } else if constexpr (sizeof(T) == 4) {
+        __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rsrc, (int)off, 0, 0);
+    } else {
+        typedef uint32_t v2 __attribute__((ext_vector_type(2)));
+        const v2 w = {(uint32_t)__double2loint(v), (uint32_t)__double2hiint(v)};
+        __builtin_amdgcn_raw_buffer_store_b64(w, rsrc, (int)off, 0, 0);
     }
 }
 
@@ -294,28 +341,6 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
     const int tl = lane < KK ? lane : KK - 1;   // lane t holds tap t of a channel (flipped for the gradient)
     const int tsel = BWD ? KK - 1 - tl : tl;
 
-    // feature rows and channel taps of channel ci, stage ST; a channel past the
-    // wave's last one reads zeros (empty descriptor)
-    uint32_t xw[NST][ROWS][NW];
-    T cfl[NST];
-    A cfu[NST][kScalarTaps ? KK : 1];
-    auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
-        constexpr int ST = decltype(st_tag)::value;
-        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * plane, ci < nch ? plane_bytes : 0u);
-#pragma unroll
-        for (int rr = 0; rr < ROWS; ++rr) load_words<NW>(pr, xb[rr], xw[ST][rr]);
-        const int cc = ci < nch ? ci : nch - 1;   // (the taps are read through plain pointers: stay inside)
-        if constexpr (kScalarTaps) {
-#pragma unroll
-            for (int t = 0; t < KK; ++t) cfu[ST][t] = cfs[(int64_t)cc * KK + (BWD ? KK - 1 - t : t)];
-        } else {
-            cfl[ST] = cfs[(int64_t)cc * KK + tsel];
-        }
-    };
-    issue(std::integral_constant<int, 0>{}, 0);
-    if constexpr (NST > 2) issue(std::integral_constant<int, 1>{}, 1);
-    if constexpr (NST > 3) issue(std::integral_constant<int, 2>{}, 2);
-
     // Spatial taps of the lane's pixels, in storage format.  Forward: tap t at
     // the pixel itself.  Gradient: slot (i, j) holds tap (K-1-i, K-1-j) at the
     // pixel (i-RAD)*D rows and (j-RAD)*D columns away - the pixel whose result
@@ -351,6 +376,38 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
         }
     }
 
+    // feature rows and channel taps of channel ci, stage ST; a channel past the
+    // wave's last one reads zeros (empty descriptor)
+    uint32_t xw[NST][ROWS][NW];
+    T cfl[NST];
+    A cfu[NST][kScalarTaps ? KK : 1];
+    auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * plane, ci < nch ? plane_bytes : 0u);
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr)
+            if (row_needed<R, K, D>(rr)) load_words<NW>(pr, xb[rr], xw[ST][rr]);
+        const int cc = ci < nch ? ci : nch - 1;   // (the taps are read through plain pointers: stay inside)
+        if constexpr (kScalarTaps) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) cfu[ST][t] = cfs[(int64_t)cc * KK + (BWD ? KK - 1 - t : t)];
+        } else {
+            cfl[ST] = cfs[(int64_t)cc * KK + tsel];
+        }
+    };
+    issue(std::integral_constant<int, 0>{}, 0);
+    if constexpr (NST > 2) issue(std::integral_constant<int, 1>{}, 1);
+    if constexpr (NST > 3) issue(std::integral_constant<int, 2>{}, 2);
+
+    // The taps were requested before the first channels.  Wait for them here:
+    // a wait inside the walk would drain the channel pipeline every round.
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int t = 0; t < KK; ++t)
+#pragma unroll
+            for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfw[r][t][k]));
+
     auto compute = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         if constexpr (sizeof(T) == 2) {
@@ -368,6 +425,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
         Row row[ROWS];
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr) {
+            if (!row_needed<R, K, D>(rr)) continue;
 #pragma unroll
             for (int k = 0; k < NW; ++k) row[rr].own[k] = xw[ST][rr][k];
             row[rr].sides(ln.first, ln.last);
@@ -429,8 +487,13 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
     // computed from zeros and its stores are dropped.
     auto step = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
+        // The loads of channel ci + NST - 1 go out before the arithmetic of channel ci,
+        // and nothing moves from one step into another: left to itself the scheduler
+        // sinks the loads to where their values are needed, which leaves nothing in flight.
         issue(std::integral_constant<int, (ST + NST - 1) % NST>{}, ci + NST - 1);
+        __builtin_amdgcn_sched_barrier(0);
         compute(st_tag, ci);
+        __builtin_amdgcn_sched_barrier(0);
     };
     for (int ci = 0; ci < nch; ci += NST) {
         step(std::integral_constant<int, 0>{}, ci);

@@ -125,10 +125,6 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             }
         }
     };
-    issue(std::integral_constant<int, 0>{}, 0);
-    if constexpr (NST > 2) issue(std::integral_constant<int, 1>{}, 1);
-    if constexpr (NST > 3) issue(std::integral_constant<int, 2>{}, 2);
-
     // spatial taps of the lane's pixels (needed for dCF under 'mul' only)
     uint32_t sfw[MUL ? R : 1][KK][NW];
     if constexpr (MUL) {
@@ -163,6 +159,20 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                     pack<T, VX, A>(v, sfg[r][i * K + j]);
                 }
             }
+    }
+    // first channels of the walk; then wait for the spatial taps, which were requested
+    // before them: a wait inside the walk would drain the channel pipeline every round
+    static_for<0, NST - 1>([&](auto s) { issue(s, decltype(s)::value); });
+    if constexpr (MUL || DX) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < KK; ++t)
+#pragma unroll
+                for (int k = 0; k < NW; ++k) {
+                    if constexpr (MUL) asm volatile("" : "+v"(sfw[r][t][k]));
+                    if constexpr (DX) asm volatile("" : "+v"(sfg[r][t][k]));
+                }
     }
     A acc_sf[R][KK][VX];
 #pragma unroll
@@ -260,6 +270,14 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                             pcf[t] += gx;
                         }
                     }
+        // The accumulators are not read before the walk ends: without this the compiler
+        // moves every update behind the flush branch and keeps (spills) the products.
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int t = 0; t < KK; ++t)
+#pragma unroll
+                for (int e = 0; e < VX; ++e) asm volatile("" : "+v"(acc_sf[r][t][e]));
         if constexpr (DX) {
             // feature gradient of the lane's pixels: dO at the flipped tap offsets
             Row grow[ROWS];
@@ -312,8 +330,11 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     // whole rounds of NST channels (see k_rows)
     auto step = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
+        // (loads first, and nothing moves between steps: see k_rows)
         issue(std::integral_constant<int, (ST + NST - 1) % NST>{}, ci + NST - 1);
+        __builtin_amdgcn_sched_barrier(0);
         compute(st_tag, ci);
+        __builtin_amdgcn_sched_barrier(0);
     };
     for (int ci = 0; ci < nch; ci += NST) {
         step(std::integral_constant<int, 0>{}, ci);

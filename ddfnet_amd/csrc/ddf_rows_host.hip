@@ -3,7 +3,7 @@
 // walks.
 #include <algorithm>
 
-#include "ddf_rows_filters.h"
+#include "ddf_rows_taprow.h"
 
 namespace ddf {
 
@@ -45,7 +45,7 @@ bool rows_variant_built(int esz, int vx, int r) {
     return false;
 }
 
-bool rows_shape_built(int k, int d, int s) { return s == 1 && k == 3 && (d == 1 || d == 2); }
+bool rows_shape_built(int k, int d, int s) { return s == 1 && (k == 3 || k == 5) && (d == 1 || d == 2); }
 
 bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx_out, int *r_out) {
     if (!rows_shape_built(p.k, p.d, p.s)) return false;
@@ -72,6 +72,10 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     // is then one strip, and the shorter prologue matters more there.
     int R = (esz == 4 && vx == 2 && H % 2 == 0 && H * W <= 1024) ? 2 : 1;
     R = tune_int("DDF_TUNE_ROWS_R", R);
+    if (p.k == 5) {   // 25 taps: built for one row per lane and vectors of four pixels or more
+        R = 1;
+        if (vx < 4) return false;
+    }
     if (!rows_variant_built(esz, vx, R)) return false;
 
     RowsGeom t{};
@@ -86,8 +90,9 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     const int target = tune_int("DDF_TUNE_ROWS_WAVES", 8192);
     const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
     int cpw = (int)(C / want_split);
-    const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", 2 * kRowsStages);
-    cpw = std::max(cpw / kRowsStages * kRowsStages, min_cpw);
+    const int nst = p.k == 5 ? 2 : kRowsStages;
+    const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", 2 * nst);
+    cpw = std::max(cpw / nst * nst, min_cpw);
     const int forced = tune_int("DDF_TUNE_ROWS_CPW", 0);
     if (forced) cpw = forced;
     t.cpw = std::max(1, std::min(cpw, C));
@@ -180,15 +185,83 @@ bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g,
     return true;
 }
 
+// Built: 5 x 5 filters (and, as a tuning alternative, 3 x 3 without dilation).
+bool rows_taprow_shape_built(int k, int d, int s) {
+    if (s != 1) return false;
+    if (k == 5) return d == 1 || d == 2;
+    return k == 3 && d == 1 && tune_int("DDF_TUNE_TAPROW_K3", 0) != 0;
+}
+
+bool rows_taprow_geometry(const Problem &p, int dtype, RowsGeom *g, int *vx_out, int *r_out) {
+    if (!rows_taprow_shape_built(p.k, p.d, p.s)) return false;
+    if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
+    if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
+    if (dtype != DDF_F16 && dtype != DDF_F32) return false;
+    const int esz = dtype == DDF_F16 ? 2 : 4;
+    const int H = (int)p.H, W = (int)p.W, C = (int)p.C;
+    const int hx = p.r * p.d;
+    if ((int64_t)H * W * 8 >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
+    // Widest vector that still leaves enough workgroups; below that, channel
+    // splits (dSF partial sums through the workspace) make up the number.
+    const int target = tune_int("DDF_TUNE_TAPROW_WAVES", 2048);
+    RowsGeom t{};
+    int vx = 0;
+    for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
+        if (cand > tune_int("DDF_TUNE_TAPROW_VX", 16)) continue;
+        if (W % cand != 0 || cand < hx || cand < 2) continue;
+        if (W / cand > 32) continue;
+        RowsGeom c{};
+        c.C = C; c.H = H; c.W = W;
+        lay_out_lanes(&c, H, W, cand, 1);
+        t = c;
+        vx = cand;
+        if (p.N * c.nstrips * p.k >= target) break;
+    }
+    if (vx == 0) return false;
+    const int flush = p.k <= 4 ? rows::taprow_flush_channels<3>() : rows::taprow_flush_channels<5>();
+    const int64_t base = p.N * t.nstrips;
+    const int64_t want_split = std::max<int64_t>(1, (target + base * p.k - 1) / (base * p.k));
+    int cpw = (int)((C + want_split - 1) / want_split);
+    cpw = (cpw + flush - 1) / flush * flush;   // whole flush groups (and pipeline rounds)
+    cpw = std::max(cpw, tune_int("DDF_TUNE_TAPROW_MIN_CPW", 2 * flush));
+    const int forced = tune_int("DDF_TUNE_TAPROW_CPW", 0);
+    if (forced) cpw = forced;
+    t.cpw = std::max(1, std::min(cpw, C));
+    t.cpb = t.cpw;
+    t.csplit = (C + t.cpw - 1) / t.cpw;
+    t.wpb = rows::kTaprowWaves;
+    const int64_t nwork = base * t.csplit * p.k;   // one wave per filter row
+    if (nwork > (1 << 30)) return false;
+    if (nwork * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
+    t.csplit_magic = magic_of(t.csplit);
+    t.nstrips_magic = magic_of(t.nstrips);
+    const int64_t ngroups = (nwork + t.wpb - 1) / t.wpb;
+    t.xcd_per = (unsigned)((ngroups + rows::kXcd - 1) / rows::kXcd);
+    t.nwork = (int)nwork;
+    *g = t;
+    *vx_out = vx;
+    *r_out = 1;
+    return true;
+}
+
+bool rows_cover_backward(const Problem &p, int dtype) {
+    RowsGeom g; int vx, r;
+    return rows_geometry(p, dtype, 0, &g, &vx, &r) &&
+           (rows_taprow_geometry(p, dtype, &g, &vx, &r) ||
+            rows_filters_geometry(p, dtype, false, &g, &vx, &r));
+}
+
 size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need) {
     if (!(need & (DDF_NEED_DCF | DDF_NEED_DSF))) return 0;
     const size_t asz = dtype == DDF_F64 ? 8 : 4;
     size_t most = 0;
     // (room for either cut of the problem: which one runs also depends on pointer alignment)
-    for (int fused = 0; fused < 2; ++fused) {
+    for (int cut = 0; cut < 3; ++cut) {
         RowsGeom g; int vx, r;
-        if (fused && !(need & DDF_NEED_DX)) continue;
-        if (!rows_filters_geometry(p, dtype, fused != 0, &g, &vx, &r)) continue;
+        if (cut == 1 && !(need & DDF_NEED_DX)) continue;
+        if (cut < 2 ? !rows_filters_geometry(p, dtype, cut != 0, &g, &vx, &r)
+                    : !rows_taprow_geometry(p, dtype, &g, &vx, &r))
+            continue;
         size_t bytes = 0;
         if ((need & DDF_NEED_DSF) && g.csplit > 1)
             bytes += ((size_t)p.N * g.csplit * p.kk * p.H * p.W * asz + 255) / 256 * 256;

@@ -1,7 +1,7 @@
 // Launch code of the row-register kernels, instantiated once per element type.
 #pragma once
 
-#include "ddf_rows_filters.h"
+#include "ddf_rows_taprow.h"
 #include "ddf_wave.h"
 
 namespace ddf {
@@ -9,8 +9,13 @@ namespace rows {
 
 constexpr int kStages = 3;   // channels in flight per wave (one computed, two loading)
 // waves per SIMD the registers are budgeted for (fp16 with 16 pixels per lane needs the room)
-template <typename T, int VX, int R>
-constexpr int waves_per_simd() { return sizeof(T) == 2 && VX * R >= 16 ? 2 : 3; }
+template <typename T, int K, int VX, int R>
+constexpr int waves_per_simd() {
+    if (K == 5) return 2;   // 25 taps of 4 or 8 pixels in registers
+    return sizeof(T) == 2 && VX * R >= 16 ? 2 : 3;
+}
+template <int K>
+constexpr int stages() { return K == 5 ? 2 : kStages; }
 
 template <typename T, int K, int D, int VX, int R>
 hipError_t launch_kdv(const Problem &p, const RowsGeom &g, bool backward, const T *x, const T *cf,
@@ -20,12 +25,12 @@ hipError_t launch_kdv(const Problem &p, const RowsGeom &g, bool backward, const 
 #define DDF_ROWS_CASE(MUL_, BWD_)                                                               \
     do {                                                                                        \
         if (pad)                                                                                \
-            hipLaunchKernelGGL((k_rows<T, K, D, MUL_, BWD_, VX, R, true, kStages,               \
-                                       waves_per_simd<T, VX, R>()>),                            \
+            hipLaunchKernelGGL((k_rows<T, K, D, MUL_, BWD_, VX, R, true, stages<K>(),           \
+                                       waves_per_simd<T, K, VX, R>()>),                         \
                                grid, block, 0, st, g, x, cf, sf, out);                          \
         else                                                                                    \
-            hipLaunchKernelGGL((k_rows<T, K, D, MUL_, BWD_, VX, R, false, kStages,              \
-                                       waves_per_simd<T, VX, R>()>),                            \
+            hipLaunchKernelGGL((k_rows<T, K, D, MUL_, BWD_, VX, R, false, stages<K>(),          \
+                                       waves_per_simd<T, K, VX, R>()>),                         \
                                grid, block, 0, st, g, x, cf, sf, out);                          \
     } while (0)
     if (p.mul) {
@@ -46,6 +51,12 @@ hipError_t launch_v(const Problem &p, const RowsGeom &g, bool backward, const T 
     if constexpr (VX >= 2) {
         if (p.k == 3 && p.d == 2)
             return launch_kdv<T, 3, 2, VX, R>(p, g, backward, x, cf, sf, out, st);
+    }
+    // 25 taps: one row per lane, vectors of four pixels or more (the taps reach
+    // two, with dilation four, pixels into the neighbouring lane)
+    if constexpr (R == 1 && VX >= 4) {
+        if (p.k == 5 && p.d == 1) return launch_kdv<T, 5, 1, VX, R>(p, g, backward, x, cf, sf, out, st);
+        if (p.k == 5 && p.d == 2) return launch_kdv<T, 5, 2, VX, R>(p, g, backward, x, cf, sf, out, st);
     }
     return hipErrorNotSupported;
 }
@@ -112,6 +123,52 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
     return hipGetLastError();
 }
 
+#ifndef DDF_TAPROW_NST
+#define DDF_TAPROW_NST 8
+#endif
+#ifndef DDF_TAPROW_WPE
+#define DDF_TAPROW_WPE 3
+#endif
+template <typename T, int K, int D, int VX>
+hipError_t launch_taprow_kdv(const Problem &p, const RowsGeom &g, const T *go, const T *x,
+                             const T *cf, const T *sf, T *dcf, T *dsf,
+                             typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
+                             unsigned need, hipStream_t st) {
+    using A = typename Acc<T>::type;
+    constexpr int kTaprowStages = DDF_TAPROW_NST, kWpe = DDF_TAPROW_WPE;
+    const dim3 grid(g.xcd_per * kXcd), block(kWave * kTaprowWaves);
+    const int lds = taprow_lds_bytes<K>((int)sizeof(A));
+    const bool pad = g.lp > g.lpr;
+#define DDF_TAPROW_CASE(MUL_, PAD_)                                                              \
+    hipLaunchKernelGGL((k_rows_taprow_filters<T, K, D, MUL_, VX, 1, PAD_, kTaprowStages, kWpe>), \
+                       grid, block, lds, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need)
+    if (p.mul) {
+        if (pad) DDF_TAPROW_CASE(true, true);
+        else DDF_TAPROW_CASE(true, false);
+    } else {
+        if (pad) DDF_TAPROW_CASE(false, true);
+        else DDF_TAPROW_CASE(false, false);
+    }
+#undef DDF_TAPROW_CASE
+    return hipGetLastError();
+}
+
+template <typename T, int VX>
+hipError_t launch_taprow_v(const Problem &p, const RowsGeom &g, const T *go, const T *x,
+                           const T *cf, const T *sf, T *dcf, T *dsf,
+                           typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
+                           unsigned need, hipStream_t st) {
+    if (p.k == 3 && p.d == 1)
+        return launch_taprow_kdv<T, 3, 1, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+    if (p.k == 5 && p.d == 1)
+        return launch_taprow_kdv<T, 5, 1, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+    if constexpr (VX >= 4) {
+        if (p.k == 5 && p.d == 2)
+            return launch_taprow_kdv<T, 5, 2, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+    }
+    return hipErrorNotSupported;
+}
+
 }  // namespace rows
 
 // Filter gradients on the row-register kernel, partial sums included; with
@@ -127,7 +184,9 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     const bool fused = dx != nullptr;
     RowsGeom g;
     int vx, r;
-    if (!rows_filters_geometry(p, dtype, fused, &g, &vx, &r)) return hipErrorNotSupported;
+    // (5 x 5: the tap rows go to the waves of a workgroup)
+    const bool taprow = !fused && rows_taprow_geometry(p, dtype, &g, &vx, &r);
+    if (!taprow && !rows_filters_geometry(p, dtype, fused, &g, &vx, &r)) return hipErrorNotSupported;
     const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
     if ((((uintptr_t)x | (uintptr_t)go | (uintptr_t)sf | (uintptr_t)dsf | (uintptr_t)dx) & mask) != 0)
         return hipErrorNotSupported;
@@ -141,7 +200,16 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     if ((need & DDF_NEED_DCF) && g.nstrips > 1) ws_cf = reinterpret_cast<A *>(wp);
     hipError_t err = hipErrorNotSupported;
     if constexpr (sizeof(T) != 8) {
-        if (fused) {
+        if (taprow) {
+            if (vx == 4)
+                err = rows::launch_taprow_v<T, 4>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            else if (vx == 2)
+                err = rows::launch_taprow_v<T, 2>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            if constexpr (sizeof(T) == 2) {
+                if (vx == 8)
+                    err = rows::launch_taprow_v<T, 8>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            }
+        } else if (fused) {
             if (vx == 2 && r == 2)
                 err = rows::launch_filters_v<T, 2, 2, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
             else if (vx == 4 && r == 1)

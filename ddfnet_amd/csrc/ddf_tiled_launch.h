@@ -186,7 +186,14 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     }
     WaveGeom g; int ps, nv;
     bool fuse = false;
-    if ((need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_FUSED", 1) != 0) {
+    // (where the row-register kernels cover both halves, two of their launches beat
+    // the fused tile kernel)
+    bool rows_both = false;
+    if constexpr (sizeof(T) != 8) {
+        rows_both = tune_int("DDF_TUNE_ROWS", 1) != 0 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
+                    !small_supported(p) && rows_cover_backward(p, dtype);
+    }
+    if ((need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0) {
         WaveGeom gp; int pps, pnv;
         fuse = wave_plan<T>(p, kWaveFused, {go, x, sf, dx}, &g, &ps, &nv) &&
                wave_geometry(p, dtype, kWaveFilters, 0, &gp, &pps, &pnv) && gp.TH == g.TH &&

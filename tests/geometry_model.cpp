@@ -185,8 +185,12 @@ static void check_geometry(int kind, long N, long C, long H, long W, int k, int 
 // the buffer descriptor), every pixel of the plane owned by exactly one lane, an idle lane
 // after every image row in the padded layout, all lanes within the wavefront, every work
 // item mapped to its own (sample, strip, channel range), the channel ranges covering C.
+// kind 0: k_rows; 1: k_rows_filters (four waves of a workgroup split its channels);
+// 2: k_rows_taprow_filters (K waves of a workgroup, wave i reads the feature rows
+// (i - K/2) * D rows away: `taps` = K, `dil` = D).
 template <int R, int HY, int VX>
-static void replay_rows(const RowsGeom &g, long N, long C, bool filters) {
+static void replay_rows(const RowsGeom &g, long N, long C, int kind, int taps = 0, int dil = 0) {
+    const bool filters = kind == 1;
     const long plane = (long)g.H * g.W;
     std::vector<int> owner(plane, 0);
     CHECK(g.lp == g.lpr || g.lp == g.lpr + 1, "lane pitch %d for %d lanes per row", g.lp, g.lpr);
@@ -211,14 +215,30 @@ static void replay_rows(const RowsGeom &g, long N, long C, bool filters) {
             if (g.lp > g.lpr && v == g.lpr)
                 for (int rr = 0; rr < R + 2 * HY; ++rr) CHECK(ln.xoff[rr] < 0, "padding lane %d is live", lane);
             CHECK(ln.first == (v == 0) && ln.last == (v == g.lpr - 1), "row ends");
+            for (int i = 0; i < taps; ++i) {
+                // the shifted window of wave i: same result rows, feature rows dy further down
+                const int dy = (i - taps / 2) * dil;
+                rows::Lane<R, HY, VX> sh;
+                sh.init(g, strip, lane, dy);
+                for (int r = 0; r < R; ++r) CHECK(sh.ooff[r] == ln.ooff[r], "result rows move with the tap row");
+                for (int rr = 0; rr < R + 2 * HY; ++rr) {
+                    const int off = sh.xoff[rr];
+                    if (off < 0) continue;
+                    const int yy = strip * g.rps + grp * R - HY + rr + dy;
+                    CHECK(grp < g.rg && v < g.lpr && yy >= 0 && yy < g.H && off == yy * g.W + v * VX,
+                          "shifted offset %d is not row %d vector %d", off, yy, v);
+                }
+            }
         }
     for (long i = 0; i < plane; ++i)
         if (owner[i] != 1) { CHECK(false, "pixel %ld owned %d times", i, owner[i]); break; }
     // work items
-    const long items = (long)N * g.nstrips * g.csplit;
+    const int per = kind == 2 ? taps : 1;   // waves (one per filter row) per (sample, strip, channel range)
+    const long items = (long)N * g.nstrips * g.csplit * per;
     CHECK(items == g.nwork, "work items %d", g.nwork);
     CHECK((long)g.csplit * g.cpb >= C && (long)(g.csplit - 1) * g.cpb < C, "channel ranges");
     if (filters) CHECK(g.cpb == g.cpw * rows::kFilterWaves && g.wpb == 1, "filter workgroup shape");
+    else if (kind == 2) CHECK(g.cpb == g.cpw && g.wpb == rows::kTaprowWaves, "tap-row workgroup shape");
     else CHECK(g.cpb == g.cpw && g.wpb >= 1 && g.wpb <= rows::kMaxWpb, "waves per workgroup");
     const long groups = (items + g.wpb - 1) / g.wpb;
     CHECK((long)g.xcd_per * 8 >= groups && (long)(g.xcd_per - 1) * 8 < groups, "workgroups per XCD");
@@ -228,8 +248,10 @@ static void replay_rows(const RowsGeom &g, long N, long C, bool filters) {
     for (long blk = 0; blk < nblk; blk += stepb)
         for (int w = 0; w < g.wpb; ++w) {
             rows::Work wk;
-            if (!wk.init(g, (int)blk, w)) continue;
-            const long id = ((long)wk.n * g.nstrips + wk.strip) * g.csplit + wk.cs;
+            const int item = rows::Work::item_of(g, (int)blk, w);
+            if (item < 0) continue;
+            wk.decode(g, item / per);   // (as the kernels do)
+            const long id = (((long)wk.n * g.nstrips + wk.strip) * g.csplit + wk.cs) * per + item % per;
             CHECK(wk.n < N && wk.strip < g.nstrips && wk.cs < g.csplit && id < items, "work item out of range");
             if (id < items) { CHECK(!seen[id], "work item %ld handed out twice", id); seen[id] = 1; }
             CHECK(wk.c_begin == wk.cs * g.cpb && wk.c_end <= C && wk.c_end > wk.c_begin, "channel range");
@@ -239,18 +261,34 @@ static void replay_rows(const RowsGeom &g, long N, long C, bool filters) {
             if (!seen[i]) { CHECK(false, "work item %ld never handed out", i); break; }
 }
 
-static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, bool filters, bool fused = false) {
+static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, bool filters, bool fused = false,
+                       bool taprow = false) {
     const Problem p = make_problem(N, C, H, W, k, d, 1, 0);
     RowsGeom g;
     int vx, r;
-    const bool ok = filters ? rows_filters_geometry(p, dtype, fused, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r);
+    const bool ok = taprow ? rows_taprow_geometry(p, dtype, &g, &vx, &r)
+                  : filters ? rows_filters_geometry(p, dtype, fused, &g, &vx, &r)
+                            : rows_geometry(p, dtype, 0, &g, &vx, &r);
+    const char *name = taprow ? "-taprow" : filters ? "-filters" : "";
     if (!ok) {
-        printf("kind rows%s %ldx%ldx%ldx%ld k%d d%d dt%d: unsupported\n", filters ? "-filters" : "", N, C, H, W, k, d, dtype);
+        printf("kind rows%s %ldx%ldx%ldx%ld k%d d%d dt%d: unsupported\n", name, N, C, H, W, k, d, dtype);
         return;
     }
     printf("kind rows%s %ldx%ldx%ldx%ld k%d d%d dt%d: vx=%d r=%d lpr=%d lp=%d rg=%d rps=%d nstrips=%d cpw=%d cpb=%d "
-           "csplit=%d wpb=%d nwork=%d\n", filters ? "-filters" : "", N, C, H, W, k, d, dtype, vx, r, g.lpr, g.lp,
+           "csplit=%d wpb=%d nwork=%d\n", name, N, C, H, W, k, d, dtype, vx, r, g.lpr, g.lp,
            g.rg, g.rps, g.nstrips, g.cpw, g.cpb, g.csplit, g.wpb, g.nwork);
+    if (taprow) {
+        CHECK(dtype != 2 && r == 1, "tap-row kernel variant");
+        CHECK((k / 2) * d <= vx, "taps reach beyond the neighbouring lane");
+        const int lds = k == 3 ? rows::taprow_lds_bytes<3>(4) : rows::taprow_lds_bytes<5>(4);
+        CHECK(lds <= 64 * 1024, "tap-row kernel LDS %d", lds);
+#define TAPROW_CASE(VX_) if (vx == VX_) replay_rows<1, 0, VX_>(g, N, C, 2, k, d);
+        TAPROW_CASE(2) TAPROW_CASE(4) TAPROW_CASE(8)
+#undef TAPROW_CASE
+        if (g_fails) printf("  -> %d violations\n", g_fails);
+        g_fails = 0;
+        return;
+    }
     const int esz = dtype == 0 ? 2 : dtype == 1 ? 4 : 8;
     CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4, "vector of %d bytes", vx * esz);
     CHECK((k / 2) * d <= vx, "taps reach beyond the neighbouring lane");
@@ -261,10 +299,11 @@ static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, 
         CHECK(g.cpw % rows::kFlushChannels == 0, "channels per wave %d not whole flush groups", g.cpw);
     }
     const int hy = (k / 2) * d;
-#define ROWS_CASE(R_, HY_, VX_) if (r == R_ && hy == HY_ && vx == VX_) { replay_rows<R_, HY_, VX_>(g, N, C, filters); done = true; }
+#define ROWS_CASE(R_, HY_, VX_) if (r == R_ && hy == HY_ && vx == VX_) { replay_rows<R_, HY_, VX_>(g, N, C, filters ? 1 : 0); done = true; }
     bool done = false;
     ROWS_CASE(1, 1, 2) ROWS_CASE(1, 1, 4) ROWS_CASE(1, 1, 8) ROWS_CASE(2, 1, 2) ROWS_CASE(2, 1, 4) ROWS_CASE(2, 1, 8)
     ROWS_CASE(1, 2, 2) ROWS_CASE(1, 2, 4) ROWS_CASE(1, 2, 8) ROWS_CASE(2, 2, 2) ROWS_CASE(2, 2, 4) ROWS_CASE(2, 2, 8)
+    ROWS_CASE(1, 4, 4) ROWS_CASE(1, 4, 8)
 #undef ROWS_CASE
     CHECK(done, "no replay for r=%d hy=%d vx=%d", r, hy, vx);
     if (g_fails) printf("  -> %d violations\n", g_fails);
@@ -292,6 +331,13 @@ int main() {
             for (int dtype = 0; dtype < 3; ++dtype)
                 for (int filters = 0; filters < 3; ++filters)
                     check_rows(sh[0], sh[1], sh[2], sh[3], 3, d, dtype, filters != 0, filters == 2);
+    for (auto &sh : shapes)
+        for (int d = 1; d <= 2; ++d)
+            for (int dtype = 0; dtype < 3; ++dtype) {
+                check_rows(sh[0], sh[1], sh[2], sh[3], 5, d, dtype, false);
+                check_rows(sh[0], sh[1], sh[2], sh[3], 5, d, dtype, true, false, true);
+                check_rows(sh[0], sh[1], sh[2], sh[3], 3, d, dtype, true, false, true);
+            }
     // seeded random shapes on top of the fixed list
     unsigned long long state = 0x9E3779B97F4A7C15ull;
     auto next = [&](int lo, int hi) {
@@ -306,6 +352,8 @@ int main() {
             check_geometry(kind, N, C, H, W, q[0], q[1], q[2], next(0, 2), next(0, 1));
         check_rows(N, C, H, W / 2 * 2 + 2, 3, next(1, 2), next(0, 1), next(0, 1) != 0);
         check_rows(N, C, H, (W / 8 + 1) * 8, 3, next(1, 2), next(0, 1), next(0, 1) != 0);
+        check_rows(N, C, H, (W / 8 + 1) * 8, 5, next(1, 2), next(0, 1), false);
+        check_rows(N, C, H, (W / 4 + 1) * 4, 5, next(1, 2), next(0, 1), true, false, true);
     }
     return 0;
 }

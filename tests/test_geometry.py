@@ -39,7 +39,8 @@ def test_every_launch_geometry_stays_in_bounds(tmp_path):
     for extra in ({}, {'DDF_TUNE_WPB': '4'}, {'DDF_TUNE_WIDE': '0'}, {'DDF_TUNE_WAVES': '512'},
                   {'DDF_TUNE_CPW': '3', 'DDF_TUNE_CPW_FILTERS': '3'}, {'DDF_TUNE_VEC': '1'},
                   {'DDF_TUNE_ROWS_R': '2'}, {'DDF_TUNE_ROWS_R': '1', 'DDF_TUNE_ROWS_PAD': '0'},
-                  {'DDF_TUNE_ROWS_WAVES': '512', 'DDF_TUNE_ROWS_WPB': '4', 'DDF_TUNE_ROWS_LPR': '64'}):
+                  {'DDF_TUNE_ROWS_WAVES': '512', 'DDF_TUNE_ROWS_WPB': '4', 'DDF_TUNE_ROWS_LPR': '64'},
+                  {'DDF_TUNE_TAPROW_K3': '1', 'DDF_TUNE_TAPROW_WAVES': '8192'}):
         run = subprocess.run([exe], capture_output=True, text=True, timeout=600,
                              env=dict(env, **extra))
         assert run.returncode == 0
