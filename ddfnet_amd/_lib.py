@@ -33,6 +33,10 @@ SYMBOLS = {
                             [_i, _vp]),
     'ddf_hip_filter_norm_backward': (_i, [_vp] * 4 + [_i64] * 2 + [_i, _i64, ctypes.c_double, _vp,
                                           _i, _vp]),
+    'ddf_hip_spatial_branch': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 3 + [ctypes.c_double] +
+                               [_vp] * 2 + [_i, _vp]),
+    'ddf_hip_channel_branch': (_i, [_vp] * 6 + [_i64] * 3 + [_i, ctypes.c_double] + [_vp] * 2 +
+                               [_i, _vp]),
     'ddf_hip_up_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 5 + [_vp]),
     'ddf_hip_up_backward_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u]),
     'ddf_hip_up_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _vp]),
@@ -167,6 +171,39 @@ def filter_norm_backward(grad_y, x, outer, groups, taps, inner, gain, gain_vec=N
             float(gain), _ptr(gain_vec), DTYPE[x.dtype], _stream())
     check(rc)
     return grad_x, terms
+
+
+def spatial_branch(features, weight, bias, head, k, stride, gain, gain_vec=None, offset_vec=None):
+    """1x1 convolution (stride as the operator's) + spatial filter normalisation
+    in one launch; returns the (N, head*k*k, H//stride, W//stride) taps."""
+    N, C, H, W = features.shape
+    sf = features.new_empty((N, head * k * k, H // stride, W // stride))
+    with on_device_of(features):
+        rc = lib().ddf_hip_spatial_branch(
+            _ptr(features), _ptr(weight), _ptr(bias), _ptr(sf), N, C, H, W, head, k, stride,
+            float(gain), _ptr(gain_vec), _ptr(offset_vec), DTYPE[features.dtype], _stream())
+    check(rc)
+    return sf
+
+
+def channel_branch(pooled, weight1, bias1, weight2, bias2, k, gain, gain_vec=None,
+                   offset_vec=None):
+    """Bottleneck MLP on the pooled (N, C) features + channel filter
+    normalisation in one launch; returns the (N, C, k, k) filters."""
+    N, C = pooled.shape
+    mid = weight1.shape[0]
+    cf = pooled.new_empty((N, C, k, k))
+    with on_device_of(pooled):
+        rc = lib().ddf_hip_channel_branch(
+            _ptr(pooled), _ptr(weight1), _ptr(bias1), _ptr(weight2), _ptr(bias2), _ptr(cf), N, C,
+            mid, k, float(gain), _ptr(gain_vec), _ptr(offset_vec), DTYPE[pooled.dtype], _stream())
+    check(rc)
+    return cf
+
+
+def branches_cover(k, dtype):
+    """(kernel_size, dtype) pairs the two branch kernels are built for."""
+    return k in (3, 5) and dtype in (torch.float16, torch.float32)
 
 
 def up_forward(features, channel_filters, spatial_filters, output, k, d, scale, combine):

@@ -1,8 +1,11 @@
-"""Builds ``libddf_hip.so`` (the C-ABI DDF library) for gfx950 with hipcc.
+"""Builds ``libddf_hip.so`` (the C-ABI DDF library) for gfx950 with hipcc, and
+the PyTorch C++ extension ``_C`` on top of it.
 
 Every ``csrc/*.hip`` file is one translation unit; they compile in parallel and
 link into ``ddfnet_amd/libddf_hip.so`` next to this file, so the built library
-travels with the source tree.  Run ``python -m ddfnet_amd.build``.
+travels with the source tree.  ``csrc/torch/ddf_torch.cpp`` (host code only) is
+compiled against torch's headers into ``ddfnet_amd/_C<EXT_SUFFIX>`` and links
+the library by a relative run path.  Run ``python -m ddfnet_amd.build``.
 """
 import glob
 import os
@@ -69,5 +72,40 @@ def build(verbose=True, extra_flags=(), jobs=None):
     return LIB_PATH
 
 
+def torch_extension_path():
+    import sysconfig
+    return os.path.join(HERE, '_C' + sysconfig.get_config_var('EXT_SUFFIX'))
+
+
+def build_torch_extension(verbose=True):
+    """Compile the C++ autograd front end (no device code) and link it against
+    torch and ``libddf_hip.so``.  Needs the library built first."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension
+    src = os.path.join(CSRC, 'torch', 'ddf_torch.cpp')
+    out = torch_extension_path()
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), 'lib')
+    rocm = os.environ.get('ROCM_PATH', '/opt/rocm')
+    cmd = [os.environ.get('CXX', 'g++'), '-O2', '-fPIC', '-shared', '-std=c++17', '-w',
+           '-D__HIP_PLATFORM_AMD__=1', '-DUSE_ROCM=1', '-DTORCH_EXTENSION_NAME=_C',
+           '-DTORCH_API_INCLUDE_EXTENSION_H',
+           '-D_GLIBCXX_USE_CXX11_ABI=%d' % int(torch._C._GLIBCXX_USE_CXX11_ABI)]
+    cmd += ['-I' + p for p in cpp_extension.include_paths()]
+    cmd += ['-I' + sysconfig.get_paths()['include'], '-I' + os.path.join(rocm, 'include'),
+            '-I' + os.path.join(ROOT, 'include'), src, '-o', out + '.tmp',
+            '-L' + torch_lib, '-L' + HERE, '-lddf_hip', '-lc10', '-lc10_hip', '-ltorch_cpu',
+            '-ltorch_hip', '-ltorch', '-ltorch_python',
+            '-Wl,-rpath,$ORIGIN', '-Wl,-rpath,' + torch_lib]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError('building the torch extension failed:\n' + proc.stdout)
+    os.replace(out + '.tmp', out)
+    if verbose:
+        print('built', out)
+    return out
+
+
 if __name__ == '__main__':
     build(extra_flags=sys.argv[1:])
+    build_torch_extension()

@@ -395,6 +395,61 @@ int ddf_hip_filter_norm_backward(const void *grad_y, const void *x, void *grad_x
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_filter_norm_backward launch");
 }
 
+int ddf_hip_spatial_branch(const void *features, const void *weight, const void *bias,
+                           void *spatial_filter, int64_t N, int64_t C, int64_t H, int64_t W,
+                           int head, int kernel_size, int stride, double gain,
+                           const void *gain_vec, const void *offset_vec, int dtype, void *stream) {
+    if (N < 0 || C < 0 || H < 0 || W < 0 || head < 0) return fail(DDF_ERR_BAD_ARG, "negative tensor size");
+    if (stride < 1) return fail(DDF_ERR_BAD_ARG, "stride must be >= 1 (got %d)", stride);
+    if (dtype != DDF_F16 && dtype != DDF_F32)
+        return fail(DDF_ERR_UNSUPPORTED, "the branch kernels cover fp16 and fp32 (dtype %d)", dtype);
+    if (!ddf::branch_kernel_size_built(kernel_size))
+        return fail(DDF_ERR_UNSUPPORTED, "the branch kernels cover kernel sizes 3 and 5 (got %d)", kernel_size);
+    if (N * C * (H / stride) * (W / stride) * head == 0) return DDF_OK;
+    if (!features || !weight || !spatial_filter) return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const hipError_t err =
+        dtype == DDF_F16
+            ? ddf::spatial_branch<__half>((const __half *)features, (const __half *)weight,
+                                          (const __half *)bias, (__half *)spatial_filter, N, C, H, W,
+                                          head, kernel_size, stride, gain, (const __half *)gain_vec,
+                                          (const __half *)offset_vec, st)
+            : ddf::spatial_branch<float>((const float *)features, (const float *)weight,
+                                         (const float *)bias, (float *)spatial_filter, N, C, H, W, head,
+                                         kernel_size, stride, gain, (const float *)gain_vec,
+                                         (const float *)offset_vec, st);
+    if (err == hipErrorNotSupported) return fail(DDF_ERR_UNSUPPORTED, "spatial branch: sizes not covered");
+    return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_spatial_branch launch");
+}
+
+int ddf_hip_channel_branch(const void *pooled, const void *weight1, const void *bias1,
+                           const void *weight2, const void *bias2, void *channel_filter, int64_t N,
+                           int64_t C, int64_t mid, int kernel_size, double gain,
+                           const void *gain_vec, const void *offset_vec, int dtype, void *stream) {
+    if (N < 0 || C < 0 || mid < 0) return fail(DDF_ERR_BAD_ARG, "negative tensor size");
+    if (dtype != DDF_F16 && dtype != DDF_F32)
+        return fail(DDF_ERR_UNSUPPORTED, "the branch kernels cover fp16 and fp32 (dtype %d)", dtype);
+    if (!ddf::branch_kernel_size_built(kernel_size))
+        return fail(DDF_ERR_UNSUPPORTED, "the branch kernels cover kernel sizes 3 and 5 (got %d)", kernel_size);
+    if (N * C == 0) return DDF_OK;
+    if (!pooled || !weight1 || !weight2 || !channel_filter) return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const hipError_t err =
+        dtype == DDF_F16
+            ? ddf::channel_branch<__half>((const __half *)pooled, (const __half *)weight1,
+                                          (const __half *)bias1, (const __half *)weight2,
+                                          (const __half *)bias2, (__half *)channel_filter, N, C, mid,
+                                          kernel_size, gain, (const __half *)gain_vec,
+                                          (const __half *)offset_vec, st)
+            : ddf::channel_branch<float>((const float *)pooled, (const float *)weight1,
+                                         (const float *)bias1, (const float *)weight2,
+                                         (const float *)bias2, (float *)channel_filter, N, C, mid,
+                                         kernel_size, gain, (const float *)gain_vec,
+                                         (const float *)offset_vec, st);
+    if (err == hipErrorNotSupported) return fail(DDF_ERR_UNSUPPORTED, "channel branch: sizes not covered");
+    return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_channel_branch launch");
+}
+
 int ddf_hip_up_forward(const void *features, const void *const *channel_filters,
                        const void *const *spatial_filters, void *output, int64_t N, int64_t C,
                        int64_t H, int64_t W, int kernel_size, int dilation, int scale,

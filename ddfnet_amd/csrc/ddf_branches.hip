@@ -1,0 +1,255 @@
+// The two filter branches of DDFPack as one launch each (gfx950, inference):
+//
+//   spatial (ddf/ddf.py:176-180 of the reference, FilterNorm 'spatial' :145-157):
+//     sf[n, g*KK + t, yo, xo] = norm_t( bias[g*KK + t] + sum_c w[g*KK + t, c] * x[n, c, yo*s, xo*s] )
+//   a 1x1 convolution with the operator's stride followed by the filter
+//   normalisation over the KK taps of every pixel.  It reads x once and writes
+//   the normalised taps; the un-normalised taps never reach memory.
+//
+//   channel (ddf/ddf.py:183-192, FilterNorm 'channel' :158-170), after the global
+//   average pool:
+//     cf[n, c, t] = norm_t( b2[c*KK + t] + sum_m w2[c*KK + t, m] * relu(b1[m] + sum_c' w1[m, c'] * v[n, c']) )
+//   the two 1x1 convolutions on the pooled (n, c) vector are small matrix
+//   products; one workgroup computes the hidden vector of its sample and 16
+//   channels' filters, and normalises them in place.
+//
+// norm_t(u) = gain_t * (u_t - mean(u)) / (std(u) + 1e-10) + offset_t with the
+// unbiased standard deviation over the KK taps, as in ddf_filter_norm.hip.
+// Both kernels are bound by memory and launch latency, not by arithmetic: the
+// spatial branch does KK multiply-adds per 4-byte (2-byte) load.
+#include "ddf_common.h"
+
+namespace ddf {
+namespace {
+
+constexpr int kBranchThreads = 256;
+constexpr int kBranchWaves = kBranchThreads / kWave;
+constexpr int kChunk = 256;   // channels whose weights sit in LDS at a time (64 per wave)
+
+// Standardise v[0..KK) in place and apply gain / offset of filter group `g`.
+template <typename T, int KK, typename A>
+__device__ __forceinline__ void normalise(A (&v)[KK], int64_t g, A gain, const T *gain_vec,
+                                          const T *offset_vec) {
+    A sum = 0;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) sum += v[t];
+    const A mean = sum / (A)KK;
+    A sq = 0;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        v[t] -= mean;
+        sq += v[t] * v[t];
+    }
+    const A inv = (A)1 / (sqrtf(sq / (A)(KK - 1)) + (A)1e-10);
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        const A w = gain_vec ? (A)ld(gain_vec + g * KK + t) : gain;
+        v[t] = v[t] * inv * w;
+        if (offset_vec) v[t] += (A)ld(offset_vec + g * KK + t);
+    }
+}
+
+// grid (pixel tiles of 64, head, N); the four waves of a workgroup cover the
+// same 64 result pixels (lane = pixel) and a quarter of every channel chunk each.
+template <typename T, int KK>
+__global__ __launch_bounds__(kBranchThreads) void k_spatial_branch(
+    const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias,
+    T *__restrict__ sf, int C, int H, int W, int Ho, int Wo, int stride, float gain,
+    const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
+    __shared__ float wt[kChunk][KK];                    // weights of the chunk, [channel][tap]
+    __shared__ float red[kBranchWaves][KK][kWave];      // per-wave sums, [wave][tap][pixel]
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int g = blockIdx.y, heads = gridDim.y;
+    const int64_t n = blockIdx.z;
+    const int npix = Ho * Wo;
+    const int pix = blockIdx.x * kWave + lane;
+    const bool live = pix < npix;
+    const int yo = live ? pix / Wo : 0, xo = live ? pix - yo * Wo : 0;
+    const int64_t plane = (int64_t)H * W;
+    const T *xp = x + n * C * plane + (int64_t)yo * stride * W + (int64_t)xo * stride;
+    const T *wg = w + (int64_t)g * KK * C;
+
+    float acc[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) acc[t] = 0.f;
+    for (int c0 = 0; c0 < C; c0 += kChunk) {
+        if (c0 > 0) __syncthreads();
+        // weights of channels c0 .. c0+255 (zero past C), coalesced along a weight row
+        {
+            const int c = c0 + (int)threadIdx.x;
+#pragma unroll
+            for (int t = 0; t < KK; ++t) wt[threadIdx.x][t] = c < C ? ld(wg + (int64_t)t * C + c) : 0.f;
+        }
+        __syncthreads();
+        const int cw = c0 + wave * kWave;               // this wave's 64 channels of the chunk
+        const int nc = min(kWave, C - cw);              // (<= 0: none left)
+        for (int i0 = 0; i0 < nc; i0 += 8) {
+            float xv[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i = min(i0 + u, nc - 1);      // past the end: repeats, with zero weights
+                xv[u] = live ? ld(xp + (int64_t)(cw + i) * plane) : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                // (rows past the wave's last channel belong to channels >= C: zeros)
+                const float *wr = wt[wave * kWave + i0 + u];
+#pragma unroll
+                for (int t = 0; t < KK; ++t) acc[t] = fmaf(wr[t], xv[u], acc[t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < KK; ++t) red[wave][t][lane] = acc[t];
+    __syncthreads();
+    if (wave != 0 || !live) return;
+    float v[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        float s = bias ? ld(bias + g * KK + t) : 0.f;
+#pragma unroll
+        for (int q = 0; q < kBranchWaves; ++q) s += red[q][t][lane];
+        v[t] = s;
+    }
+    normalise<T, KK, float>(v, g, gain, gain_vec, offset_vec);
+    T *op = sf + ((n * heads + g) * KK) * (int64_t)npix + pix;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) st(op + (int64_t)t * npix, v[t]);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+constexpr int kChannelBlock = 16;   // channels whose filters one workgroup makes
+
+// grid (channel blocks of kChannelBlock, N).  LDS: the pooled vector (C floats),
+// the hidden vector (mid floats), the block's un-normalised taps.  Every dot
+// product has the lanes of a wave along the weight row (coalesced) and ends in
+// a wave reduction; several rows are in flight at a time, which is what the
+// run time depends on (the loads are dependent on nothing but latency).
+template <typename T, int KK>
+__global__ __launch_bounds__(kBranchThreads) void k_channel_branch(
+    const T *__restrict__ pooled, const T *__restrict__ w1, const T *__restrict__ b1,
+    const T *__restrict__ w2, const T *__restrict__ b2, T *__restrict__ cf, int C, int mid,
+    float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
+    extern __shared__ float branch_smem[];
+    float *v = branch_smem;            // [C]
+    float *h = v + C;                  // [mid]
+    float *f = h + mid;                // [kChannelBlock * KK]
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t n = blockIdx.y;
+    const int cb = blockIdx.x * kChannelBlock;
+    for (int c = threadIdx.x; c < C; c += kBranchThreads) v[c] = ld(pooled + n * C + c);
+    __syncthreads();
+    // hidden vector: four rows of w1 per wave at a time
+    constexpr int RH = 4;
+    for (int m0 = wave * RH; m0 < mid; m0 += kBranchWaves * RH) {
+        float p[RH];
+#pragma unroll
+        for (int u = 0; u < RH; ++u) p[u] = 0.f;
+        for (int c = lane; c < C; c += kWave) {
+            const float vc = v[c];
+#pragma unroll
+            for (int u = 0; u < RH; ++u) {
+                const int m = min(m0 + u, mid - 1);
+                p[u] = fmaf(ld(w1 + (int64_t)m * C + c), vc, p[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < RH; ++u) {
+            const float tot = wave_sum(p[u]);
+            if (lane == 0 && m0 + u < mid) h[m0 + u] = fmaxf(tot + (b1 ? ld(b1 + m0 + u) : 0.f), 0.f);
+        }
+    }
+    __syncthreads();
+    // the block's taps: rows (cb * KK + r) of w2, eight per wave at a time
+    constexpr int RT = 8;
+    const int rows = min(kChannelBlock, C - cb) * KK;
+    for (int r0 = wave * RT; r0 < rows; r0 += kBranchWaves * RT) {
+        float p[RT];
+#pragma unroll
+        for (int u = 0; u < RT; ++u) p[u] = 0.f;
+        for (int m = lane; m < mid; m += kWave) {
+            const float hm = h[m];
+#pragma unroll
+            for (int u = 0; u < RT; ++u) {
+                const int64_t row = (int64_t)cb * KK + min(r0 + u, rows - 1);
+                p[u] = fmaf(ld(w2 + row * mid + m), hm, p[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < RT; ++u) {
+            const float tot = wave_sum(p[u]);
+            if (lane == 0 && r0 + u < rows)
+                f[r0 + u] = tot + (b2 ? ld(b2 + (int64_t)cb * KK + r0 + u) : 0.f);
+        }
+    }
+    __syncthreads();
+    const int i = threadIdx.x;
+    if (i >= kChannelBlock || cb + i >= C) return;
+    float u[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) u[t] = f[i * KK + t];
+    normalise<T, KK, float>(u, cb + i, gain, gain_vec, offset_vec);
+    T *op = cf + (n * C + cb + i) * KK;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) st(op + t, u[t]);
+}
+
+}  // namespace
+
+bool branch_kernel_size_built(int k) { return k == 3 || k == 5; }
+
+template <typename T>
+hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t N, int64_t C,
+                          int64_t H, int64_t W, int head, int k, int stride, double gain,
+                          const T *gain_vec, const T *offset_vec, hipStream_t st) {
+    const int64_t Ho = H / stride, Wo = W / stride;
+    if (N == 0 || C == 0 || Ho * Wo == 0 || head == 0) return hipSuccess;
+    if (N > 65535 || head > 65535 || C > (1 << 24) || H * W >= (1ll << 31)) return hipErrorNotSupported;
+    const dim3 grid((unsigned)cdiv(Ho * Wo, kWave), (unsigned)head, (unsigned)N);
+#define DDF_SPATIAL_CASE(KK_)                                                                   \
+    hipLaunchKernelGGL((k_spatial_branch<T, KK_>), grid, dim3(kBranchThreads), 0, st, x, w, bias, \
+                       sf, (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, (float)gain,       \
+                       gain_vec, offset_vec)
+    if (k == 3) DDF_SPATIAL_CASE(9);
+    else if (k == 5) DDF_SPATIAL_CASE(25);
+    else return hipErrorNotSupported;
+#undef DDF_SPATIAL_CASE
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2, const T *b2,
+                          T *cf, int64_t N, int64_t C, int64_t mid, int k, double gain,
+                          const T *gain_vec, const T *offset_vec, hipStream_t st) {
+    if (N == 0 || C == 0) return hipSuccess;
+    const int kk = k * k;
+    const size_t lds = ((size_t)C + (size_t)mid + (size_t)kChannelBlock * kk) * sizeof(float);
+    if (N > 65535 || mid < 1 || lds > 48 * 1024) return hipErrorNotSupported;
+    const dim3 grid((unsigned)cdiv(C, kChannelBlock), (unsigned)N);
+#define DDF_CHANNEL_CASE(KK_)                                                                    \
+    hipLaunchKernelGGL((k_channel_branch<T, KK_>), grid, dim3(kBranchThreads), lds, st, pooled, w1, \
+                       b1, w2, b2, cf, (int)C, (int)mid, (float)gain, gain_vec, offset_vec)
+    if (k == 3) DDF_CHANNEL_CASE(9);
+    else if (k == 5) DDF_CHANNEL_CASE(25);
+    else return hipErrorNotSupported;
+#undef DDF_CHANNEL_CASE
+    return hipGetLastError();
+}
+
+#define DDF_INSTANTIATE_BRANCHES(T)                                                              \
+    template hipError_t spatial_branch<T>(const T *, const T *, const T *, T *, int64_t, int64_t, \
+                                          int64_t, int64_t, int, int, int, double, const T *,    \
+                                          const T *, hipStream_t);                               \
+    template hipError_t channel_branch<T>(const T *, const T *, const T *, const T *, const T *, \
+                                          T *, int64_t, int64_t, int64_t, int, double, const T *, \
+                                          const T *, hipStream_t);
+DDF_INSTANTIATE_BRANCHES(__half)
+DDF_INSTANTIATE_BRANCHES(float)
+#undef DDF_INSTANTIATE_BRANCHES
+
+}  // namespace ddf

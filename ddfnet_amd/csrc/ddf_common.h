@@ -70,6 +70,20 @@ hipError_t filter_norm_backward(const T *dy, const T *x, T *dx, T *terms, int64_
                                 int64_t groups, int taps, int64_t inner, double gain,
                                 const T *gain_vec, hipStream_t st);
 
+// The filter branches of DDFPack, one launch each (ddf_branches.hip): 1x1
+// convolution (stride as the operator's) + spatial filter normalisation, and
+// bottleneck MLP on the pooled features + channel filter normalisation.
+// hipErrorNotSupported: kernel size or sizes not covered, nothing launched.
+bool branch_kernel_size_built(int k);
+template <typename T>
+hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t N, int64_t C,
+                          int64_t H, int64_t W, int head, int k, int stride, double gain,
+                          const T *gain_vec, const T *offset_vec, hipStream_t st);
+template <typename T>
+hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2, const T *b2,
+                          T *cf, int64_t N, int64_t C, int64_t mid, int k, double gain,
+                          const T *gain_vec, const T *offset_vec, hipStream_t st);
+
 // All scale*scale sub-pixel branches of an up-sampling DDF in one launch,
 // written into the pixel-shuffled (N, C, H*scale, W*scale) result; cf / sf are
 // host arrays of scale*scale device pointers.

@@ -39,9 +39,8 @@ void lay_out_lanes(RowsGeom *t, int H, int W, int vx, int R) {
 
 // Instantiated (elements per lane and row, rows per lane) per element size.
 bool rows_variant_built(int esz, int vx, int r) {
-    if (r != 2 && r != 1) return false;
-    if (esz == 2) return vx == 8 || vx == 4 || vx == 2;
-    if (esz == 4) return vx == 4 || vx == 2;
+    if (esz == 2) return r == 1 && (vx == 8 || vx == 4 || vx == 2);
+    if (esz == 4) return (r == 1 && (vx == 4 || vx == 2)) || (r == 2 && vx == 2);
     return false;
 }
 

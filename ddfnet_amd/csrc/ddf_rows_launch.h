@@ -77,16 +77,12 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
     const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
     if ((((uintptr_t)x | (uintptr_t)sf | (uintptr_t)out) & mask) != 0) return hipErrorNotSupported;
     if constexpr (sizeof(T) == 2) {
-        if (vx == 8 && r == 2) return rows::launch_v<T, 8, 2>(p, g, backward, x, cf, sf, out, st);
-        if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
-        if (vx == 2 && r == 2) return rows::launch_v<T, 2, 2>(p, g, backward, x, cf, sf, out, st);
         if (vx == 8 && r == 1) return rows::launch_v<T, 8, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
     } else if constexpr (sizeof(T) == 4) {
         if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
-        if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 2) return rows::launch_v<T, 2, 2>(p, g, backward, x, cf, sf, out, st);
     }
     return hipErrorNotSupported;
@@ -103,7 +99,8 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
     // waves per SIMD the registers are budgeted for: 'mul' keeps the spatial taps
     // as well, the fused feature gradient a second set of them
     constexpr int WPE_MUL = (DX || VX * R >= 4) ? 2 : 3, WPE_ADD = DX ? 2 : 3;
-    constexpr int kFilterStages = 2;   // channels in flight per wave
+    // channels in flight per wave, a divisor of kFlushChannels (whole rounds)
+    constexpr int kFilterStages = DX ? 2 : 4;
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kFilterWaves);
     const int lds = filters_lds_bytes<9>((int)sizeof(A), R, VX);
     if (p.k != 3 || p.d != 1) return hipErrorNotSupported;
@@ -123,19 +120,13 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
     return hipGetLastError();
 }
 
-#ifndef DDF_TAPROW_NST
-#define DDF_TAPROW_NST 8
-#endif
-#ifndef DDF_TAPROW_WPE
-#define DDF_TAPROW_WPE 3
-#endif
 template <typename T, int K, int D, int VX>
 hipError_t launch_taprow_kdv(const Problem &p, const RowsGeom &g, const T *go, const T *x,
                              const T *cf, const T *sf, T *dcf, T *dsf,
                              typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                              unsigned need, hipStream_t st) {
     using A = typename Acc<T>::type;
-    constexpr int kTaprowStages = DDF_TAPROW_NST, kWpe = DDF_TAPROW_WPE;
+    constexpr int kTaprowStages = 8, kWpe = 3;   // channels in flight per wave; waves per SIMD
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kTaprowWaves);
     const int lds = taprow_lds_bytes<K>((int)sizeof(A));
     const bool pad = g.lp > g.lpr;

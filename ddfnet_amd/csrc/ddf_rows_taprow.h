@@ -24,11 +24,8 @@ namespace rows {
 
 // Channels whose dCF partials are parked before one lane per (channel, tap of
 // the wave's row) adds them up: as many as 64 lanes serve, a power of two.
-#ifndef DDF_TAPROW_G
-#define DDF_TAPROW_G 8
-#endif
 template <int K>
-constexpr int taprow_flush_channels() { return K <= 4 ? 16 : DDF_TAPROW_G; }
+constexpr int taprow_flush_channels() { return K <= 4 ? 16 : 8; }
 
 constexpr int kTaprowWaves = 4;   // independent waves per workgroup
 

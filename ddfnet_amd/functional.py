@@ -180,7 +180,15 @@ class DDFFunction(Function):
         return grad_input, grad_channel_filter, grad_spatial_filter, None, None, None, None, None
 
 
-ddf = DDFFunction.apply
+# The operator callers use: the C++ autograd function of the torch extension
+# (csrc/torch/ddf_torch.cpp: same checks, same messages, same library calls,
+# without the interpreter in between) where it has been built, else the Python
+# Function above.  Both enqueue the same kernels.
+try:
+    from . import _C
+except ImportError:      # extension (or the library it links) not built
+    _C = None
+ddf = _C.ddf if _C is not None else DDFFunction.apply
 
 
 class DDFUpFunction(Function):

@@ -12,7 +12,7 @@ import torch.nn.functional as F
 from torch.nn.init import calculate_gain
 
 from . import _lib
-from .functional import ddf, ddf_up
+from .functional import _C, ddf, ddf_up
 
 __all__ = ['FilterNorm', 'build_spatial_branch', 'build_channel_branch',
            'DDFPack', 'DDFUpPack']
@@ -120,6 +120,20 @@ class FilterNorm(nn.Module):
         raise RuntimeError('Unsupported filter type {}'.format(self.filter_type))
 
 
+def _unhooked(module):
+    """No forward / backward hook is registered on the module."""
+    return not (module._forward_hooks or module._forward_pre_hooks or module._backward_hooks or
+                getattr(module, '_backward_pre_hooks', None))
+
+
+def _plain_pointwise_conv(module, stride):
+    """A 1x1 nn.Conv2d that is a matrix product per (strided) pixel: no groups,
+    padding or dilation, nothing hooked."""
+    return (type(module) is nn.Conv2d and _unhooked(module) and module.kernel_size == (1, 1) and
+            module.stride == (stride, stride) and module.padding == (0, 0) and
+            module.dilation == (1, 1) and module.groups == 1 and module.padding_mode == 'zeros')
+
+
 def build_spatial_branch(in_channels, kernel_size, head=1,
                          nonlinearity='relu', stride=1):
     """1x1 convolution (strided like the operator) to ``head * k*k`` taps per
@@ -162,6 +176,27 @@ class DDFPack(nn.Module):
         self.channel_branch = build_channel_branch(
             in_channels, kernel_size, nonlinearity, se_ratio)
 
+    def _stock_channel_branch(self):
+        """The channel branch is exactly what build_channel_branch makes (global
+        average pool, plain 1x1 convolution, ReLU, plain 1x1 convolution,
+        FilterNorm) and nothing listens on its modules."""
+        branch = self.channel_branch
+        return (isinstance(branch, nn.Sequential) and len(branch) == 5 and _unhooked(branch) and
+                isinstance(branch[0], nn.AdaptiveAvgPool2d) and _unhooked(branch[0]) and
+                branch[0].output_size in (1, (1, 1)) and
+                _plain_pointwise_conv(branch[1], 1) and
+                type(branch[2]) is nn.ReLU and _unhooked(branch[2]) and
+                _plain_pointwise_conv(branch[3], 1) and
+                type(branch[4]) is FilterNorm and _unhooked(branch[4]) and
+                branch[4].filter_type == 'channel')
+
+    def _stock_spatial_branch(self):
+        branch = self.spatial_branch
+        return (isinstance(branch, nn.Sequential) and len(branch) == 2 and _unhooked(branch) and
+                _plain_pointwise_conv(branch[0], self.stride) and
+                type(branch[1]) is FilterNorm and _unhooked(branch[1]) and
+                branch[1].filter_type == 'spatial' and branch[1].in_channels == self.head)
+
     def _channel_filter(self, x):
         """The channel branch.  Its two 1x1 convolutions act on a pooled
         (b, c, 1, 1) tensor, i.e. they are matrix products: evaluating them as
@@ -169,19 +204,69 @@ class DDFPack(nn.Module):
         library's launch path, which costs more host time than the whole layer
         has GPU work at small feature maps."""
         branch = self.channel_branch
-        if not (x.is_cuda and isinstance(branch, nn.Sequential) and len(branch) == 5 and
-                isinstance(branch[0], nn.AdaptiveAvgPool2d) and isinstance(branch[2], nn.ReLU) and
-                all(isinstance(m, nn.Conv2d) and m.kernel_size == (1, 1) for m in (branch[1], branch[3]))):
+        if not (x.is_cuda and self._stock_channel_branch()):
             return branch(x)   # not the stock branch: run it as it is
         fc1, fc2, norm = branch[1], branch[3], branch[4]
         v = x.mean((2, 3))
         v = F.relu(F.linear(v, fc1.weight.flatten(1), fc1.bias))
         return norm(F.linear(v, fc2.weight.flatten(1), fc2.bias))
 
+    def _inference_filters(self, x):
+        """Both filters with one launch per branch (plus the pooling) - or, with
+        the torch extension, the layer's result itself - or None where that
+        path does not apply: gradients wanted, branches that are not
+        the stock ones, a dtype or kernel size the branch kernels lack, or
+        parameters in another dtype than the features (autocast)."""
+        if torch.is_grad_enabled() and (x.requires_grad or
+                                        any(p.requires_grad for p in self.parameters())):
+            return None
+        k = self.kernel_size
+        if not (x.is_cuda and x.dim() == 4 and _lib.branches_cover(k, x.dtype) and
+                self._stock_channel_branch() and self._stock_spatial_branch()):
+            return None
+        conv, sp_norm = self.spatial_branch
+        fc1, fc2, ch_norm = self.channel_branch[1], self.channel_branch[3], self.channel_branch[4]
+        tensors = [conv.weight, conv.bias, fc1.weight, fc1.bias, fc2.weight, fc2.bias]
+        for norm in (sp_norm, ch_norm):
+            tensors += [norm.std if norm.runing_std else None,
+                        norm.mean if norm.runing_mean else None]
+        if any(t is not None and (t.dtype != x.dtype or t.device != x.device) for t in tensors):
+            return None
+        if ch_norm.in_channels != x.size(1) or fc1.in_channels != x.size(1):
+            return None
+        if _C is not None:
+            # the same four launches without the interpreter in between
+            return _C.ddf_pack_forward(
+                x, conv.weight, conv.bias,
+                1.0 if sp_norm.runing_std else sp_norm.std, tensors[6], tensors[7],
+                fc1.weight, fc1.bias, fc2.weight, fc2.bias,
+                1.0 if ch_norm.runing_std else ch_norm.std, tensors[8], tensors[9],
+                k, self.dilation, self.stride, self.head, self.kernel_combine)
+        x = x.contiguous()
+        cf = _lib.channel_branch(
+            x.mean((2, 3)), fc1.weight, fc1.bias, fc2.weight, fc2.bias, k,
+            1.0 if ch_norm.runing_std else ch_norm.std,
+            ch_norm.std if ch_norm.runing_std else None,
+            ch_norm.mean if ch_norm.runing_mean else None)
+        sf = _lib.spatial_branch(
+            x, conv.weight, conv.bias, self.head, k, self.stride,
+            1.0 if sp_norm.runing_std else sp_norm.std,
+            sp_norm.std if sp_norm.runing_std else None,
+            sp_norm.mean if sp_norm.runing_mean else None)
+        return cf, sf
+
     def forward(self, x):
         b, c, h, w = x.shape
         g, k, s = self.head, self.kernel_size, self.stride
         ho, wo = h // s, w // s
+        filters = self._inference_filters(x)
+        if torch.is_tensor(filters):      # the whole layer was run
+            return filters
+        if filters is not None:
+            cf, sf = filters
+            out = ddf(x.reshape(b * g, c // g, h, w), cf.reshape(b * g, c // g, k, k),
+                      sf.reshape(b * g, k * k, ho, wo), k, self.dilation, s, self.kernel_combine)
+            return out.reshape(b, c, ho, wo)
         cf = self._channel_filter(x).reshape(b * g, c // g, k, k)
         sf = self.spatial_branch(x).reshape(b * g, k * k, ho, wo)
         out = ddf(x.reshape(b * g, c // g, h, w), cf, sf,

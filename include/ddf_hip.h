@@ -196,6 +196,44 @@ int ddf_hip_filter_norm_backward(const void *grad_y, const void *x,
                                  void *stream);
 
 /*
+ * Spatial filter branch of DDFPack in one launch (build_spatial_branch,
+ * ddf/ddf.py:176-180: a 1x1 convolution with the operator's stride to
+ * head * k*k taps per pixel, then FilterNorm 'spatial', ddf/ddf.py:145-157).
+ * `features` is (N, C, H, W), `weight` the convolution weight (head * k*k, C)
+ * (its trailing 1x1 dimensions dropped), `bias` (head * k*k) or NULL;
+ * `spatial_filter` receives the normalised (N, head * k*k, H/stride, W/stride)
+ * taps, which is the (N * head, k*k, Ho, Wo) operand of the operator.  gain /
+ * gain_vec / offset_vec as in ddf_hip_filter_norm with groups = head.
+ * Inference path: there is no gradient counterpart; training runs the
+ * convolution and ddf_hip_filter_norm / _backward separately.
+ * DDF_ERR_UNSUPPORTED: kernel size other than 3 or 5, or fp64.
+ */
+int ddf_hip_spatial_branch(const void *features, const void *weight,
+                           const void *bias, void *spatial_filter, int64_t N,
+                           int64_t C, int64_t H, int64_t W, int head,
+                           int kernel_size, int stride, double gain,
+                           const void *gain_vec, const void *offset_vec,
+                           int dtype, void *stream);
+
+/*
+ * Channel filter branch of DDFPack after its global average pool, in one
+ * launch (build_channel_branch, ddf/ddf.py:183-192: 1x1 convolution C -> mid,
+ * ReLU, 1x1 convolution mid -> C * k*k, then FilterNorm 'channel',
+ * ddf/ddf.py:158-170).  `pooled` is the (N, C) mean of the features over H x W,
+ * `weight1` (mid, C), `bias1` (mid) or NULL, `weight2` (C * k*k, mid), `bias2`
+ * (C * k*k) or NULL; `channel_filter` receives the normalised (N, C, k, k)
+ * filters.  gain / gain_vec / offset_vec as in ddf_hip_filter_norm with
+ * groups = C.  Inference path, as above.  DDF_ERR_UNSUPPORTED: kernel size
+ * other than 3 or 5, fp64, or C + mid beyond what one workgroup's LDS holds.
+ */
+int ddf_hip_channel_branch(const void *pooled, const void *weight1,
+                           const void *bias1, const void *weight2,
+                           const void *bias2, void *channel_filter, int64_t N,
+                           int64_t C, int64_t mid, int kernel_size,
+                           double gain, const void *gain_vec,
+                           const void *offset_vec, int dtype, void *stream);
+
+/*
  * Up-sampling DDF forward (DDFUpPack.forward, ddf/ddf.py:257-272): the
  * reference calls `ddf` once per sub-pixel branch b = 0 .. scale*scale-1 on
  * the same features with that branch's filters (ddf.py:264-269), stacks the

@@ -513,3 +513,38 @@ def test_tiny_planes(N, C, H, W, d, combine, dtype):
     case = random_case(N, C, H, W, 3, 1, dtype, seed=N + C)
     check_against_oracle(*case, 3, d, 1, combine, '', what='tiny plane')
     check_against_oracle(*case, 3, d, 1, combine, 'f', what='tiny plane, tiled forced')
+
+
+def test_cpp_operator_equals_python_operator():
+    """ddf is the C++ autograd function of the torch extension where that is
+    built; DDFFunction is the Python one.  Same checks, same library calls:
+    results and gradients are bit-identical."""
+    from ddfnet_amd import DDFFunction, ddf, functional
+    if functional._C is None:
+        pytest.skip('torch extension not built')
+    assert ddf is functional._C.ddf
+    for dtype in (torch.float32, torch.float16):
+        for (N, C, H, W, k, d, s, combine) in [(2, 16, 14, 14, 3, 1, 1, 'mul'), (2, 8, 9, 11, 3, 2, 2, 'add'),
+                                               (1, 4, 12, 12, 5, 1, 1, 'mul')]:
+            x, cf, sf, go = oracle.make_inputs(N, C, H, W, k, s, dtype)
+            a = [t.cuda().requires_grad_(True) for t in (x, cf, sf)]
+            b = [t.cuda().requires_grad_(True) for t in (x, cf, sf)]
+            out_a = ddf(*a, k, d, s, combine)
+            out_b = DDFFunction.apply(*b, k, d, s, combine)
+            assert torch.equal(out_a, out_b)
+            ga = torch.autograd.grad(out_a, a, go.cuda())
+            gb = torch.autograd.grad(out_b, b, go.cuda())
+            for u, v in zip(ga, gb):
+                assert torch.equal(u, v)
+    # mixed dtypes are promoted, only the wanted gradients are computed
+    x, cf, sf, go = oracle.make_inputs(2, 8, 10, 10, 3, 1, torch.float32)
+    xh = x.cuda().half().requires_grad_(True)
+    out = ddf(xh, cf.cuda(), sf.cuda())
+    assert out.dtype == torch.float32
+    (gx,) = torch.autograd.grad(out, [xh], go.cuda())
+    assert gx.dtype == torch.float16 and gx.shape == xh.shape
+    # keyword arguments and defaults as in the reference's signature
+    assert torch.equal(ddf(x.cuda(), cf.cuda(), sf.cuda(), kernel_combine='add', kernel_size=3),
+                       DDFFunction.apply(x.cuda(), cf.cuda(), sf.cuda(), 3, 1, 1, 'add'))
+    with torch.autocast('cuda', dtype=torch.float16):
+        assert ddf(x.cuda(), cf.cuda(), sf.cuda()).dtype == torch.float16

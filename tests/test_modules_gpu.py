@@ -56,6 +56,53 @@ def test_ddfpack_matches_cpu_reference(stride, head, combine, monkeypatch):
         assert torch.allclose(p.grad.cpu().double(), pr.grad, rtol=1e-3, atol=1e-4), name
 
 
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-4), (torch.float16, 2e-2)])
+@pytest.mark.parametrize('k,stride,head,c,hw', [(3, 1, 1, 16, 12), (3, 2, 1, 16, 12), (3, 1, 4, 16, 9),
+                                                (5, 1, 1, 70, 10), (3, 1, 1, 300, 7), (3, 1, 2, 64, 30)])
+def test_ddfpack_inference_path_matches_cpu_reference(k, stride, head, c, hw, dtype, tol, monkeypatch):
+    """Without gradients the two filter branches run as one launch each
+    (ddf_hip_channel_branch, ddf_hip_spatial_branch); checked against the CPU
+    fp64 modules and against the op-by-op path the same module takes in training."""
+    torch.manual_seed(3)
+    pack = ddfnet_amd.DDFPack(c, kernel_size=k, stride=stride, head=head).cuda().to(dtype)
+    x = torch.randn(3, c, hw, hw + 2, device='cuda').to(dtype)
+    with torch.no_grad():
+        assert pack._inference_filters(x) is not None       # the one-launch branches do run
+        out = pack(x)
+        # the ctypes route of the same launches (what runs without the torch extension)
+        monkeypatch.setattr(ddf_modules, '_C', None)
+        cf, sf = pack._inference_filters(x)
+        monkeypatch.undo()
+        g = head
+        again = ddfnet_amd.ddf(x.reshape(3 * g, c // g, hw, hw + 2), cf.reshape(3 * g, c // g, k, k),
+                               sf.reshape(3 * g, k * k, hw // stride, (hw + 2) // stride), k, 1, stride)
+        assert torch.equal(out, again.reshape(out.shape))
+    _, _, out_r = cpu_reference(pack, monkeypatch, x)
+    err = (out.double().cpu() - out_r.detach()).abs().max() / out_r.detach().abs().max()
+    assert err < tol, err
+    trained = pack(x.clone().requires_grad_(True))           # op-by-op branches
+    assert (out.float() - trained.detach().float()).abs().max() / out.float().abs().max() < tol
+
+
+def test_ddfpack_inference_path_only_for_stock_branches():
+    pack = ddfnet_amd.DDFPack(16).cuda()
+    x = torch.randn(2, 16, 8, 8, device='cuda')
+    with torch.no_grad():
+        assert pack._inference_filters(x) is not None
+        assert pack._inference_filters(x.double()) is None           # dtype the kernels lack
+    assert pack._inference_filters(x) is None                         # parameters want gradients
+    with torch.no_grad():
+        handle = pack.spatial_branch[0].register_forward_hook(lambda m, i, o: o)
+        assert pack._inference_filters(x) is None                     # somebody listens
+        handle.remove()
+        pack.channel_branch[1] = torch.nn.Conv2d(16, 3, 1, groups=1, padding=1).cuda()
+        assert pack._inference_filters(x) is None                     # not a plain 1x1 product
+    with torch.no_grad(), torch.autocast('cuda', dtype=torch.float16):
+        pack = ddfnet_amd.DDFPack(16).cuda()
+        out = pack(x.half())                                          # fp16 features, fp32 parameters
+        assert torch.isfinite(out).all()
+
+
 def test_ddfuppack_matches_cpu_reference(monkeypatch):
     torch.manual_seed(1)
     up = ddfnet_amd.DDFUpPack(8, kernel_size=3, scale_factor=2).cuda()
