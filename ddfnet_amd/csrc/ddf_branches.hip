@@ -10,7 +10,7 @@
 //   average pool:
 //     cf[n, c, t] = norm_t( b2[c*KK + t] + sum_m w2[c*KK + t, m] * relu(b1[m] + sum_c' w1[m, c'] * v[n, c']) )
 //   the two 1x1 convolutions on the pooled (n, c) vector are small matrix
-//   products; one workgroup computes the hidden vector of its sample and 16
+//   products; one workgroup computes the hidden vector of its sample and 64
 //   channels' filters, and normalises them in place.
 //
 // norm_t(u) = gain_t * (u_t - mean(u)) / (std(u) + 1e-10) + offset_t with the
@@ -22,8 +22,6 @@
 namespace ddf {
 namespace {
 
-constexpr int kBranchThreads = 256;
-constexpr int kBranchWaves = kBranchThreads / kWave;
 constexpr int kChunk = 256;   // channels whose weights sit in LDS at a time (64 per wave)
 
 // Standardise v[0..KK) in place and apply gain / offset of filter group `g`.
@@ -49,15 +47,19 @@ __device__ __forceinline__ void normalise(A (&v)[KK], int64_t g, A gain, const T
     }
 }
 
-// grid (pixel tiles of 64, head, N); the four waves of a workgroup cover the
-// same 64 result pixels (lane = pixel) and a quarter of every channel chunk each.
-template <typename T, int KK>
-__global__ __launch_bounds__(kBranchThreads) void k_spatial_branch(
+// grid (pixel tiles of 64, head, N); the WAVES waves of a workgroup cover the
+// same 64 result pixels (lane = pixel) and 1/WAVES of every channel chunk each,
+// 16 channels' loads in flight at a time.
+template <typename T, int KK, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void k_spatial_branch(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias,
     T *__restrict__ sf, int C, int H, int W, int Ho, int Wo, int stride, float gain,
     const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
+    constexpr int PER = kChunk / WAVES;                 // channels of a chunk per wave
+    constexpr int U = 16;
+    static_assert(PER % U == 0, "whole batches");
     __shared__ float wt[kChunk][KK];                    // weights of the chunk, [channel][tap]
-    __shared__ float red[kBranchWaves][KK][kWave];      // per-wave sums, [wave][tap][pixel]
+    __shared__ float red[WAVES][KK][kWave];             // per-wave sums, [wave][tap][pixel]
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int g = blockIdx.y, heads = gridDim.y;
     const int64_t n = blockIdx.z;
@@ -75,25 +77,25 @@ __global__ __launch_bounds__(kBranchThreads) void k_spatial_branch(
     for (int c0 = 0; c0 < C; c0 += kChunk) {
         if (c0 > 0) __syncthreads();
         // weights of channels c0 .. c0+255 (zero past C), coalesced along a weight row
-        {
-            const int c = c0 + (int)threadIdx.x;
+        for (int i = threadIdx.x; i < kChunk; i += WAVES * kWave) {
+            const int c = c0 + i;
 #pragma unroll
-            for (int t = 0; t < KK; ++t) wt[threadIdx.x][t] = c < C ? ld(wg + (int64_t)t * C + c) : 0.f;
+            for (int t = 0; t < KK; ++t) wt[i][t] = c < C ? ld(wg + (int64_t)t * C + c) : 0.f;
         }
         __syncthreads();
-        const int cw = c0 + wave * kWave;               // this wave's 64 channels of the chunk
-        const int nc = min(kWave, C - cw);              // (<= 0: none left)
-        for (int i0 = 0; i0 < nc; i0 += 8) {
-            float xv[8];
+        const int cw = c0 + wave * PER;                 // this wave's channels of the chunk
+        const int nc = min(PER, C - cw);                // (<= 0: none left)
+        for (int i0 = 0; i0 < nc; i0 += U) {
+            float xv[U];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < U; ++u) {
                 const int i = min(i0 + u, nc - 1);      // past the end: repeats, with zero weights
                 xv[u] = live ? ld(xp + (int64_t)(cw + i) * plane) : 0.f;
             }
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
+            for (int u = 0; u < U; ++u) {
                 // (rows past the wave's last channel belong to channels >= C: zeros)
-                const float *wr = wt[wave * kWave + i0 + u];
+                const float *wr = wt[wave * PER + i0 + u];
 #pragma unroll
                 for (int t = 0; t < KK; ++t) acc[t] = fmaf(wr[t], xv[u], acc[t]);
             }
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(kBranchThreads) void k_spatial_branch(
     for (int t = 0; t < KK; ++t) {
         float s = bias ? ld(bias + g * KK + t) : 0.f;
 #pragma unroll
-        for (int q = 0; q < kBranchWaves; ++q) s += red[q][t][lane];
+        for (int q = 0; q < WAVES; ++q) s += red[q][t][lane];
         v[t] = s;
     }
     normalise<T, KK, float>(v, g, gain, gain_vec, offset_vec);
@@ -117,21 +119,37 @@ __global__ __launch_bounds__(kBranchThreads) void k_spatial_branch(
     for (int t = 0; t < KK; ++t) st(op + (int64_t)t * npix, v[t]);
 }
 
+// Sum over the 64 lanes (the same value in every lane): four butterfly steps
+// inside each row of 16 lanes through the VALU's lane-permute path, then the
+// four row sums through scalar registers.  (Shuffles through the LDS crossbar
+// cost a round trip each and made these kernels several times slower.)
+template <int CTRL>
+__device__ __forceinline__ float add_permuted(float x) {
+    return x + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), CTRL, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    v = add_permuted<0xB1>(v);    // quad_perm [1,0,3,2]
+    v = add_permuted<0x4E>(v);    // quad_perm [2,3,0,1]
+    v = add_permuted<0x141>(v);   // row_half_mirror
+    v = add_permuted<0x140>(v);   // row_mirror
+    const int b = __float_as_int(v);
+    return (__int_as_float(__builtin_amdgcn_readlane(b, 0)) + __int_as_float(__builtin_amdgcn_readlane(b, 16))) +
+           (__int_as_float(__builtin_amdgcn_readlane(b, 32)) + __int_as_float(__builtin_amdgcn_readlane(b, 48)));
 }
 
-constexpr int kChannelBlock = 16;   // channels whose filters one workgroup makes
+constexpr int kChannelBlock = 64;     // channels whose filters one workgroup makes
+constexpr int kChannelThreads = 1024;  // sixteen waves: the rows of a block's taps are dealt out to them
+constexpr int kChannelWaves = kChannelThreads / kWave;
 
 // grid (channel blocks of kChannelBlock, N).  LDS: the pooled vector (C floats),
 // the hidden vector (mid floats), the block's un-normalised taps.  Every dot
 // product has the lanes of a wave along the weight row (coalesced) and ends in
-// a wave reduction; several rows are in flight at a time, which is what the
-// run time depends on (the loads are dependent on nothing but latency).
+// a wave reduction; several rows are in flight per wave.  Every workgroup of a
+// sample recomputes the hidden vector, so the blocks are large: smaller ones
+// had all compute units read the same rows of w1 at once, which the L2 serves
+// one after the other.
 template <typename T, int KK>
-__global__ __launch_bounds__(kBranchThreads) void k_channel_branch(
+__global__ __launch_bounds__(kChannelThreads) void k_channel_branch(
     const T *__restrict__ pooled, const T *__restrict__ w1, const T *__restrict__ b1,
     const T *__restrict__ w2, const T *__restrict__ b2, T *__restrict__ cf, int C, int mid,
     float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
@@ -142,14 +160,15 @@ __global__ __launch_bounds__(kBranchThreads) void k_channel_branch(
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int64_t n = blockIdx.y;
     const int cb = blockIdx.x * kChannelBlock;
-    for (int c = threadIdx.x; c < C; c += kBranchThreads) v[c] = ld(pooled + n * C + c);
+    for (int c = threadIdx.x; c < C; c += kChannelThreads) v[c] = ld(pooled + n * C + c);
     __syncthreads();
     // hidden vector: four rows of w1 per wave at a time
     constexpr int RH = 4;
-    for (int m0 = wave * RH; m0 < mid; m0 += kBranchWaves * RH) {
+    for (int m0 = wave * RH; m0 < mid; m0 += kChannelWaves * RH) {
         float p[RH];
 #pragma unroll
         for (int u = 0; u < RH; ++u) p[u] = 0.f;
+#pragma unroll 4   // (all of a 256-channel row's loads go out before the first is used)
         for (int c = lane; c < C; c += kWave) {
             const float vc = v[c];
 #pragma unroll
@@ -165,13 +184,14 @@ __global__ __launch_bounds__(kBranchThreads) void k_channel_branch(
         }
     }
     __syncthreads();
-    // the block's taps: rows (cb * KK + r) of w2, eight per wave at a time
-    constexpr int RT = 8;
+    // the block's taps: rows (cb * KK + r) of w2, eighteen per wave at a time
+    constexpr int RT = 18;
     const int rows = min(kChannelBlock, C - cb) * KK;
-    for (int r0 = wave * RT; r0 < rows; r0 += kBranchWaves * RT) {
+    for (int r0 = wave * RT; r0 < rows; r0 += kChannelWaves * RT) {
         float p[RT];
 #pragma unroll
         for (int u = 0; u < RT; ++u) p[u] = 0.f;
+#pragma unroll 2
         for (int m = lane; m < mid; m += kWave) {
             const float hm = h[m];
 #pragma unroll
@@ -211,12 +231,13 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
     if (N == 0 || C == 0 || Ho * Wo == 0 || head == 0) return hipSuccess;
     if (N > 65535 || head > 65535 || C > (1 << 24) || H * W >= (1ll << 31)) return hipErrorNotSupported;
     const dim3 grid((unsigned)cdiv(Ho * Wo, kWave), (unsigned)head, (unsigned)N);
-#define DDF_SPATIAL_CASE(KK_)                                                                   \
-    hipLaunchKernelGGL((k_spatial_branch<T, KK_>), grid, dim3(kBranchThreads), 0, st, x, w, bias, \
-                       sf, (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, (float)gain,       \
+    // (as many waves per pixel tile as the LDS of the per-wave sums allows)
+#define DDF_SPATIAL_CASE(KK_, WAVES_)                                                           \
+    hipLaunchKernelGGL((k_spatial_branch<T, KK_, WAVES_>), grid, dim3(WAVES_ * kWave), 0, st, x, w, \
+                       bias, sf, (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, (float)gain, \
                        gain_vec, offset_vec)
-    if (k == 3) DDF_SPATIAL_CASE(9);
-    else if (k == 5) DDF_SPATIAL_CASE(25);
+    if (k == 3) DDF_SPATIAL_CASE(9, 8);
+    else if (k == 5) DDF_SPATIAL_CASE(25, 4);
     else return hipErrorNotSupported;
 #undef DDF_SPATIAL_CASE
     return hipGetLastError();
@@ -232,7 +253,7 @@ hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2
     if (N > 65535 || mid < 1 || lds > 48 * 1024) return hipErrorNotSupported;
     const dim3 grid((unsigned)cdiv(C, kChannelBlock), (unsigned)N);
 #define DDF_CHANNEL_CASE(KK_)                                                                    \
-    hipLaunchKernelGGL((k_channel_branch<T, KK_>), grid, dim3(kBranchThreads), lds, st, pooled, w1, \
+    hipLaunchKernelGGL((k_channel_branch<T, KK_>), grid, dim3(kChannelThreads), lds, st, pooled, w1, \
                        b1, w2, b2, cf, (int)C, (int)mid, (float)gain, gain_vec, offset_vec)
     if (k == 3) DDF_CHANNEL_CASE(9);
     else if (k == 5) DDF_CHANNEL_CASE(25);

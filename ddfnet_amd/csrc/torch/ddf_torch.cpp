@@ -191,6 +191,152 @@ at::Tensor ddf(at::Tensor features, at::Tensor channel_filter, at::Tensor spatia
                               (int64_t)combine, (int64_t)variant);
 }
 
+// Up-sampling DDF (DDFUpPack.forward, ddf/ddf.py:264-272 of the reference: one
+// ddf call per sub-pixel branch, torch.stack, F.pixel_shuffle) as one operator:
+// one library call forward, one backward.  `filters` holds the scale*scale
+// channel filters followed by the scale*scale spatial filters.
+class DDFUpAutograd : public torch::autograd::Function<DDFUpAutograd> {
+public:
+    // (filters as a TensorList: that is the list type whose elements autograd tracks)
+    static at::Tensor forward(AutogradContext *ctx, const at::Tensor &features, at::TensorList filters,
+                              int64_t k, int64_t d, int64_t scale, int64_t combine) {
+        const int64_t branches = scale * scale;
+        const int64_t b = features.size(0), c = features.size(1), h = features.size(2),
+                      w = features.size(3);
+        const void *cf[DDF_UP_MAX_BRANCHES], *sf[DDF_UP_MAX_BRANCHES];
+        for (int64_t i = 0; i < branches; ++i) {
+            cf[i] = filters[i].data_ptr();
+            sf[i] = filters[branches + i].data_ptr();
+        }
+        at::Tensor out = at::empty({b, c, h * scale, w * scale}, features.options());
+        {
+            c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(features.device());
+            check_status(ddf_hip_up_forward(features.data_ptr(), cf, sf, out.data_ptr(), b, c, h, w,
+                                            (int)k, (int)d, (int)scale, (int)combine,
+                                            dtype_code(features.scalar_type()),
+                                            current_stream(features)));
+        }
+        bool any = features.requires_grad();
+        for (const auto &t : filters) any = any || t.requires_grad();
+        if (any) {
+            variable_list saved;
+            saved.reserve(1 + filters.size());
+            saved.push_back(features);
+            for (const auto &t : filters) saved.push_back(t);
+            ctx->save_for_backward(saved);
+        }
+        ctx->saved_data["k"] = k;
+        ctx->saved_data["d"] = d;
+        ctx->saved_data["scale"] = scale;
+        ctx->saved_data["combine"] = combine;
+        return out;
+    }
+
+    static variable_list backward(AutogradContext *ctx, variable_list grads) {
+        const auto saved = ctx->get_saved_variables();
+        const at::Tensor &features = saved[0];
+        const int k = (int)ctx->saved_data["k"].toInt(), d = (int)ctx->saved_data["d"].toInt(),
+                  scale = (int)ctx->saved_data["scale"].toInt(),
+                  combine = (int)ctx->saved_data["combine"].toInt();
+        const int branches = scale * scale;
+        const at::Tensor go = grads[0].to(features.scalar_type()).contiguous();
+        variable_list result(1 + 2 * branches + 4);
+        unsigned need = 0;
+        const void *cf[DDF_UP_MAX_BRANCHES], *sf[DDF_UP_MAX_BRANCHES];
+        void *dcf[DDF_UP_MAX_BRANCHES], *dsf[DDF_UP_MAX_BRANCHES];
+        if (ctx->needs_input_grad(0)) {
+            need |= DDF_NEED_DX;
+            result[0] = at::empty_like(features);
+        }
+        for (int i = 0; i < branches; ++i) {
+            cf[i] = saved[1 + i].data_ptr();
+            sf[i] = saved[1 + branches + i].data_ptr();
+            dcf[i] = dsf[i] = nullptr;
+            if (ctx->needs_input_grad(1 + i)) {
+                need |= DDF_NEED_DCF;
+                result[1 + i] = at::empty_like(saved[1 + i]);
+                dcf[i] = result[1 + i].data_ptr();
+            }
+            if (ctx->needs_input_grad(1 + branches + i)) {
+                need |= DDF_NEED_DSF;
+                result[1 + branches + i] = at::empty_like(saved[1 + branches + i]);
+                dsf[i] = result[1 + branches + i].data_ptr();
+            }
+        }
+        if (need) {
+            const int64_t b = features.size(0), c = features.size(1), h = features.size(2),
+                          w = features.size(3);
+            const int dt = dtype_code(features.scalar_type());
+            c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(features.device());
+            const size_t bytes = ddf_hip_up_backward_workspace_bytes(b, c, h, w, k, d, scale, combine,
+                                                                     dt, need);
+            at::Tensor ws = at::empty({(int64_t)std::max<size_t>(bytes, 1)},
+                                      features.options().dtype(at::kByte));
+            check_status(ddf_hip_up_backward(
+                go.data_ptr(), features.data_ptr(), cf, sf,
+                result[0].defined() ? result[0].data_ptr() : nullptr, dcf, dsf, ws.data_ptr(), bytes,
+                b, c, h, w, k, d, scale, combine, dt, need, current_stream(features)));
+        }
+        return result;
+    }
+};
+
+// ddf_up(features, channel_filters, spatial_filters, kernel_size, dilation, scale_factor,
+// kernel_combine): the checks of DDFUpFunction.forward in functional.py.  The caller has
+// asked ddf_hip_up_forward's coverage (functional.ddf_up falls back to the composition).
+at::Tensor ddf_up(at::Tensor features, std::vector<at::Tensor> channel_filters,
+                  std::vector<at::Tensor> spatial_filters, int64_t kernel_size, int64_t dilation,
+                  int64_t scale, const std::string &kernel_combine) {
+    const int64_t branches = scale * scale;
+    if (scale < 2 || branches > DDF_UP_MAX_BRANCHES ||
+        (int64_t)channel_filters.size() != branches || (int64_t)spatial_filters.size() != branches)
+        assertion_error("expected " + std::to_string(branches) + " channel filters followed by " +
+                        std::to_string(branches) + " spatial filters");
+    if (!features.is_cuda()) assertion_error("input feature must be a CUDA tensor.");
+    int combine;
+    if (kernel_combine == "mul") combine = DDF_MUL;
+    else if (kernel_combine == "add") combine = DDF_ADD;
+    else assertion_error("only support mul or add combination, instead of " + kernel_combine);
+    if ((kernel_size - 1) % 2 != 0 || kernel_size < 1 || dilation < 1) assertion_error("");
+    at::ScalarType dtype = features.scalar_type();
+    for (const auto *list : {&channel_filters, &spatial_filters})
+        for (const auto &t : *list) {
+            if (!t.is_cuda()) assertion_error("filters must be CUDA tensors.");
+            dtype = at::promote_types(dtype, t.scalar_type());
+        }
+    if (at::autocast::is_autocast_enabled(at::kCUDA) &&
+        at::autocast::get_autocast_dtype(at::kCUDA) == at::kHalf && dtype == at::kFloat)
+        dtype = at::kHalf;
+    if (dtype_code(dtype) < 0) {
+        std::ostringstream os;
+        os << "unsupported dtype " << dtype;
+        assertion_error(os.str());
+    }
+    if (features.dim() != 4) assertion_error("features must be 4-dimensional");
+    features = features.to(dtype).contiguous();
+    const int64_t b = features.size(0), c = features.size(1), h = features.size(2), w = features.size(3);
+    variable_list filters;
+    filters.reserve(2 * branches);
+    for (auto &t : channel_filters) {
+        t = t.to(dtype).contiguous();
+        if (t.dim() != 4 || t.size(0) != b || t.size(1) != c || t.size(2) != kernel_size ||
+            t.size(3) != kernel_size)
+            assertion_error("channel_filter size " + size_string(t) + " does not match feature size " +
+                            size_string(features));
+        filters.push_back(t);
+    }
+    for (auto &t : spatial_filters) {
+        t = t.to(dtype).contiguous();
+        if (t.dim() != 4 || t.size(0) != b || t.size(1) != kernel_size * kernel_size ||
+            t.size(2) != h || t.size(3) != w)
+            assertion_error("spatial_filter size " + size_string(t) + " does not match feature size " +
+                            size_string(features));
+        filters.push_back(t);
+    }
+    return DDFUpAutograd::apply(features, at::TensorList(filters), kernel_size, dilation, scale,
+                                (int64_t)combine);
+}
+
 const void *ptr_or_null(const c10::optional<at::Tensor> &t) {
     return t.has_value() && t->defined() ? t->data_ptr() : nullptr;
 }
@@ -256,6 +402,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("ddf", &ddf, py::arg("features"), py::arg("channel_filter"), py::arg("spatial_filter"),
           py::arg("kernel_size") = 3, py::arg("dilation") = 1, py::arg("stride") = 1,
           py::arg("kernel_combine") = "mul", py::arg("version") = "");
+    m.def("ddf_up", &ddf_up, py::arg("features"), py::arg("channel_filters"),
+          py::arg("spatial_filters"), py::arg("kernel_size") = 3, py::arg("dilation") = 1,
+          py::arg("scale_factor") = 2, py::arg("kernel_combine") = "mul");
     m.def("ddf_pack_forward", &ddf_pack_forward,
           "DDFPack.forward without gradients: pool, channel branch, spatial branch, operator");
     m.def("library_version", []() { return ddf_hip_version(); });

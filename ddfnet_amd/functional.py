@@ -269,6 +269,9 @@ def ddf_up(features, channel_filters, spatial_filters, kernel_size=3, dilation=1
     channel_filters, spatial_filters = tuple(channel_filters), tuple(spatial_filters)
     assert len(channel_filters) == len(spatial_filters) == scale_factor ** 2
     if _lib.up_forward_covers(kernel_size, scale_factor):
+        if _C is not None:   # the same operator as a C++ autograd function
+            return _C.ddf_up(features, list(channel_filters), list(spatial_filters), kernel_size,
+                             dilation, scale_factor, kernel_combine)
         return DDFUpFunction.apply(features, kernel_size, dilation, scale_factor, kernel_combine,
                                    *(channel_filters + spatial_filters))
     outs = [ddf(features, cf, sf, kernel_size, dilation, 1, kernel_combine)

@@ -144,13 +144,23 @@ def test_full_size_equals_composition_of_ddf(dtype):
 
 
 def test_ddfuppack_uses_the_fused_operator(monkeypatch):
+    from ddfnet_amd import functional
+    up = ddfnet_amd.DDFUpPack(8, scale_factor=2).cuda()
+    x = torch.randn(1, 8, 6, 6, device='cuda')
+
+    def no_branch_calls(*a, **kw):
+        raise AssertionError('the per-branch composition ran')
+    monkeypatch.setattr(functional, 'ddf', no_branch_calls)
+    with torch.no_grad():
+        out = up(x)                      # C++ operator where the torch extension is built
+    # the ctypes route of the same library call
     calls = []
     real = _lib.up_forward
+    monkeypatch.setattr(functional, '_C', None)
     monkeypatch.setattr(_lib, 'up_forward', lambda *a: (calls.append(1), real(*a))[1])
-    up = ddfnet_amd.DDFUpPack(8, scale_factor=2).cuda()
     with torch.no_grad():
-        up(torch.randn(1, 8, 6, 6, device='cuda'))
-    assert calls == [1]
+        again = up(x)
+    assert calls == [1] and torch.equal(out, again)
 
 
 def _random_up_cases(count, seed):
