@@ -138,18 +138,39 @@ int scratch_of_current_device(void **out) {
 // feature gradients (when dX is wanted) and one branch's own workspace.
 struct UpWorkspace {
     size_t lattices, dx_parts, branch, total;
+    // all branches as one batch on the row-register kernels (batched = false: not covered)
+    bool batched;
+    size_t cf_all, sf_all, dcf_all, dsf_all, batch_ws;
 };
 
 UpWorkspace up_workspace(const ddf::Problem &p, int scale, int dtype, unsigned need) {
     const size_t esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
     const size_t n_x = (size_t)(p.N * p.C * p.H * p.W);
-    UpWorkspace w;
-    w.lattices = align256(n_x * esz * scale * scale);
-    w.dx_parts = (need & DDF_NEED_DX) ? align256(n_x * esz * scale * scale) : 0;
+    const size_t branches = (size_t)scale * scale;
+    UpWorkspace w{};
+    w.lattices = align256(n_x * esz * branches);
+    w.dx_parts = (need & DDF_NEED_DX) ? align256(n_x * esz * branches) : 0;
     w.branch = ddf::tiled_backward_supported(p, dtype)
                    ? align256(ddf::tiled_backward_workspace(p, dtype, need))
                    : 0;
     w.total = w.lattices + w.dx_parts + w.branch;
+    // The batch of scale*scale * N samples: the branches' filters and filter
+    // gradients back to back, and the kernels' own workspace for that batch.
+    const ddf::Problem pb = ddf::make_problem(p.N * (int64_t)branches, p.C, p.H, p.W, p.k, p.d, 1,
+                                              p.mul ? DDF_MUL : DDF_ADD);
+    w.batched = dtype != DDF_F64 && p.N * (int64_t)branches <= (1 << 24) &&
+                ddf::rows_cover_backward(pb, dtype) && !ddf::small_supported(pb);
+    if (w.batched) {
+        const size_t n_cf = (size_t)(p.N * p.C * p.kk), n_sf = (size_t)(p.N * p.kk * p.H * p.W);
+        w.cf_all = align256(n_cf * esz * branches);
+        w.sf_all = align256(n_sf * esz * branches);
+        w.dcf_all = (need & DDF_NEED_DCF) ? w.cf_all : 0;
+        w.dsf_all = (need & DDF_NEED_DSF) ? w.sf_all : 0;
+        w.batch_ws = align256(ddf::rows_filters_workspace(pb, dtype, need));
+        const size_t total = w.lattices + w.dx_parts + w.cf_all + w.sf_all + w.dcf_all + w.dsf_all +
+                             w.batch_ws;
+        w.total = std::max(w.total, total);   // (room for the branch-by-branch route as well)
+    }
     return w;
 }
 
@@ -161,11 +182,40 @@ int up_backward_typed(const ddf::Problem &p, int scale, const void *go, const vo
     unsigned char *base = static_cast<unsigned char *>(ws);
     T *lat = reinterpret_cast<T *>(base);
     T *parts = reinterpret_cast<T *>(base + w.lattices);
-    void *branch_ws = w.branch ? base + w.lattices + w.dx_parts : nullptr;
     const int64_t n_x = p.N * p.C * p.H * p.W;
+    const int branches = scale * scale;
     hipError_t err = ddf::up_split_lattices<T>((const T *)go, lat, p.N * p.C, p.H, p.W, scale, stream);
     if (err != hipSuccess) return fail_hip(err, "ddf_hip_up_backward split launch");
-    for (int b = 0; b < scale * scale; ++b) {
+
+    // All branches as one batch of scale*scale * N samples that share the features:
+    // a handful of launches that fill the machine, instead of three or four small
+    // ones per branch.
+    if constexpr (sizeof(T) != 8) if (w.batched) {
+        unsigned char *q = base + w.lattices + w.dx_parts;
+        T *cf_all = reinterpret_cast<T *>(q); q += w.cf_all;
+        T *sf_all = reinterpret_cast<T *>(q); q += w.sf_all;
+        T *dcf_all = w.dcf_all ? reinterpret_cast<T *>(q) : nullptr; q += w.dcf_all;
+        T *dsf_all = w.dsf_all ? reinterpret_cast<T *>(q) : nullptr; q += w.dsf_all;
+        const int64_t n_cf = p.N * p.C * p.kk, n_sf = p.N * p.kk * p.H * p.W;
+        err = ddf::up_gather_filters<T>(cfs, sfs, cf_all, sf_all, n_cf, n_sf, branches, stream);
+        if (err != hipSuccess) return fail_hip(err, "ddf_hip_up_backward gather launch");
+        const ddf::Problem pb = ddf::make_problem(p.N * branches, p.C, p.H, p.W, p.k, p.d, 1,
+                                                  p.mul ? DDF_MUL : DDF_ADD);
+        err = ddf::rows_backward_shared_features<T>(
+            pb, (int)p.N, lat, (const T *)x, cf_all, sf_all, (need & DDF_NEED_DX) ? parts : nullptr,
+            dcf_all, dsf_all, w.batch_ws ? q : nullptr, need, stream);
+        if (err == hipSuccess) {
+            err = ddf::up_finish<T>((need & DDF_NEED_DX) ? parts : nullptr, (T *)dx, n_x, branches,
+                                    dcf_all, dsf_all, dcfs, dsfs, n_cf, n_sf, stream);
+            if (err != hipSuccess) return fail_hip(err, "ddf_hip_up_backward finish launch");
+            return DDF_OK;
+        }
+        // (e.g. features not 16-byte aligned: nothing was launched, take the other route)
+        if (err != hipErrorNotSupported) return fail_hip(err, "ddf_hip_up_backward batch launch");
+    }
+
+    void *branch_ws = w.branch ? base + w.lattices + w.dx_parts : nullptr;
+    for (int b = 0; b < branches; ++b) {
         unsigned bneed = need & DDF_NEED_DX;
         if ((need & DDF_NEED_DCF) && dcfs && dcfs[b]) bneed |= DDF_NEED_DCF;
         if ((need & DDF_NEED_DSF) && dsfs && dsfs[b]) bneed |= DDF_NEED_DSF;
@@ -178,7 +228,7 @@ int up_backward_typed(const ddf::Problem &p, int scale, const void *go, const vo
         if (rc != DDF_OK) return rc;
     }
     if (need & DDF_NEED_DX) {
-        err = ddf::up_sum_parts<T>(parts, (T *)dx, n_x, scale * scale, stream);
+        err = ddf::up_sum_parts<T>(parts, (T *)dx, n_x, branches, stream);
         if (err != hipSuccess) return fail_hip(err, "ddf_hip_up_backward sum launch");
     }
     return DDF_OK;

@@ -101,6 +101,18 @@ hipError_t up_split_lattices(const T *go, T *lat, int64_t planes, int64_t H, int
                              hipStream_t st);
 template <typename T>
 hipError_t up_sum_parts(const T *in, T *out, int64_t count, int parts, hipStream_t st);
+// For the backward pass of all branches as one batch: the branches' filters
+// copied back to back (cf / sf: host arrays of `branches` device pointers), and
+// afterwards dX summed from the branches' parts (parts may be null) together
+// with the batch's filter gradients copied out to the branches' tensors (null
+// destinations are skipped; dcf_all / dsf_all may be null).
+template <typename T>
+hipError_t up_gather_filters(const void *const *cf, const void *const *sf, T *cf_all, T *sf_all,
+                             int64_t n_cf, int64_t n_sf, int branches, hipStream_t st);
+template <typename T>
+hipError_t up_finish(const T *parts, T *dx, int64_t n_x, int branches, const T *dcf_all,
+                     const T *dsf_all, void *const *dcfs, void *const *dsfs, int64_t n_cf,
+                     int64_t n_sf, hipStream_t st);
 
 // Tiny planes (H*W <= 64), 3x3, stride 1: forward (backward = false: x -> out)
 // and feature gradient (backward = true: dO -> dX), G = 256 / (H*W) channel
@@ -127,9 +139,19 @@ size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);
 // The row-register kernels cover the feature gradient and, in a launch of its
 // own, the filter gradients of this problem (pointer alignment assumed).
 bool rows_cover_backward(const Problem &p, int dtype);
+// x_mod != 0: the batch p.N is several groups of x_mod samples sharing one set
+// of features x (x_mod samples long); everything else is indexed by the sample.
 template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
-                               T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st);
+                               T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st,
+                               int x_mod = 0);
+// The whole backward pass of such a batch on the row-register kernels, or
+// hipErrorNotSupported before anything is launched (shape or alignment not
+// covered).  `ws`: rows_filters_workspace(p) bytes.
+template <typename T>
+hipError_t rows_backward_shared_features(const Problem &p, int x_mod, const T *go, const T *x,
+                                         const T *cf, const T *sf, T *dx, T *dcf, T *dsf, void *ws,
+                                         unsigned need, hipStream_t st);
 
 // Names of the kernels a forward / backward call on the tiled families would
 // launch, written into buf (at most len bytes); returns snprintf's count.

@@ -59,7 +59,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     RowsGeom g, const T *__restrict__ go, const T *__restrict__ x, const T *__restrict__ cf,
     const T *__restrict__ sf, T *__restrict__ dx, T *__restrict__ dcf, T *__restrict__ dsf,
     typename Acc<T>::type *__restrict__ ws_sf, typename Acc<T>::type *__restrict__ ws_cf,
-    unsigned need) {
+    unsigned need, int x_mod) {
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RAD = K / 2, HX = RAD * D, HY = RAD * D;
     constexpr int ROWS = R + 2 * HY;
@@ -86,7 +86,10 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     Lane<R, HY, VX> ln;
     ln.init(g, wk.strip, lane);
 
-    const T *xs = x + (wk.n * g.C + c_first) * plane;
+    // x_mod != 0: the batch is several groups of x_mod samples that share one set of
+    // features (the sub-pixel branches of the up-sampling operator's gradient)
+    const int64_t xn = x_mod ? wk.n % x_mod : wk.n;
+    const T *xs = x + (xn * g.C + c_first) * plane;
     const T *gs = go + (wk.n * g.C + c_first) * plane;
     T *ds = DX ? dx + (wk.n * g.C + c_first) * plane : nullptr;
     uint32_t xb[ROWS], ob[R];

@@ -94,7 +94,7 @@ template <typename T, int VX, int R, bool DX>
 hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, const T *x,
                             const T *cf, const T *sf, T *dx, T *dcf, T *dsf,
                             typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
-                            unsigned need, hipStream_t st) {
+                            unsigned need, int x_mod, hipStream_t st) {
     using A = typename Acc<T>::type;
     // waves per SIMD the registers are budgeted for: 'mul' keeps the spatial taps
     // as well, the fused feature gradient a second set of them
@@ -108,7 +108,7 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
 #define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
     hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, R, PAD_, DX, kFilterStages,            \
                                        MUL_ ? WPE_MUL : WPE_ADD>),                               \
-                       grid, block, lds, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need)
+                       grid, block, lds, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod)
     if (p.mul) {
         if (pad) DDF_ROWSF_CASE(true, true);
         else DDF_ROWSF_CASE(true, false);
@@ -124,7 +124,7 @@ template <typename T, int K, int D, int VX>
 hipError_t launch_taprow_kdv(const Problem &p, const RowsGeom &g, const T *go, const T *x,
                              const T *cf, const T *sf, T *dcf, T *dsf,
                              typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
-                             unsigned need, hipStream_t st) {
+                             unsigned need, int x_mod, hipStream_t st) {
     using A = typename Acc<T>::type;
     constexpr int kTaprowStages = 8, kWpe = 3;   // channels in flight per wave; waves per SIMD
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kTaprowWaves);
@@ -132,7 +132,7 @@ hipError_t launch_taprow_kdv(const Problem &p, const RowsGeom &g, const T *go, c
     const bool pad = g.lp > g.lpr;
 #define DDF_TAPROW_CASE(MUL_, PAD_)                                                              \
     hipLaunchKernelGGL((k_rows_taprow_filters<T, K, D, MUL_, VX, 1, PAD_, kTaprowStages, kWpe>), \
-                       grid, block, lds, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need)
+                       grid, block, lds, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod)
     if (p.mul) {
         if (pad) DDF_TAPROW_CASE(true, true);
         else DDF_TAPROW_CASE(true, false);
@@ -148,14 +148,14 @@ template <typename T, int VX>
 hipError_t launch_taprow_v(const Problem &p, const RowsGeom &g, const T *go, const T *x,
                            const T *cf, const T *sf, T *dcf, T *dsf,
                            typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
-                           unsigned need, hipStream_t st) {
+                           unsigned need, int x_mod, hipStream_t st) {
     if (p.k == 3 && p.d == 1)
-        return launch_taprow_kdv<T, 3, 1, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+        return launch_taprow_kdv<T, 3, 1, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
     if (p.k == 5 && p.d == 1)
-        return launch_taprow_kdv<T, 5, 1, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+        return launch_taprow_kdv<T, 5, 1, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
     if constexpr (VX >= 4) {
         if (p.k == 5 && p.d == 2)
-            return launch_taprow_kdv<T, 5, 2, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            return launch_taprow_kdv<T, 5, 2, VX>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
     }
     return hipErrorNotSupported;
 }
@@ -169,7 +169,8 @@ hipError_t launch_taprow_v(const Problem &p, const RowsGeom &g, const T *go, con
 // rows_filters_workspace() bytes.
 template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
-                               T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st) {
+                               T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st,
+                               int x_mod) {
     using A = typename Acc<T>::type;
     const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
     const bool fused = dx != nullptr;
@@ -193,23 +194,23 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     if constexpr (sizeof(T) != 8) {
         if (taprow) {
             if (vx == 4)
-                err = rows::launch_taprow_v<T, 4>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+                err = rows::launch_taprow_v<T, 4>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             else if (vx == 2)
-                err = rows::launch_taprow_v<T, 2>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+                err = rows::launch_taprow_v<T, 2>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             if constexpr (sizeof(T) == 2) {
                 if (vx == 8)
-                    err = rows::launch_taprow_v<T, 8>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+                    err = rows::launch_taprow_v<T, 8>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             }
         } else if (fused) {
             if (vx == 2 && r == 2)
-                err = rows::launch_filters_v<T, 2, 2, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+                err = rows::launch_filters_v<T, 2, 2, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             else if (vx == 4 && r == 1)
-                err = rows::launch_filters_v<T, 4, 1, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+                err = rows::launch_filters_v<T, 4, 1, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
         } else {
             if (vx == 4 && r == 1)
-                err = rows::launch_filters_v<T, 4, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+                err = rows::launch_filters_v<T, 4, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             else if (vx == 2 && r == 1)
-                err = rows::launch_filters_v<T, 2, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, st);
+                err = rows::launch_filters_v<T, 2, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
         }
     }
     if (err != hipSuccess) return err;
@@ -221,11 +222,49 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     return err;
 }
 
+template <typename T>
+hipError_t rows_backward_shared_features(const Problem &p, int x_mod, const T *go, const T *x,
+                                         const T *cf, const T *sf, T *dx, T *dcf, T *dsf, void *ws,
+                                         unsigned need, hipStream_t st) {
+    if constexpr (sizeof(T) == 8) {
+        return hipErrorNotSupported;
+    } else {
+        const int dtype = sizeof(T) == 2 ? DDF_F16 : DDF_F32;
+        const unsigned fneed = need & (DDF_NEED_DCF | DDF_NEED_DSF);
+        const bool want_dx = need & DDF_NEED_DX;
+        RowsGeom g;
+        int vx, r;
+        // every vector access 16-byte aligned, so no launch below can turn the call down
+        if ((((uintptr_t)go | (uintptr_t)x | (uintptr_t)sf | (uintptr_t)dx | (uintptr_t)dsf) & 15u) != 0)
+            return hipErrorNotSupported;
+        if (small_supported(p)) return hipErrorNotSupported;
+        if (want_dx && fneed && rows_filters_geometry(p, dtype, true, &g, &vx, &r))
+            return rows_filters_launch<T>(p, go, x, cf, sf, dx, dcf, dsf, ws, fneed, st, x_mod);
+        if (want_dx && !rows_geometry(p, dtype, 0, &g, &vx, &r)) return hipErrorNotSupported;
+        if (fneed && !rows_taprow_geometry(p, dtype, &g, &vx, &r) &&
+            !rows_filters_geometry(p, dtype, false, &g, &vx, &r))
+            return hipErrorNotSupported;
+        hipError_t err = hipSuccess;
+        if (want_dx) {
+            err = rows_launch<T>(p, true, go, cf, sf, dx, st);
+            if (err != hipSuccess) return err;
+        }
+        if (fneed) {
+            err = rows_filters_launch<T>(p, go, x, cf, sf, (T *)nullptr, dcf, dsf, ws, fneed, st, x_mod);
+            if (err == hipErrorNotSupported) err = hipErrorUnknown;   // (ruled out above)
+        }
+        return err;
+    }
+}
+
 #define DDF_INSTANTIATE_ROWS(T)                                                              \
     template hipError_t rows_filters_launch<T>(const Problem &, const T *, const T *, const T *, \
                                                const T *, T *, T *, T *, void *, unsigned,   \
-                                               hipStream_t);                                  \
+                                               hipStream_t, int);                             \
     template hipError_t rows_launch<T>(const Problem &, bool, const T *, const T *, const T *, \
-                                       T *, hipStream_t);
+                                       T *, hipStream_t);                                     \
+    template hipError_t rows_backward_shared_features<T>(const Problem &, int, const T *,    \
+                                                         const T *, const T *, const T *, T *, \
+                                                         T *, T *, void *, unsigned, hipStream_t);
 
 }  // namespace ddf

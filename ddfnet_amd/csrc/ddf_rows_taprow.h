@@ -41,7 +41,7 @@ __global__ __launch_bounds__(kWave * kTaprowWaves, WPE) void k_rows_taprow_filte
     RowsGeom g, const T *__restrict__ go, const T *__restrict__ x, const T *__restrict__ cf,
     const T *__restrict__ sf, T *__restrict__ dcf, T *__restrict__ dsf,
     typename Acc<T>::type *__restrict__ ws_sf, typename Acc<T>::type *__restrict__ ws_cf,
-    unsigned need) {
+    unsigned need, int x_mod) {
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RAD = K / 2, HX = RAD * D;
     constexpr int NW = VX * sizeof(T) / 4;
@@ -65,7 +65,8 @@ __global__ __launch_bounds__(kWave * kTaprowWaves, WPE) void k_rows_taprow_filte
     Lane<R, 0, VX> ln;
     ln.init(g, wk.strip, lane, (trow - RAD) * D);
 
-    const T *xs = x + (wk.n * g.C + c0) * plane;
+    const int64_t xn = x_mod ? wk.n % x_mod : wk.n;   // (see k_rows_filters)
+    const T *xs = x + (xn * g.C + c0) * plane;
     const T *gs = go + (wk.n * g.C + c0) * plane;
     uint32_t xb[R], ob[R];
 #pragma unroll

@@ -279,7 +279,95 @@ __global__ __launch_bounds__(kThreads) void k_up_sum(const T *__restrict__ in,
     st(out + idx, acc);
 }
 
+// The branches' filters, back to back: cf_all[b] = cf of branch b (n_cf elements),
+// sf_all[b] = sf of branch b (n_sf elements).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void k_up_gather(UpFilters<T> f, T *__restrict__ cf_all,
+                                                        T *__restrict__ sf_all, int64_t n_cf,
+                                                        int64_t n_sf, int branches) {
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t per = n_cf + n_sf;
+    if (idx >= per * branches) return;
+    const int b = (int)(idx / per);
+    const int64_t e = idx - b * per;
+    if (e < n_cf) cf_all[b * n_cf + e] = f.cf[b][e];
+    else sf_all[b * n_sf + (e - n_cf)] = f.sf[b][e - n_cf];
+}
+
+template <typename T>
+struct UpGrads {
+    T *dcf[DDF_UP_MAX_BRANCHES];
+    T *dsf[DDF_UP_MAX_BRANCHES];
+};
+
+// dX = sum of the branches' parts (parts != null); the branches' filter
+// gradients from where the batched kernels left them back to back to the
+// tensors they belong to (a null destination was not asked for).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void k_up_finish(
+    const T *__restrict__ parts, T *__restrict__ dx, int64_t n_x, int branches,
+    const T *__restrict__ dcf_all, const T *__restrict__ dsf_all, UpGrads<T> g, int64_t n_cf,
+    int64_t n_sf) {
+    using A = typename Acc<T>::type;
+    int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t n_dx = parts ? n_x : 0;
+    if (idx < n_dx) {
+        A acc = 0;
+        for (int b = 0; b < branches; ++b) acc += (A)ld(parts + (int64_t)b * n_x + idx);
+        st(dx + idx, acc);
+        return;
+    }
+    idx -= n_dx;
+    const int64_t all_cf = dcf_all ? n_cf * branches : 0;
+    if (idx < all_cf) {
+        const int b = (int)(idx / n_cf);
+        if (g.dcf[b]) g.dcf[b][idx - b * n_cf] = dcf_all[idx];
+        return;
+    }
+    idx -= all_cf;
+    if (dsf_all && idx < n_sf * branches) {
+        const int b = (int)(idx / n_sf);
+        if (g.dsf[b]) g.dsf[b][idx - b * n_sf] = dsf_all[idx];
+    }
+}
+
 }  // namespace
+
+template <typename T>
+hipError_t up_gather_filters(const void *const *cf, const void *const *sf, T *cf_all, T *sf_all,
+                             int64_t n_cf, int64_t n_sf, int branches, hipStream_t stream) {
+    const int64_t total = (n_cf + n_sf) * branches;
+    if (total == 0) return hipSuccess;
+    UpFilters<T> f;
+    for (int b = 0; b < DDF_UP_MAX_BRANCHES; ++b) {
+        f.cf[b] = b < branches ? (const T *)cf[b] : nullptr;
+        f.sf[b] = b < branches ? (const T *)sf[b] : nullptr;
+    }
+    const int64_t grid = cdiv(total, kThreads);
+    if (grid > 2147483647) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((k_up_gather<T>), dim3((unsigned)grid), dim3(kThreads), 0, stream, f, cf_all,
+                       sf_all, n_cf, n_sf, branches);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t up_finish(const T *parts, T *dx, int64_t n_x, int branches, const T *dcf_all,
+                     const T *dsf_all, void *const *dcfs, void *const *dsfs, int64_t n_cf,
+                     int64_t n_sf, hipStream_t stream) {
+    const int64_t total = (parts ? n_x : 0) + (dcf_all ? n_cf * branches : 0) +
+                          (dsf_all ? n_sf * branches : 0);
+    if (total == 0) return hipSuccess;
+    UpGrads<T> g;
+    for (int b = 0; b < DDF_UP_MAX_BRANCHES; ++b) {
+        g.dcf[b] = (b < branches && dcfs) ? (T *)dcfs[b] : nullptr;
+        g.dsf[b] = (b < branches && dsfs) ? (T *)dsfs[b] : nullptr;
+    }
+    const int64_t grid = cdiv(total, kThreads);
+    if (grid > 2147483647) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((k_up_finish<T>), dim3((unsigned)grid), dim3(kThreads), 0, stream, parts, dx,
+                       n_x, branches, dcf_all, dsf_all, g, n_cf, n_sf);
+    return hipGetLastError();
+}
 
 template <typename T>
 hipError_t up_split_lattices(const T *go, T *lat, int64_t planes, int64_t H, int64_t W, int scale,
@@ -338,7 +426,11 @@ hipError_t up_forward(int64_t N, int64_t C, int64_t H, int64_t W, int k, int d, 
                                       hipStream_t);                                             \
     template hipError_t up_split_lattices<T>(const T *, T *, int64_t, int64_t, int64_t, int,    \
                                              hipStream_t);                                      \
-    template hipError_t up_sum_parts<T>(const T *, T *, int64_t, int, hipStream_t);
+    template hipError_t up_sum_parts<T>(const T *, T *, int64_t, int, hipStream_t);             \
+    template hipError_t up_gather_filters<T>(const void *const *, const void *const *, T *, T *, \
+                                             int64_t, int64_t, int, hipStream_t);              \
+    template hipError_t up_finish<T>(const T *, T *, int64_t, int, const T *, const T *,        \
+                                     void *const *, void *const *, int64_t, int64_t, hipStream_t);
 DDF_UP_INSTANCE(__half)
 DDF_UP_INSTANCE(float)
 DDF_UP_INSTANCE(double)

@@ -108,6 +108,29 @@ def test_misaligned_output(scale, dtype):
     assert buf[0].item() == 7.0 and buf[-1].item() == 7.0    # nothing outside the result
 
 
+def test_backward_routes_agree():
+    """The gradient runs all branches as one batch on the row-register kernels;
+    features that are not 16-byte aligned take the branch-by-branch route."""
+    x, cfs, sfs, go = up_case(2, 6, 8, 12, 3, 2, torch.float32, seed=9)
+    want_x, want_cf, want_sf = oracle.up_backward(go, x, cfs, sfs, 3, 1, 2, 'mul')
+    cfd, sfd, god = [t.cuda() for t in cfs], [t.cuda() for t in sfs], go.cuda()
+    buf = torch.zeros(x.numel() + 1, device='cuda')
+    for shift in (0, 1):
+        xd = buf[shift:shift + x.numel()].view_as(x)
+        xd.copy_(x)
+        assert xd.data_ptr() % 16 == 4 * shift
+        gx = torch.empty(x.shape, device='cuda')
+        gcf = [torch.empty_like(t) for t in cfd]
+        gsf = [torch.empty_like(t) if b != 2 else None for b, t in enumerate(sfd)]   # one not wanted
+        _lib.up_backward(god, xd, cfd, sfd, gx, gcf, gsf, 3, 1, 2, 'mul')
+        torch.cuda.synchronize()
+        assert rel_err(gx, want_x) <= 1e-5
+        for b in range(4):
+            assert rel_err(gcf[b], want_cf[b]) <= 1e-5
+            if gsf[b] is not None:
+                assert rel_err(gsf[b], want_sf[b]) <= 1e-5
+
+
 def test_mixed_dtypes_and_partial_gradients():
     """fp16 features with fp32 filters promote to fp32; only the gradients
     asked for come back."""
