@@ -159,7 +159,7 @@ UpWorkspace up_workspace(const ddf::Problem &p, int scale, int dtype, unsigned n
     const ddf::Problem pb = ddf::make_problem(p.N * (int64_t)branches, p.C, p.H, p.W, p.k, p.d, 1,
                                               p.mul ? DDF_MUL : DDF_ADD);
     w.batched = dtype != DDF_F64 && p.N * (int64_t)branches <= (1 << 24) &&
-                ddf::rows_cover_backward(pb, dtype) && !ddf::small_supported(pb);
+                ddf::rows_cover_backward(pb, dtype);
     if (w.batched) {
         const size_t n_cf = (size_t)(p.N * p.C * p.kk), n_sf = (size_t)(p.N * p.kk * p.H * p.W);
         w.cf_all = align256(n_cf * esz * branches);

@@ -12,9 +12,9 @@ namespace ddf {
 int describe_forward(const Problem &p, int dtype, char *buf, int len) {
     RowsGeom rg; int vx, r;
     WaveGeom wg; int ps, nv;
-    if (small_supported(p)) return snprintf(buf, len, "k_small");
     if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 && rows_geometry(p, dtype, 0, &rg, &vx, &r))
         return snprintf(buf, len, "k_rows<VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
+    if (small_supported(p)) return snprintf(buf, len, "k_small");
     if (wave_geometry(p, dtype, kWaveForward, 0, &wg, &ps, &nv))
         return snprintf(buf, len, "k_forward<PS=%d,NV=%d,V=%d>", ps, nv, wg.vec);
     return snprintf(buf, len, "generic_forward");
@@ -33,7 +33,7 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
                        wave_geometry(p, dtype, kWaveFilters, 0, &wg, &ps, &nv);
     if (!tiled) { add("%s", "generic_backward"); return n; }
     const bool rows_both = dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
-                           tune_int("DDF_TUNE_ROWSF", 1) != 0 && !small_supported(p) &&
+                           tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
                            rows_cover_backward(p, dtype);
     const bool fuse = (need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0 &&
                       wave_geometry(p, dtype, kWaveFused, 0, &wg, &ps, &nv) &&
@@ -53,7 +53,7 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
         return n;
     }
     if (need & DDF_NEED_DX) {
-        if (!small_supported(p) && dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
+        if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
             rows_geometry(p, dtype, 0, &rg, &vx, &r))
             add("k_rows<dX,VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
         else if (small_supported(p)) add("%s", "k_small<dX>");

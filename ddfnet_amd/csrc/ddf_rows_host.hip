@@ -40,7 +40,7 @@ void lay_out_lanes(RowsGeom *t, int H, int W, int vx, int R) {
 // Instantiated (elements per lane and row, rows per lane) per element size.
 bool rows_variant_built(int esz, int vx, int r) {
     if (esz == 2) return r == 1 && (vx == 8 || vx == 4 || vx == 2);
-    if (esz == 4) return (r == 1 && (vx == 4 || vx == 2)) || (r == 2 && vx == 2);
+    if (esz == 4) return (r == 1 && (vx == 4 || vx == 2 || vx == 1)) || (r == 2 && vx == 2);
     return false;
 }
 
@@ -117,6 +117,7 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
 // fused: of the variant that also writes the feature gradient.
 bool rows_filters_variant_built(int esz, int vx, int r, bool fused) {
     if (esz != 2 && esz != 4) return false;
+    if (vx == 1) return esz == 4 && r == 1;   // odd row lengths, fp32: one pixel per lane
     if (fused) return (vx == 2 && r == 2) || (vx == 4 && r == 1);
     return r == 1 && (vx == 4 || vx == 2);
 }

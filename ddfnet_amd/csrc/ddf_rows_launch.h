@@ -84,6 +84,7 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
         if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 2) return rows::launch_v<T, 2, 2>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 1 && r == 1) return rows::launch_v<T, 1, 1>(p, g, backward, x, cf, sf, out, st);
     }
     return hipErrorNotSupported;
 }
@@ -201,6 +202,13 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
                 if (vx == 8)
                     err = rows::launch_taprow_v<T, 8>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             }
+        } else if (vx == 1) {
+            if constexpr (sizeof(T) == 4) {
+                if (fused)
+                    err = rows::launch_filters_v<T, 1, 1, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
+                else
+                    err = rows::launch_filters_v<T, 1, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
+            }
         } else if (fused) {
             if (vx == 2 && r == 2)
                 err = rows::launch_filters_v<T, 2, 2, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
@@ -237,7 +245,6 @@ hipError_t rows_backward_shared_features(const Problem &p, int x_mod, const T *g
         // every vector access 16-byte aligned, so no launch below can turn the call down
         if ((((uintptr_t)go | (uintptr_t)x | (uintptr_t)sf | (uintptr_t)dx | (uintptr_t)dsf) & 15u) != 0)
             return hipErrorNotSupported;
-        if (small_supported(p)) return hipErrorNotSupported;
         if (want_dx && fneed && rows_filters_geometry(p, dtype, true, &g, &vx, &r))
             return rows_filters_launch<T>(p, go, x, cf, sf, dx, dcf, dsf, ws, fneed, st, x_mod);
         if (want_dx && !rows_geometry(p, dtype, 0, &g, &vx, &r)) return hipErrorNotSupported;

@@ -153,13 +153,14 @@ bool wave_plan(const Problem &p, int kind, std::initializer_list<const void *> p
 template <typename T>
 hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf, T *out,
                          hipStream_t st) {
-    if (small_supported(p)) return small_launch<T>(p, false, x, cf, sf, out, st);
     if constexpr (sizeof(T) != 8) {
         if (tune_int("DDF_TUNE_ROWS", 1) != 0) {
             const hipError_t err = rows_launch<T>(p, false, x, cf, sf, out, st);
             if (err != hipErrorNotSupported) return err;
         }
     }
+    // (tiny planes the row-register kernels lack a vector width for: fp16 with odd rows)
+    if (small_supported(p)) return small_launch<T>(p, false, x, cf, sf, out, st);
     WaveGeom g; int ps, nv;
     if (!wave_plan<T>(p, kWaveForward, {x, sf, out}, &g, &ps, &nv))
         return generic_forward<T>(p, x, cf, sf, out, st);   // e.g. pointers not 16-byte aligned
@@ -191,7 +192,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     bool rows_both = false;
     if constexpr (sizeof(T) != 8) {
         rows_both = tune_int("DDF_TUNE_ROWS", 1) != 0 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
-                    !small_supported(p) && rows_cover_backward(p, dtype);
+                    rows_cover_backward(p, dtype);
     }
     if ((need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0) {
         WaveGeom gp; int pps, pnv;
@@ -202,7 +203,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     if ((need & DDF_NEED_DX) && !fuse) {
         bool done = false;
         if constexpr (sizeof(T) != 8) {
-            if (!small_supported(p) && tune_int("DDF_TUNE_ROWS", 1) != 0) {
+            if (tune_int("DDF_TUNE_ROWS", 1) != 0) {
                 err = rows_launch<T>(p, true, go, cf, sf, dx, st);
                 done = err != hipErrorNotSupported;
             }

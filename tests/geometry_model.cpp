@@ -303,7 +303,7 @@ static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, 
     bool done = false;
     ROWS_CASE(1, 1, 2) ROWS_CASE(1, 1, 4) ROWS_CASE(1, 1, 8) ROWS_CASE(2, 1, 2) ROWS_CASE(2, 1, 4) ROWS_CASE(2, 1, 8)
     ROWS_CASE(1, 2, 2) ROWS_CASE(1, 2, 4) ROWS_CASE(1, 2, 8) ROWS_CASE(2, 2, 2) ROWS_CASE(2, 2, 4) ROWS_CASE(2, 2, 8)
-    ROWS_CASE(1, 4, 4) ROWS_CASE(1, 4, 8)
+    ROWS_CASE(1, 4, 4) ROWS_CASE(1, 4, 8) ROWS_CASE(1, 1, 1)
 #undef ROWS_CASE
     CHECK(done, "no replay for r=%d hy=%d vx=%d", r, hy, vx);
     if (g_fails) printf("  -> %d violations\n", g_fails);
