@@ -7,13 +7,19 @@
 
 namespace ddf {
 
+namespace {
+const char *layout_name(const RowsGeom &g) {
+    return g.segs > 0 ? "segments" : g.lp > g.lpr ? "padded" : "plain";
+}
+}  // namespace
+
 // Which kernels a call would launch, in words (pointer alignment assumed).
 // Mirrors the choices of tiled_forward / tiled_backward in ddf_tiled_launch.h.
 int describe_forward(const Problem &p, int dtype, char *buf, int len) {
     RowsGeom rg; int vx, r;
     WaveGeom wg; int ps, nv;
     if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 && rows_geometry(p, dtype, 0, &rg, &vx, &r))
-        return snprintf(buf, len, "k_rows<VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
+        return snprintf(buf, len, "k_rows<VX=%d,R=%d,%s>", vx, r, layout_name(rg));
     if (small_supported(p)) return snprintf(buf, len, "k_small");
     if (wave_geometry(p, dtype, kWaveForward, 0, &wg, &ps, &nv))
         return snprintf(buf, len, "k_forward<PS=%d,NV=%d,V=%d>", ps, nv, wg.vec);
@@ -31,17 +37,17 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
     if (len > 0) buf[0] = 0;
     const bool tiled = wave_geometry(p, dtype, kWaveFeatures, 0, &wg, &ps, &nv) &&
                        wave_geometry(p, dtype, kWaveFilters, 0, &wg, &ps, &nv);
-    if (!tiled) { add("%s", "generic_backward"); return n; }
     const bool rows_both = dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
                            tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
                            rows_cover_backward(p, dtype);
-    const bool fuse = (need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0 &&
+    if (!tiled && !rows_both) { add("%s", "generic_backward"); return n; }
+    const bool fuse = tiled && (need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0 &&
                       wave_geometry(p, dtype, kWaveFused, 0, &wg, &ps, &nv) &&
                       wave_geometry(p, dtype, kWaveFilters, 0, &gp, &pps, &pnv) && gp.TH == wg.TH &&
                       gp.csplit == wg.csplit;
     if ((need & DDF_NEED_DX) && fneed && dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
         rows_filters_geometry(p, dtype, true, &rg, &vx, &r)) {
-        add("k_rows_filters<dX,VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
+        add("k_rows_filters<dX,VX=%d,R=%d,%s>", vx, r, layout_name(rg));
         if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
         if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
         return n;
@@ -55,7 +61,7 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
     if (need & DDF_NEED_DX) {
         if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
             rows_geometry(p, dtype, 0, &rg, &vx, &r))
-            add("k_rows<dX,VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
+            add("k_rows<dX,VX=%d,R=%d,%s>", vx, r, layout_name(rg));
         else if (small_supported(p)) add("%s", "k_small<dX>");
         else add("%s", "k_backward_features");
     }
@@ -63,12 +69,12 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
         if (n) add("%s", " + ");
         if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
             rows_taprow_geometry(p, dtype, &rg, &vx, &r)) {
-            add("k_rows_taprow_filters<VX=%d,%s>", vx, rg.lp > rg.lpr ? "padded" : "plain");
+            add("k_rows_taprow_filters<VX=%d,%s>", vx, layout_name(rg));
             if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
             if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
         } else if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
             rows_filters_geometry(p, dtype, false, &rg, &vx, &r)) {
-            add("k_rows_filters<VX=%d,R=%d,%s>", vx, r, rg.lp > rg.lpr ? "padded" : "plain");
+            add("k_rows_filters<VX=%d,R=%d,%s>", vx, r, layout_name(rg));
             if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
             if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
         } else {

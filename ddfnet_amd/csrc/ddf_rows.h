@@ -51,7 +51,19 @@ struct RowsGeom {
     int wpb;                  // work items (independent waves) per workgroup
     int nwork;                // N * nstrips * csplit wave-sized work items
     unsigned csplit_magic, nstrips_magic, xcd_per;
+    // Image rows longer than a wave (segs > 0): a strip is one segment of one
+    // row group; its wave holds seg_out vectors that it produces results for,
+    // between one vector of the neighbouring segment (or of nothing, at the
+    // ends of the image row) on either side, which it only reads.  rg = 1,
+    // lp = lpr = seg_out + 2, nstrips = row groups * segs.
+    int segs, seg_out;
+    unsigned segs_magic;
 };
+
+// The vectors shifted in from the neighbouring lanes are right as they arrive
+// (an idle lane or a neighbouring segment's vector sits next to every row end):
+// the kernels' PAD variants.
+inline bool rows_shift_in_as_is(const RowsGeom &g) { return g.lp > g.lpr || g.segs > 0; }
 
 namespace rows {
 
@@ -109,6 +121,25 @@ struct Lane {
     int ooff[R];
     // dy: the window rows (xoff) are taken dy image rows further down
     __host__ __device__ __forceinline__ void init(const RowsGeom &g, int strip, int lane, int dy = 0) {
+        if (g.segs > 0) {
+            // one segment of one row group: lane 0 and lane seg_out + 1 read the
+            // neighbouring segments' edge vectors and produce nothing themselves
+            const int grp = magic_div(strip, g.segs_magic);
+            const int seg = strip - grp * g.segs;
+            const int x0 = (seg * g.seg_out + lane - 1) * VX;
+            const int y0 = grp * R;
+            const bool reads = lane <= g.seg_out + 1 && x0 >= 0 && x0 < g.W;
+            const bool owns = reads && lane >= 1 && lane <= g.seg_out;
+            first = last = false;   // (the shifted-in vectors are right as they are)
+#pragma unroll
+            for (int rr = 0; rr < ROWS; ++rr) {
+                const int yy = y0 - HY + rr + dy;
+                xoff[rr] = (reads && yy >= 0 && yy < g.H) ? yy * g.W + x0 : -1;
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r) ooff[r] = (owns && y0 + r < g.H) ? (y0 + r) * g.W + x0 : -1;
+            return;
+        }
         const int grp = magic_div(lane, g.lp_magic);
         const int v = lane - grp * g.lp;
         const bool live = grp < g.rg && v < g.lpr;

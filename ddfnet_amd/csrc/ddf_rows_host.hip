@@ -12,6 +12,7 @@ int tune_int(const char *name, int fallback);
 namespace {
 
 constexpr int kRowsStages = 3;   // channels in flight per wave of k_rows (rows::kStages)
+constexpr int kMaxRowLanes = 32;  // lanes per image row before the row is cut into segments
 
 unsigned magic_of(int d) { return d == 1 ? 0u : (unsigned)((0x100000000ull + d - 1) / d); }
 
@@ -20,6 +21,22 @@ unsigned magic_of(int d) { return d == 1 ? 0u : (unsigned)((0x100000000ull + d -
 // row is followed by an idle lane (lane pitch lpr + 1): its loads return zero,
 // which is exactly what the neighbour shift must bring in at the row ends.
 void lay_out_lanes(RowsGeom *t, int H, int W, int vx, int R) {
+    t->segs = t->seg_out = 0;
+    t->segs_magic = 0;
+    if (W / vx > kMaxRowLanes) {
+        // an image row is longer than the lanes of a wave take: even segments of at
+        // most 62 vectors, each with a vector of its neighbours on either side
+        const int vectors = W / vx;
+        t->segs = (vectors + kWave - 3) / (kWave - 2);
+        t->seg_out = (vectors + t->segs - 1) / t->segs;
+        t->segs_magic = magic_of(t->segs);
+        t->lpr = t->lp = t->seg_out + 2;
+        t->lp_magic = magic_of(t->lp);
+        t->rg = 1;
+        t->rps = R;
+        t->nstrips = ((H + R - 1) / R) * t->segs;
+        return;
+    }
     t->lpr = W / vx;
     const int row_units = (H + R - 1) / R;                  // lane-sized row groups of the plane
     const int fit_plain = std::min(kWave / t->lpr, row_units);
@@ -60,7 +77,6 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
         if (max_vx > 0 && cand > max_vx) continue;
         if (cand > tune_int("DDF_TUNE_ROWS_VX", 16)) continue;
         if (W % cand != 0 || cand < hx) continue;
-        if (W / cand > tune_int("DDF_TUNE_ROWS_LPR", 32)) continue;
         vx = cand;
         break;
     }
@@ -140,7 +156,6 @@ bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g,
     for (int cand = std::min(16 / esz, 4); cand * esz >= 4; cand /= 2) {
         if (cand > tune_int("DDF_TUNE_ROWSF_VX", 16)) continue;
         if (W % cand != 0 || cand < hx) continue;
-        if (W / cand > 32) continue;
         // two rows per lane where a row is a few 2-pixel vectors (14 x 14: one strip per plane)
         const int r = (fused && cand == 2 && H % 2 == 0) ? 2 : 1;
         if (!rows_filters_variant_built(esz, cand, r, fused)) continue;
@@ -209,7 +224,6 @@ bool rows_taprow_geometry(const Problem &p, int dtype, RowsGeom *g, int *vx_out,
     for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
         if (cand > tune_int("DDF_TUNE_TAPROW_VX", 16)) continue;
         if (W % cand != 0 || cand < hx || cand < 2) continue;
-        if (W / cand > 32) continue;
         RowsGeom c{};
         c.C = C; c.H = H; c.W = W;
         lay_out_lanes(&c, H, W, cand, 1);

@@ -21,7 +21,7 @@ template <typename T, int K, int D, int VX, int R>
 hipError_t launch_kdv(const Problem &p, const RowsGeom &g, bool backward, const T *x, const T *cf,
                       const T *sf, T *out, hipStream_t st) {
     const dim3 grid(g.xcd_per * kXcd), block(kWave * g.wpb);
-    const bool pad = g.lp > g.lpr;
+    const bool pad = rows_shift_in_as_is(g);
 #define DDF_ROWS_CASE(MUL_, BWD_)                                                               \
     do {                                                                                        \
         if (pad)                                                                                \
@@ -105,7 +105,7 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kFilterWaves);
     const int lds = filters_lds_bytes<9>((int)sizeof(A), R, VX);
     if (p.k != 3 || p.d != 1) return hipErrorNotSupported;
-    const bool pad = g.lp > g.lpr;
+    const bool pad = rows_shift_in_as_is(g);
 #define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
     hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, R, PAD_, DX, kFilterStages,            \
                                        MUL_ ? WPE_MUL : WPE_ADD>),                               \
@@ -130,7 +130,7 @@ hipError_t launch_taprow_kdv(const Problem &p, const RowsGeom &g, const T *go, c
     constexpr int kTaprowStages = 8, kWpe = 3;   // channels in flight per wave; waves per SIMD
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kTaprowWaves);
     const int lds = taprow_lds_bytes<K>((int)sizeof(A));
-    const bool pad = g.lp > g.lpr;
+    const bool pad = rows_shift_in_as_is(g);
 #define DDF_TAPROW_CASE(MUL_, PAD_)                                                              \
     hipLaunchKernelGGL((k_rows_taprow_filters<T, K, D, MUL_, VX, 1, PAD_, kTaprowStages, kWpe>), \
                        grid, block, lds, st, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod)

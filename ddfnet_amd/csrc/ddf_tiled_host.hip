@@ -245,15 +245,20 @@ bool wave_geometry(const Problem &p, int dtype, int kind, int max_vec, WaveGeom 
     return true;
 }
 
+// (either family covers the problem; what one of them lacks at run time - a
+// shape, an alignment - the launch code takes to the other or to the generic kernels)
 bool tiled_forward_supported(const Problem &p, int dtype) {
     WaveGeom g; int ps, nv;
-    return wave_geometry(p, dtype, kWaveForward, 0, &g, &ps, &nv);
+    RowsGeom rg; int vx, r;
+    return wave_geometry(p, dtype, kWaveForward, 0, &g, &ps, &nv) ||
+           (dtype != DDF_F64 && rows_geometry(p, dtype, 0, &rg, &vx, &r));
 }
 
 bool tiled_backward_supported(const Problem &p, int dtype) {
     WaveGeom w; int ps, nv;
-    return wave_geometry(p, dtype, kWaveFeatures, 0, &w, &ps, &nv) &&
-           wave_geometry(p, dtype, kWaveFilters, 0, &w, &ps, &nv);
+    return (wave_geometry(p, dtype, kWaveFeatures, 0, &w, &ps, &nv) &&
+            wave_geometry(p, dtype, kWaveFilters, 0, &w, &ps, &nv)) ||
+           (dtype != DDF_F64 && rows_cover_backward(p, dtype));
 }
 
 // Workspace layout: [dSF partials over channel splits][dCF partials over strips],

@@ -195,26 +195,42 @@ static void replay_rows(const RowsGeom &g, long N, long C, int kind, int taps = 
     std::vector<int> owner(plane, 0);
     CHECK(g.lp == g.lpr || g.lp == g.lpr + 1, "lane pitch %d for %d lanes per row", g.lp, g.lpr);
     CHECK((long)(g.rg - 1) * g.lp + g.lpr <= 64, "row groups do not fit the wavefront");
-    CHECK(g.lpr * VX == g.W, "lanes per row");
+    if (g.segs > 0)
+        CHECK(g.seg_out >= 1 && g.seg_out <= 62 && g.lp == g.seg_out + 2 && g.rg == 1 &&
+              (long)g.segs * g.seg_out * VX >= g.W && (long)(g.segs - 1) * g.seg_out * VX < g.W &&
+              g.nstrips == ((g.H + R - 1) / R) * g.segs, "segments of an image row");
+    else
+        CHECK(g.lpr * VX == g.W, "lanes per row");
     for (int strip = 0; strip < g.nstrips; ++strip)
         for (int lane = 0; lane < 64; ++lane) {
             rows::Lane<R, HY, VX> ln;
             ln.init(g, strip, lane);
             const int grp = lane / g.lp, v = lane % g.lp;
+            // first row of the lane and its vector's first column
+            const int row0 = g.segs > 0 ? (strip / g.segs) * R : strip * g.rps + grp * R;
+            const int col0 = g.segs > 0 ? ((strip % g.segs) * g.seg_out + lane - 1) * VX : v * VX;
             for (int rr = 0; rr < R + 2 * HY; ++rr) {
                 const int off = ln.xoff[rr];
                 if (off < 0) continue;
                 CHECK(grp < g.rg && v < g.lpr, "idle lane %d with a live offset", lane);
                 CHECK(off % VX == 0 && off + VX <= plane, "offset %d outside the plane or misaligned", off);
-                const int yy = strip * g.rps + grp * R - HY + rr;
-                CHECK(off == yy * g.W + v * VX, "offset %d is not row %d vector %d", off, yy, v);
+                const int yy = row0 - HY + rr;
+                CHECK(col0 >= 0 && col0 + VX <= g.W && off == yy * g.W + col0,
+                      "offset %d is not row %d column %d", off, yy, col0);
+            }
+            if (g.segs > 0) {
+                // a lane that produces results has both neighbours' vectors in the wave
+                // (or sits at an end of the image row)
+                for (int r = 0; r < R; ++r)
+                    if (ln.ooff[r] >= 0) CHECK(lane >= 1 && lane <= g.seg_out, "result in a halo lane %d", lane);
             }
             for (int r = 0; r < R; ++r)
                 if (ln.ooff[r] >= 0)
                     for (int e = 0; e < VX; ++e) ++owner[ln.ooff[r] + e];
             if (g.lp > g.lpr && v == g.lpr)
                 for (int rr = 0; rr < R + 2 * HY; ++rr) CHECK(ln.xoff[rr] < 0, "padding lane %d is live", lane);
-            CHECK(ln.first == (v == 0) && ln.last == (v == g.lpr - 1), "row ends");
+            if (g.segs > 0) CHECK(!ln.first && !ln.last, "row ends");
+            else CHECK(ln.first == (v == 0) && ln.last == (v == g.lpr - 1), "row ends");
             for (int i = 0; i < taps; ++i) {
                 // the shifted window of wave i: same result rows, feature rows dy further down
                 const int dy = (i - taps / 2) * dil;
@@ -224,9 +240,9 @@ static void replay_rows(const RowsGeom &g, long N, long C, int kind, int taps = 
                 for (int rr = 0; rr < R + 2 * HY; ++rr) {
                     const int off = sh.xoff[rr];
                     if (off < 0) continue;
-                    const int yy = strip * g.rps + grp * R - HY + rr + dy;
-                    CHECK(grp < g.rg && v < g.lpr && yy >= 0 && yy < g.H && off == yy * g.W + v * VX,
-                          "shifted offset %d is not row %d vector %d", off, yy, v);
+                    const int yy = row0 - HY + rr + dy;
+                    CHECK(grp < g.rg && v < g.lpr && yy >= 0 && yy < g.H && off == yy * g.W + col0,
+                          "shifted offset %d is not row %d column %d", off, yy, col0);
                 }
             }
         }
@@ -353,6 +369,7 @@ int main() {
         check_rows(N, C, H, W / 2 * 2 + 2, 3, next(1, 2), next(0, 1), next(0, 1) != 0);
         check_rows(N, C, H, (W / 8 + 1) * 8, 3, next(1, 2), next(0, 1), next(0, 1) != 0);
         check_rows(N, C, H, (W / 8 + 1) * 8, 5, next(1, 2), next(0, 1), false);
+        check_rows(N, C, H, (W / 8 + 1) * 8 * next(1, 6), 3, next(1, 2), next(0, 1), next(0, 1) != 0);
         check_rows(N, C, H, (W / 4 + 1) * 4, 5, next(1, 2), next(0, 1), true, false, true);
     }
     return 0;

@@ -217,14 +217,24 @@ def test_up_backward_validation_and_workspace_need_no_gpu():
     assert bwd(None, None, none, none, None, none, none, None, 0, *args, 2, 0, 1, 0, None) == 0
     assert bwd(None, None, none, none, None, none, none, None, 0, *args, 2, 0, 1, 7, None) == 1
     assert b'null' in lib.ddf_hip_last_error()
-    # lattices and per-branch dX of 4 branches, each padded to 256 bytes, plus
-    # the workspace of one 3x3 stride-1 branch (none at this size)
+    # Lattices and per-branch dX of 4 branches, each padded to 256 bytes; then
+    # either the workspace of one 3x3 stride-1 branch (none at this size), or, for
+    # all branches as one batch of 8 samples: the filters and the filter gradients
+    # of the 4 branches back to back plus that batch's own workspace.
     n_x = 2 * 8 * 6 * 6 * 4
     pad = lambda v: (v + 255) // 256 * 256
     branch = lib.ddf_hip_backward_workspace_bytes(2, 8, 6, 6, 3, 1, 1, 0, 1, 7, 0)
-    assert size(2, 8, 6, 6, 3, 1, 2, 0, 1, 7) == 2 * pad(4 * n_x) + pad(branch)
-    assert size(2, 8, 6, 6, 3, 1, 2, 0, 1, 6) == pad(4 * n_x) + pad(
-        lib.ddf_hip_backward_workspace_bytes(2, 8, 6, 6, 3, 1, 1, 0, 1, 6, 0))
+    batch = lib.ddf_hip_backward_workspace_bytes(8, 8, 6, 6, 3, 1, 1, 0, 1, 7, 0)
+    n_cf, n_sf = 2 * 8 * 9 * 4, 2 * 9 * 6 * 6 * 4
+    staged = 2 * (pad(4 * n_cf) + pad(4 * n_sf))
+    assert size(2, 8, 6, 6, 3, 1, 2, 0, 1, 7) == 2 * pad(4 * n_x) + max(pad(branch), staged + pad(batch))
+    # fp64 has no batched route
+    assert size(2, 8, 6, 6, 3, 1, 2, 0, 2, 7) == 2 * pad(8 * n_x) + pad(
+        lib.ddf_hip_backward_workspace_bytes(2, 8, 6, 6, 3, 1, 1, 0, 2, 7, 0))
+    # filter gradients only: no dX parts
+    assert size(2, 8, 6, 6, 3, 1, 2, 0, 1, 6) == pad(4 * n_x) + max(
+        pad(lib.ddf_hip_backward_workspace_bytes(2, 8, 6, 6, 3, 1, 1, 0, 1, 6, 0)),
+        staged + pad(lib.ddf_hip_backward_workspace_bytes(8, 8, 6, 6, 3, 1, 1, 0, 1, 6, 0)))
     assert size(2, 8, 6, 6, 3, 1, 1, 0, 1, 7) == 0
 
 
