@@ -56,8 +56,8 @@ void lay_out_lanes(RowsGeom *t, int H, int W, int vx, int R) {
 
 // Instantiated (elements per lane and row, rows per lane) per element size.
 bool rows_variant_built(int esz, int vx, int r) {
-    if (esz == 2) return r == 1 && (vx == 8 || vx == 4 || vx == 2);
-    if (esz == 4) return (r == 1 && (vx == 4 || vx == 2 || vx == 1)) || (r == 2 && vx == 2);
+    if (esz == 2) return (r == 1 && (vx == 8 || vx == 4 || vx == 2)) || (r == 2 && vx == 8);
+    if (esz == 4) return (r == 1 && (vx == 4 || vx == 2 || vx == 1)) || (r == 2 && (vx == 2 || vx == 4));
     return false;
 }
 
@@ -86,6 +86,10 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     // not a multiple of four pixels (14 x 14) take two rows per lane: the plane
     // is then one strip, and the shorter prologue matters more there.
     int R = (esz == 4 && vx == 2 && H % 2 == 0 && H * W <= 1024) ? 2 : 1;
+    // Large planes stream from HBM and a lane's halo rows come in through the
+    // L1 once more per row group: two rows per lane of full 16-byte vectors read
+    // four rows for two instead of three for one (built for 3x3 without dilation).
+    if (vx * esz == 16 && p.k == 3 && p.d == 1 && H * W >= 112 * 112) R = 2;
     R = tune_int("DDF_TUNE_ROWS_R", R);
     if (p.k == 5) {   // 25 taps: built for one row per lane and vectors of four pixels or more
         R = 1;

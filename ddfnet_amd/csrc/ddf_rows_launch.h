@@ -48,7 +48,7 @@ template <typename T, int VX, int R>
 hipError_t launch_v(const Problem &p, const RowsGeom &g, bool backward, const T *x, const T *cf,
                     const T *sf, T *out, hipStream_t st) {
     if (p.k == 3 && p.d == 1) return launch_kdv<T, 3, 1, VX, R>(p, g, backward, x, cf, sf, out, st);
-    if constexpr (VX >= 2) {
+    if constexpr (VX >= 2 && VX * (int)sizeof(T) * R < 32) {   // (16-byte vectors, two rows: 3x3 d1 only)
         if (p.k == 3 && p.d == 2)
             return launch_kdv<T, 3, 2, VX, R>(p, g, backward, x, cf, sf, out, st);
     }
@@ -80,7 +80,9 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
         if (vx == 8 && r == 1) return rows::launch_v<T, 8, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 8 && r == 2) return rows::launch_v<T, 8, 2>(p, g, backward, x, cf, sf, out, st);
     } else if constexpr (sizeof(T) == 4) {
+        if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 2) return rows::launch_v<T, 2, 2>(p, g, backward, x, cf, sf, out, st);

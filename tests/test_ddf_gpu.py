@@ -123,7 +123,21 @@ EDGE = [
     (2, 8, 33, 224, 3, 1, 2),   # wide, strided, odd height
     (1, 2, 5, 513, 5, 1, 1),    # wider than the tuned kernels' 8 x 64 columns
     (1, 3, 130, 6, 3, 2, 1),    # tall and narrow
+    (1, 3, 113, 128, 3, 1, 1),  # large plane: two rows per lane, odd height
+    (1, 2, 60, 264, 3, 1, 1),   # large plane, rows of two segments, two rows per lane
+    (1, 2, 48, 264, 5, 2, 1),   # 5x5 dilated on segmented rows
+    (2, 2, 9, 1000, 3, 1, 1),   # five segments per row
 ]
+
+
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('case', [(1, 2, 50, 272, 3, 1, 1), (1, 3, 57, 520, 3, 1, 1), (2, 2, 16, 264, 5, 1, 1),
+                                  (1, 4, 31, 304, 3, 2, 1)], ids=_ids)
+def test_wide_rows_fp16(case, combine):
+    """fp16 rows of more than 32 eight-pixel vectors are cut into segments."""
+    N, C, H, W, k, d, s = case
+    tensors = random_case(N, C, H, W, k, s, torch.float16, seed=11)
+    check_against_oracle(*tensors, k, d, s, combine, '', what=str(case))
 
 
 @pytest.mark.parametrize('version', VERSIONS)
