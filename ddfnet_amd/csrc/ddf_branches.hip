@@ -17,6 +17,8 @@
 // unbiased standard deviation over the KK taps, as in ddf_filter_norm.hip.
 // Both kernels are bound by memory and launch latency, not by arithmetic: the
 // spatial branch does KK multiply-adds per 4-byte (2-byte) load.
+#include <algorithm>
+
 #include "ddf_common.h"
 
 namespace ddf {
@@ -24,99 +26,248 @@ namespace {
 
 constexpr int kChunk = 256;   // channels whose weights sit in LDS at a time (64 per wave)
 
-// Standardise v[0..KK) in place and apply gain / offset of filter group `g`.
-template <typename T, int KK, typename A>
-__device__ __forceinline__ void normalise(A (&v)[KK], int64_t g, A gain, const T *gain_vec,
-                                          const T *offset_vec) {
-    A sum = 0;
+// Gains, offsets and biases of the KK taps of filter group `g`, read once (all
+// loads go out together; read tap by tap where they are used, every one of
+// them is a round trip of its own at the end of the kernel).
+template <typename T, int KK>
+struct TapParams {
+    float gain[KK], offset[KK], bias[KK];
+    __device__ __forceinline__ void load(int64_t g, float scalar_gain, const T *gain_vec,
+                                         const T *offset_vec, const T *bias_vec) {
 #pragma unroll
-    for (int t = 0; t < KK; ++t) sum += v[t];
-    const A mean = sum / (A)KK;
-    A sq = 0;
+        for (int t = 0; t < KK; ++t) {
+            gain[t] = scalar_gain;
+            offset[t] = 0.f;
+            bias[t] = 0.f;
+        }
+        if (gain_vec) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) gain[t] = ld(gain_vec + g * KK + t);
+        }
+        if (offset_vec) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) offset[t] = ld(offset_vec + g * KK + t);
+        }
+        if (bias_vec) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t) bias[t] = ld(bias_vec + g * KK + t);
+        }
+    }
+};
+
+// v[0..KK) + bias, standardised in place, times gain plus offset.
+template <typename T, int KK>
+__device__ __forceinline__ void normalise(float (&v)[KK], const TapParams<T, KK> &p) {
+    float sum = 0;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        v[t] += p.bias[t];
+        sum += v[t];
+    }
+    const float mean = sum / (float)KK;
+    float sq = 0;
 #pragma unroll
     for (int t = 0; t < KK; ++t) {
         v[t] -= mean;
         sq += v[t] * v[t];
     }
-    const A inv = (A)1 / (sqrtf(sq / (A)(KK - 1)) + (A)1e-10);
+    const float inv = 1.f / (sqrtf(sq / (float)(KK - 1)) + 1e-10f);
 #pragma unroll
-    for (int t = 0; t < KK; ++t) {
-        const A w = gain_vec ? (A)ld(gain_vec + g * KK + t) : gain;
-        v[t] = v[t] * inv * w;
-        if (offset_vec) v[t] += (A)ld(offset_vec + g * KK + t);
+    for (int t = 0; t < KK; ++t) v[t] = v[t] * inv * p.gain[t] + p.offset[t];
+}
+
+// VP storage-type values at p (aligned to VP * sizeof(T)), widened.
+template <typename T, int VP>
+__device__ __forceinline__ void load_pixels(const T *p, float (&v)[VP]) {
+    if constexpr (VP == 1) {
+        v[0] = ld(p);
+    } else {
+        struct alignas(VP * sizeof(T)) Pack { T e[VP]; };
+        const Pack q = *reinterpret_cast<const Pack *>(p);
+#pragma unroll
+        for (int k = 0; k < VP; ++k) v[k] = ld(&q.e[k]);
     }
 }
 
-// grid (pixel tiles of 64, head, N); the WAVES waves of a workgroup cover the
-// same 64 result pixels (lane = pixel) and 1/WAVES of every channel chunk each,
-// 16 channels' loads in flight at a time.
-template <typename T, int KK, int WAVES>
+// grid (pixel tiles of 64 * VP, head, N); the WAVES waves of a workgroup cover
+// the same result pixels (a lane owns VP consecutive pixels of a row: VP > 1
+// needs stride 1 and rows that are a whole number of such vectors) and
+// 1/WAVES of every channel chunk each, U channels' loads in flight at a time.
+template <typename T, int KK, int WAVES, int VP>
 __global__ __launch_bounds__(WAVES * kWave) void k_spatial_branch(
     const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias,
-    T *__restrict__ sf, int C, int H, int W, int Ho, int Wo, int stride, float gain,
+    T *__restrict__ sf, int C, int H, int W, int Ho, int Wo, int stride, int chunk, float gain,
     const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
-    constexpr int PER = kChunk / WAVES;                 // channels of a chunk per wave
-    constexpr int U = 16;
-    static_assert(PER % U == 0, "whole batches");
-    __shared__ float wt[kChunk][KK];                    // weights of the chunk, [channel][tap]
-    __shared__ float red[WAVES][KK][kWave];             // per-wave sums, [wave][tap][pixel]
+    constexpr int U = VP >= 4 ? 4 : 8;
+    // weights of the chunk, [channel][tap], rows padded to 16 bytes (wide LDS reads)
+    __shared__ __align__(16) float wt[kChunk][(KK + 3) / 4 * 4];
+    __shared__ float red[WAVES][KK][kWave];             // per-wave sums of one pixel of the vector
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int g = blockIdx.y, heads = gridDim.y;
     const int64_t n = blockIdx.z;
     const int npix = Ho * Wo;
-    const int pix = blockIdx.x * kWave + lane;
+    const int pix = (blockIdx.x * kWave + lane) * VP;   // first of the lane's pixels
     const bool live = pix < npix;
     const int yo = live ? pix / Wo : 0, xo = live ? pix - yo * Wo : 0;
     const int64_t plane = (int64_t)H * W;
     const T *xp = x + n * C * plane + (int64_t)yo * stride * W + (int64_t)xo * stride;
     const T *wg = w + (int64_t)g * KK * C;
+    const int per = chunk / WAVES;                      // channels of a chunk per wave (multiple of U)
+    TapParams<T, KK> params;
+    if (wave == 0) params.load(g, gain, gain_vec, offset_vec, bias);   // (wave 0 writes the taps)
 
-    float acc[KK];
+    float acc[KK][VP];
 #pragma unroll
-    for (int t = 0; t < KK; ++t) acc[t] = 0.f;
-    for (int c0 = 0; c0 < C; c0 += kChunk) {
+    for (int t = 0; t < KK; ++t)
+#pragma unroll
+        for (int k = 0; k < VP; ++k) acc[t][k] = 0.f;
+    for (int c0 = 0; c0 < C; c0 += chunk) {
         if (c0 > 0) __syncthreads();
-        // weights of channels c0 .. c0+255 (zero past C), coalesced along a weight row
-        for (int i = threadIdx.x; i < kChunk; i += WAVES * kWave) {
+        // weights of channels c0 .. c0+chunk-1 (zero past C), coalesced along a weight row
+        for (int i = threadIdx.x; i < chunk; i += WAVES * kWave) {
             const int c = c0 + i;
 #pragma unroll
             for (int t = 0; t < KK; ++t) wt[i][t] = c < C ? ld(wg + (int64_t)t * C + c) : 0.f;
         }
         __syncthreads();
-        const int cw = c0 + wave * PER;                 // this wave's channels of the chunk
-        const int nc = min(PER, C - cw);                // (<= 0: none left)
+        const int cw = c0 + wave * per;                 // this wave's channels of the chunk
+        const int nc = min(per, C - cw);                // (<= 0: none left)
         for (int i0 = 0; i0 < nc; i0 += U) {
-            float xv[U];
+            float xv[U][VP];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int i = min(i0 + u, nc - 1);      // past the end: repeats, with zero weights
-                xv[u] = live ? ld(xp + (int64_t)(cw + i) * plane) : 0.f;
+                if (live) {
+                    load_pixels<T, VP>(xp + (int64_t)(cw + i) * plane, xv[u]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < VP; ++k) xv[u][k] = 0.f;
+                }
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 // (rows past the wave's last channel belong to channels >= C: zeros)
-                const float *wr = wt[wave * PER + i0 + u];
+                const float *wr = wt[wave * per + i0 + u];
 #pragma unroll
-                for (int t = 0; t < KK; ++t) acc[t] = fmaf(wr[t], xv[u], acc[t]);
+                for (int t = 0; t < KK; ++t) {
+                    const float wv = wr[t];
+#pragma unroll
+                    for (int k = 0; k < VP; ++k) acc[t][k] = fmaf(wv, xv[u][k], acc[t][k]);
+                }
             }
         }
     }
+    // one pixel of the vectors at a time through LDS: the waves' sums, then wave 0
+    // normalises and writes that pixel's taps
 #pragma unroll
-    for (int t = 0; t < KK; ++t) red[wave][t][lane] = acc[t];
-    __syncthreads();
-    if (wave != 0 || !live) return;
-    float v[KK];
+    for (int k = 0; k < VP; ++k) {
+        if (k > 0) __syncthreads();
 #pragma unroll
-    for (int t = 0; t < KK; ++t) {
-        float s = bias ? ld(bias + g * KK + t) : 0.f;
+        for (int t = 0; t < KK; ++t) red[wave][t][lane] = acc[t][k];
+        __syncthreads();
+        if (wave == 0 && live) {
+            float v[KK];
 #pragma unroll
-        for (int q = 0; q < WAVES; ++q) s += red[q][t][lane];
-        v[t] = s;
+            for (int t = 0; t < KK; ++t) {
+                float s = 0.f;
+#pragma unroll
+                for (int q = 0; q < WAVES; ++q) s += red[q][t][lane];
+                v[t] = s;
+            }
+            normalise<T, KK>(v, params);
+            T *op = sf + ((n * heads + g) * KK) * (int64_t)npix + pix + k;
+#pragma unroll
+            for (int t = 0; t < KK; ++t) st(op + (int64_t)t * npix, v[t]);
+        }
     }
-    normalise<T, KK, float>(v, g, gain, gain_vec, offset_vec);
+}
+
+// The same for planes with many pixels: every wave of the workgroup has its own
+// 64 * VP result pixels and walks all channels, so nothing is added up across
+// waves and the taps are normalised in registers.  grid (tiles of 4 * 64 * VP
+// pixels, head, N).
+template <typename T, int KK, int VP>
+__global__ __launch_bounds__(4 * kWave) void k_spatial_branch_tiles(
+    const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias,
+    T *__restrict__ sf, int C, int H, int W, int Ho, int Wo, int stride, int chunk, float gain,
+    const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
+    constexpr int U = 16;   // channels in flight per wave: what the run time hangs on
+    __shared__ __align__(16) float wt[kChunk][(KK + 3) / 4 * 4];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int g = blockIdx.y, heads = gridDim.y;
+    const int64_t n = blockIdx.z;
+    const int npix = Ho * Wo;
+    const int pix = ((blockIdx.x * 4 + wave) * kWave + lane) * VP;
+    const bool live = pix < npix;
+    const int yo = live ? pix / Wo : 0, xo = live ? pix - yo * Wo : 0;
+    const int64_t plane = (int64_t)H * W;
+    const T *xp = x + n * C * plane + (int64_t)yo * stride * W + (int64_t)xo * stride;
+    const T *wg = w + (int64_t)g * KK * C;
+    TapParams<T, KK> params;
+    params.load(g, gain, gain_vec, offset_vec, bias);
+
+    float acc[KK][VP];
+#pragma unroll
+    for (int t = 0; t < KK; ++t)
+#pragma unroll
+        for (int k = 0; k < VP; ++k) acc[t][k] = 0.f;
+    for (int c0 = 0; c0 < C; c0 += chunk) {
+        if (c0 > 0) __syncthreads();
+        for (int i = threadIdx.x; i < chunk; i += 4 * kWave) {
+            const int c = c0 + i;
+#pragma unroll
+            for (int t = 0; t < KK; ++t) wt[i][t] = c < C ? ld(wg + (int64_t)t * C + c) : 0.f;
+        }
+        __syncthreads();
+        const int nc = min(chunk, C - c0);
+        for (int i0 = 0; i0 < nc; i0 += U) {
+            float xv[U][VP];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int i = min(i0 + u, nc - 1);      // past the end: repeats, with zero weights
+                if (live) {
+                    load_pixels<T, VP>(xp + (int64_t)(c0 + i) * plane, xv[u]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < VP; ++k) xv[u][k] = 0.f;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float *wr = wt[i0 + u];           // (i0 + u < chunk: chunk is a multiple of U)
+                float wv[KK];
+#pragma unroll
+                for (int t = 0; t < KK; ++t) wv[t] = wr[t];
+#pragma unroll
+                for (int t = 0; t < KK; ++t)
+#pragma unroll
+                    for (int k = 0; k < VP; ++k) acc[t][k] = fmaf(wv[t], xv[u][k], acc[t][k]);
+            }
+        }
+    }
+    if (!live) return;
+#pragma unroll
+    for (int k = 0; k < VP; ++k) {
+        float v[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) v[t] = acc[t][k];
+        normalise<T, KK>(v, params);
+#pragma unroll
+        for (int t = 0; t < KK; ++t) acc[t][k] = v[t];
+    }
+    // taps of the lane's VP pixels, one vector store per tap plane
     T *op = sf + ((n * heads + g) * KK) * (int64_t)npix + pix;
 #pragma unroll
-    for (int t = 0; t < KK; ++t) st(op + (int64_t)t * npix, v[t]);
+    for (int t = 0; t < KK; ++t) {
+        if constexpr (VP == 1) {
+            st(op + (int64_t)t * npix, acc[t][0]);
+        } else {
+            struct alignas(VP * sizeof(T)) Pack { T e[VP]; } q;
+#pragma unroll
+            for (int k = 0; k < VP; ++k) st(&q.e[k], acc[t][k]);
+            *reinterpret_cast<Pack *>(op + (int64_t)t * npix) = q;
+        }
+    }
 }
 
 // Sum over the 64 lanes (the same value in every lane): four butterfly steps
@@ -213,7 +364,9 @@ __global__ __launch_bounds__(kChannelThreads) void k_channel_branch(
     float u[KK];
 #pragma unroll
     for (int t = 0; t < KK; ++t) u[t] = f[i * KK + t];
-    normalise<T, KK, float>(u, cb + i, gain, gain_vec, offset_vec);
+    TapParams<T, KK> params;
+    params.load(cb + i, gain, gain_vec, offset_vec, (const T *)nullptr);   // (b2 is in f already)
+    normalise<T, KK>(u, params);
     T *op = cf + (n * C + cb + i) * KK;
 #pragma unroll
     for (int t = 0; t < KK; ++t) st(op + t, u[t]);
@@ -230,14 +383,43 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
     const int64_t Ho = H / stride, Wo = W / stride;
     if (N == 0 || C == 0 || Ho * Wo == 0 || head == 0) return hipSuccess;
     if (N > 65535 || head > 65535 || C > (1 << 24) || H * W >= (1ll << 31)) return hipErrorNotSupported;
+    const int waves = k == 3 ? 8 : 4;
+    // channels staged in LDS at a time: all of them up to kChunk, a multiple of 8 per wave
+    // (and so of the 16 the tile kernel keeps in flight)
+    const int chunk = (int)std::min<int64_t>(kChunk, (C + 8 * waves - 1) / (8 * waves) * (8 * waves));
+    // Planes with many pixels: a wave per pixel tile, as wide a vector per lane as
+    // rows and alignment allow while the waves still fill the machine.
+    if (stride == 1) {
+        for (int vp = 16 / (int)sizeof(T); vp >= 1; vp /= 2) {
+            if (k == 5 && vp > 2) continue;   // (25 taps: the accumulators of two pixels per lane)
+            if (W % vp != 0 || (((uintptr_t)x | (uintptr_t)sf) % (vp * sizeof(T))) != 0) continue;
+            if (vp == 1 && sizeof(T) == 2) continue;   // (2-byte loads: the shared-pixel kernel does better)
+            if ((Ho * Wo) % vp != 0 || N * head * cdiv(Ho * Wo, kWave * vp) < 1024) continue;
+            const dim3 grid((unsigned)cdiv(Ho * Wo, 4 * kWave * vp), (unsigned)head, (unsigned)N);
+#define DDF_TILES_CASE(KK_, VP_)                                                                \
+    hipLaunchKernelGGL((k_spatial_branch_tiles<T, KK_, VP_>), grid, dim3(4 * kWave), 0, st, x, w, \
+                       bias, sf, (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, chunk,       \
+                       (float)gain, gain_vec, offset_vec)
+            if (k == 3 && vp == 8) { if constexpr (sizeof(T) == 2) DDF_TILES_CASE(9, 8); }
+            else if (k == 3 && vp == 4) DDF_TILES_CASE(9, 4);
+            else if (k == 3 && vp == 2) DDF_TILES_CASE(9, 2);
+            else if (k == 3) DDF_TILES_CASE(9, 1);
+            else if (k == 5 && vp == 2) DDF_TILES_CASE(25, 2);
+            else if (k == 5) DDF_TILES_CASE(25, 1);
+            else return hipErrorNotSupported;
+#undef DDF_TILES_CASE
+            return hipGetLastError();
+        }
+    }
+    // Few pixels (or strided sampling): the waves of a workgroup share 64 pixels and
+    // split the channels (as many waves as the LDS of the per-wave sums allows).
     const dim3 grid((unsigned)cdiv(Ho * Wo, kWave), (unsigned)head, (unsigned)N);
-    // (as many waves per pixel tile as the LDS of the per-wave sums allows)
-#define DDF_SPATIAL_CASE(KK_, WAVES_)                                                           \
-    hipLaunchKernelGGL((k_spatial_branch<T, KK_, WAVES_>), grid, dim3(WAVES_ * kWave), 0, st, x, w, \
-                       bias, sf, (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, (float)gain, \
-                       gain_vec, offset_vec)
-    if (k == 3) DDF_SPATIAL_CASE(9, 8);
-    else if (k == 5) DDF_SPATIAL_CASE(25, 4);
+#define DDF_SPATIAL_CASE(KK_, WAVES_, VP_)                                                      \
+    hipLaunchKernelGGL((k_spatial_branch<T, KK_, WAVES_, VP_>), grid, dim3(WAVES_ * kWave), 0, st, x, \
+                       w, bias, sf, (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, chunk,    \
+                       (float)gain, gain_vec, offset_vec)
+    if (k == 3) DDF_SPATIAL_CASE(9, 8, 1);
+    else if (k == 5) DDF_SPATIAL_CASE(25, 4, 1);
     else return hipErrorNotSupported;
 #undef DDF_SPATIAL_CASE
     return hipGetLastError();
