@@ -258,6 +258,35 @@ def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
     return res
 
 
+def profile_phase(name, phase, steps, warmup, lib):
+    """One library call of a workload on its own, for runs under rocprofv3:
+    warmup + steps calls of `phase` over the rotating buffer sets, then a plain
+    256 MiB device copy (the yardstick the fetch / write counters are scaled by).
+    Every ddf:: dispatch of the process belongs to that call."""
+    N, C, H, W, k, d, s, combine, dtype = WORKLOADS[name]
+    host = make_inputs(N, C, H, W, k, s, dtype)
+    first = Workset(host)
+    nsets = max(2, LLC_BYTES * 2 // first.nbytes() + 1)
+    sets = [first] + [Workset(host) for _ in range(nsets - 1)]
+    ws_bytes = lib.backward_workspace_bytes((N, C, H, W), k, d, s, combine, dtype, 7)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda') if ws_bytes else None
+    run = Launcher(lib, sets, (N, C, H, W), k, d, s, combine, dtype, ws)
+    for i in range(warmup):
+        run.phase(phase, i)
+    ms = timed(lambda i: run.phase(phase, i), steps)
+    a = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device='cuda')
+    b = torch.empty_like(a)
+    for _ in range(4):
+        b.copy_(a)
+    torch.cuda.synchronize()
+    esz = torch.empty(0, dtype=dtype).element_size()
+    need_of = {'fwd': 0, 'bwd': 7, 'dx': 1, 'dfilters': 6}
+    return {'workload': name, 'phase': phase, 'calls': warmup + steps, 'us_per_call': round(ms * 1e3, 2),
+            'kernels': lib.describe((N, C, H, W), k, d, s, combine, dtype, need_of[phase]),
+            'algorithmic_bytes': algorithmic_bytes(N, C, H, W, k, s, esz)[phase],
+            'copy_probe_bytes': 4 * a.numel() * 4}
+
+
 def cpu_baseline(name, budget_s=12.0):
     """The CPU oracle (a port of the reference's formulation; the reference has
     no CPU path of its own) timed on this host: fp32, forward + backward, on a
@@ -446,6 +475,10 @@ def main():
     ap.add_argument('--up-pack', action='store_true',
                     help='also time the fused up-sampling forward against its composition')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--profile-phase', choices=PHASES, default=None,
+                    help='run only this library call of the workload (warm-up + steps calls, then the '
+                         'copy probe) and print what was run: the unit the profiles/ summaries are '
+                         'collected on')
     ap.add_argument('--copy-probe', action='store_true',
                     help='also run a plain 256 MiB device copy (calibrates hardware counters)')
     args = ap.parse_args()
@@ -458,6 +491,9 @@ def main():
     from ddfnet_amd import _lib as lib
     lib.lib()
 
+    if args.profile_phase:
+        print(json.dumps(profile_phase(args.workload, args.profile_phase, args.steps, args.warmup, lib)))
+        return
     res = run_workload(args.workload, args.steps, args.warmup, lib, copy_probe=args.copy_probe)
     extra = {}
     if not args.only_headline:
