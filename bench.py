@@ -326,7 +326,7 @@ def model_inference(batch=128, steps=10, warmup=3):
     """ddf_mul_resnet50 inference, fp16, random weights, synthetic input."""
     from ddfnet_amd import ddf_resnet
     torch.manual_seed(0)
-    model = ddf_resnet.ddf_mul_resnet50().cuda().half().eval()
+    model = ddf_resnet.ddf_mul_resnet50(zero_init_last_bn=False).cuda().half().eval()
     x = torch.randn(batch, 3, 224, 224, device='cuda', dtype=torch.float16)
     with torch.no_grad():
         for _ in range(warmup):

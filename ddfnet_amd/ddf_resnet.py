@@ -10,9 +10,11 @@ classifier.  Parameter counts match the reference's model table
 (``README.md:20-23``): 16 843 748 for ddf_mul_resnet50, 28 146 912 for
 ddf_mul_resnet101.
 
-Initialisation follows timm 0.4.5's ResNet: Kaiming-normal (fan-out, ReLU) for
-every convolution, BatchNorm at weight 1 / bias 0.  It cannot be checked against
-timm here; only the structure is pinned.
+Initialisation follows timm 0.4.5's ResNet as recalled: Kaiming-normal (fan-out,
+ReLU) for convolutions, BatchNorm weight 1 and bias 0, and - with
+``zero_init_last_bn`` (default on, as there) - weight 0 for the last BatchNorm
+of every bottleneck.  There is no way to check against timm here; only the
+structure is pinned.
 """
 import torch
 import torch.nn as nn
@@ -54,7 +56,12 @@ class DDFBottleneck(nn.Module):
 
 
 class DDFResNet(nn.Module):
-    def __init__(self, layers, kernel_combine='mul', num_classes=1000, in_chans=3, se_ratio=0.2):
+    def __init__(self, layers, kernel_combine='mul', num_classes=1000, in_chans=3, se_ratio=0.2,
+                 zero_init_last_bn=True):
+        """``zero_init_last_bn``: start every residual branch at zero by zeroing the
+        weight of each block's last BatchNorm (the default of the ResNet the
+        reference derives its models from), so a freshly built network is the
+        identity on its shortcuts."""
         super(DDFResNet, self).__init__()
         self.num_classes = num_classes
         self.conv1 = nn.Conv2d(in_chans, 64, kernel_size=7, stride=2, padding=3, bias=False)
@@ -86,6 +93,10 @@ class DDFResNet(nn.Module):
             elif isinstance(m, nn.BatchNorm2d):
                 nn.init.ones_(m.weight)
                 nn.init.zeros_(m.bias)
+        if zero_init_last_bn:
+            for m in self.modules():
+                if isinstance(m, DDFBottleneck):
+                    nn.init.zeros_(m.bn3.weight)
 
     def forward_features(self, x):
         x = self.maxpool(self.act1(self.bn1(self.conv1(x))))

@@ -183,7 +183,7 @@ def test_resnet50_forward_matches_cpu_reference(monkeypatch):
     at four plane sizes and both strides, fp32 against the CPU fp64 model."""
     from ddfnet_amd import ddf_resnet
     torch.manual_seed(3)
-    model = ddf_resnet.ddf_mul_resnet50(num_classes=10).cuda().eval()
+    model = ddf_resnet.ddf_mul_resnet50(num_classes=10, zero_init_last_bn=False).cuda().eval()
     x = torch.randn(2, 3, 64, 64, device='cuda')
     with torch.no_grad():
         out = model(x)
@@ -203,7 +203,7 @@ def test_resnet50_fp16_forward_matches_cpu_reference(monkeypatch):
     the DDF layers are held to 1e-2 each at operator level."""
     from ddfnet_amd import ddf_resnet
     torch.manual_seed(5)
-    model = ddf_resnet.ddf_mul_resnet50(num_classes=10).cuda().half().eval()
+    model = ddf_resnet.ddf_mul_resnet50(num_classes=10, zero_init_last_bn=False).cuda().half().eval()
     x = torch.randn(2, 3, 64, 64, device='cuda').half()
     with torch.no_grad():
         out = model(x)
@@ -219,7 +219,7 @@ def test_resnet50_fp16_forward_matches_cpu_reference(monkeypatch):
 def test_resnet50_fp16_inference_and_layer_timing():
     from ddfnet_amd import ddf_resnet
     torch.manual_seed(4)
-    model = ddf_resnet.ddf_mul_resnet50().cuda().half().eval()
+    model = ddf_resnet.ddf_mul_resnet50(zero_init_last_bn=False).cuda().half().eval()
     x = torch.randn(4, 3, 224, 224, device='cuda', dtype=torch.float16)
     with torch.no_grad():
         out = model(x)
