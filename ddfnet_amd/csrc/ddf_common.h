@@ -131,8 +131,8 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
                        T *out, hipStream_t st);
 
 // Filter gradients (dCF, dSF) on the row-register kernel; same conventions.
-// With dx != nullptr the launch also writes the feature gradient (small planes:
-// the whole backward pass in one kernel).  The workspace
+// With dx != nullptr the launch also writes the feature gradient (the whole
+// backward pass in one kernel, 3x3 without dilation).  The workspace
 // (rows_filters_workspace bytes, 256-byte aligned) holds the partial sums over
 // channel splits and strips.
 size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);

@@ -236,11 +236,17 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             for (int k = 0; k < NW; ++k) row[rr].own[k] = xw[ST][rr][k];
             row[rr].sides(ln.first, ln.last);
         }
+        // dO at the lane's own pixels.  (DX loads dO through the window offsets, so a
+        // lane that only reads for its neighbours - the outer lanes of a row segment -
+        // holds real values here: they must not enter the filter sums twice.)
         A gval[R][VX];
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int e = 0; e < VX; ++e) gval[r][e] = elem<T>(gw[ST][GOWN + r], e);
+            for (int e = 0; e < VX; ++e) {
+                const A v = elem<T>(gw[ST][GOWN + r], e);
+                gval[r][e] = (DX && ob[r] == kOutside) ? A(0) : v;
+            }
         A w[KK];
         if constexpr (kFilters) {
             if constexpr (kScalarTaps) {
@@ -413,8 +419,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 // Host-side geometry of k_rows_filters (ddf_rows_host.hip): a work item is a
 // workgroup of rows::kFilterWaves waves (g->wpb = 1) that covers g->cpb =
 // g->cpw * rows::kFilterWaves channels; g->csplit counts those ranges.
-// fused: the geometry of the launch that also writes the feature gradient
-// (covers small planes only).
+// fused: the geometry of the launch that also writes the feature gradient.
 bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g, int *vx, int *r);
 // Workspace the kernel needs (layout as the tile kernels': dSF partials over
 // channel splits, then dCF partials over strips, each 256-byte aligned).

@@ -117,7 +117,9 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     t.cpw = std::max(1, std::min(cpw, C));
     t.cpb = t.cpw;
     t.csplit = (C + t.cpw - 1) / t.cpw;
-    t.wpb = std::max(1, std::min(tune_int("DDF_TUNE_ROWS_WPB", 2), rows::kMaxWpb));
+    // (single-wave workgroups spread over the machine faster: what counts for the
+    // smallest launches)
+    t.wpb = std::max(1, std::min(tune_int("DDF_TUNE_ROWS_WPB", H * W <= 256 ? 1 : 2), rows::kMaxWpb));
     const int64_t nwork = base * t.csplit;
     if (nwork > (1 << 30)) return false;
     // magic-number division of the work id is exact while id * divisor < 2^32
@@ -151,9 +153,9 @@ bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g,
     const int H = (int)p.H, W = (int)p.W, C = (int)p.C;
     const int hx = p.r * p.d;
     if ((int64_t)H * W * 8 >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
-    // One launch for the whole backward pass pays where the plane is small: the
-    // launches are then bound by ramp and latency, not by bytes or arithmetic.
-    if (fused && (H * W > tune_int("DDF_TUNE_ROWSF_FUSED_PLANE", 400) ||
+    // One launch for the whole backward pass: dO, CF and SF are read once.  It is
+    // the faster route at every plane size measured (7 x 7 to 200 x 300).
+    if (fused && (H * W > tune_int("DDF_TUNE_ROWSF_FUSED_PLANE", 1 << 30) ||
                   tune_int("DDF_TUNE_ROWSF_FUSED", 1) == 0))
         return false;
     int vx = 0, R = 1;

@@ -166,8 +166,8 @@ hipError_t launch_taprow_v(const Problem &p, const RowsGeom &g, const T *go, con
 }  // namespace rows
 
 // Filter gradients on the row-register kernel, partial sums included; with
-// dx != nullptr the same launch also writes the feature gradient (small planes
-// only: rows_filters_geometry(..., fused = true) must cover the problem).
+// dx != nullptr the same launch also writes the feature gradient
+// (rows_filters_geometry(..., fused = true) must cover the problem).
 // hipErrorNotSupported: not covered (nothing was launched).  `ws` must hold
 // rows_filters_workspace() bytes.
 template <typename T>

@@ -178,7 +178,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     // One launch for all gradients where the fused kernel exists and cuts the
     // problem exactly as the workspace was sized for.
     if constexpr (sizeof(T) != 8) {
-        // small planes: the row-register kernel does the whole backward pass in one launch
+        // the row-register kernel does the whole backward pass in one launch where it covers it
         if ((need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_ROWSF", 1) != 0) {
             err = rows_filters_launch<T>(p, go, x, cf, sf, dx, dcf, dsf, ws, fneed, st);
             if (err != hipErrorNotSupported) return err;
