@@ -114,10 +114,13 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
         const uint32_t bytes = ci < nch ? plane_bytes : 0u;
         const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * plane, bytes);
         const __amdgpu_buffer_rsrc_t gr = plane_rsrc(gs + (int64_t)ci * plane, bytes);
+        // (with dilation the window has rows no tap lands on: see row_needed)
 #pragma unroll
-        for (int rr = 0; rr < ROWS; ++rr) load_words<NW>(pr, xb[rr], xw[ST][rr]);
+        for (int rr = 0; rr < ROWS; ++rr)
+            if (row_needed<R, K, D>(rr)) load_words<NW>(pr, xb[rr], xw[ST][rr]);
 #pragma unroll
-        for (int r = 0; r < GROWS; ++r) load_words<NW>(gr, DX ? xb[r] : ob[r], gw[ST][r]);
+        for (int r = 0; r < GROWS; ++r)
+            if (!DX || row_needed<R, K, D>(r)) load_words<NW>(gr, DX ? xb[r] : ob[r], gw[ST][r]);
         if constexpr (kFilters) {
             const int cc = ci < nch ? ci : (nch > 0 ? nch - 1 : 0);
             if constexpr (kScalarTaps) {
@@ -232,6 +235,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
         Row row[ROWS];
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr) {
+            if (!row_needed<R, K, D>(rr)) continue;
 #pragma unroll
             for (int k = 0; k < NW; ++k) row[rr].own[k] = xw[ST][rr][k];
             row[rr].sides(ln.first, ln.last);
@@ -292,6 +296,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             Row grow[ROWS];
 #pragma unroll
             for (int rr = 0; rr < ROWS; ++rr) {
+                if (!row_needed<R, K, D>(rr)) continue;
 #pragma unroll
                 for (int k = 0; k < NW; ++k) grow[rr].own[k] = gw[ST][rr][k];
                 grow[rr].sides(ln.first, ln.last);

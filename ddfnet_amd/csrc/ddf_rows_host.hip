@@ -146,7 +146,7 @@ bool rows_filters_variant_built(int esz, int vx, int r, bool fused) {
 
 bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g, int *vx_out,
                            int *r_out) {
-    if (!(p.s == 1 && p.k == 3 && p.d == 1)) return false;
+    if (!(p.s == 1 && p.k == 3 && (p.d == 1 || p.d == 2))) return false;
     if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
     if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
     const int esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
@@ -163,7 +163,7 @@ bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g,
         if (cand > tune_int("DDF_TUNE_ROWSF_VX", 16)) continue;
         if (W % cand != 0 || cand < hx) continue;
         // two rows per lane where a row is a few 2-pixel vectors (14 x 14: one strip per plane)
-        const int r = (fused && cand == 2 && H % 2 == 0) ? 2 : 1;
+        const int r = (fused && cand == 2 && H % 2 == 0 && p.d == 1) ? 2 : 1;
         if (!rows_filters_variant_built(esz, cand, r, fused)) continue;
         vx = cand;
         R = r;

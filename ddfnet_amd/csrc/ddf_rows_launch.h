@@ -106,19 +106,27 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
     constexpr int kFilterStages = DX ? 2 : 4;
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kFilterWaves);
     const int lds = filters_lds_bytes<9>((int)sizeof(A), R, VX);
-    if (p.k != 3 || p.d != 1) return hipErrorNotSupported;
+    if (p.k != 3 || (p.d != 1 && p.d != 2)) return hipErrorNotSupported;
     const bool pad = rows_shift_in_as_is(g);
-#define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
-    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, R, PAD_, DX, kFilterStages,            \
+#define DDF_ROWSF_CASE(D_, MUL_, PAD_)                                                           \
+    hipLaunchKernelGGL((k_rows_filters<T, 3, D_, MUL_, VX, R, PAD_, DX, kFilterStages,           \
                                        MUL_ ? WPE_MUL : WPE_ADD>),                               \
                        grid, block, lds, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod)
-    if (p.mul) {
-        if (pad) DDF_ROWSF_CASE(true, true);
-        else DDF_ROWSF_CASE(true, false);
-    } else {
-        if (pad) DDF_ROWSF_CASE(false, true);
-        else DDF_ROWSF_CASE(false, false);
+#define DDF_ROWSF_D(D_)                                                                          \
+    if (p.mul) {                                                                                 \
+        if (pad) DDF_ROWSF_CASE(D_, true, true);                                                 \
+        else DDF_ROWSF_CASE(D_, true, false);                                                    \
+    } else {                                                                                     \
+        if (pad) DDF_ROWSF_CASE(D_, false, true);                                                \
+        else DDF_ROWSF_CASE(D_, false, false);                                                   \
     }
+    if (p.d == 1) {
+        DDF_ROWSF_D(1)
+    } else {
+        // (dilation 2: the taps reach two pixels into the neighbouring lane; one row per lane)
+        if constexpr (VX >= 2 && R == 1) { DDF_ROWSF_D(2) } else { return hipErrorNotSupported; }
+    }
+#undef DDF_ROWSF_D
 #undef DDF_ROWSF_CASE
     return hipGetLastError();
 }
