@@ -274,13 +274,15 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
                     for (int e = 0; e < VX; ++e) {
                         const int t = i * K + j;
-                        const A gx = gval[r][e] * row[r + i * D].at(e + j * D - HX);
+                        const A xv = row[r + i * D].at(e + j * D - HX);
                         if constexpr (MUL) {
+                            const A gx = gval[r][e] * xv;
                             acc_sf[r][t][e] = fma_(gx, w[t], acc_sf[r][t][e]);
                             pcf[t] = fma_(gx, elem<T>(sfw[r][t], e), pcf[t]);
                         } else {
-                            acc_sf[r][t][e] += gx;
-                            pcf[t] += gx;
+                            // (two multiply-adds instead of a product and two additions)
+                            acc_sf[r][t][e] = fma_(gval[r][e], xv, acc_sf[r][t][e]);
+                            pcf[t] = fma_(gval[r][e], xv, pcf[t]);
                         }
                     }
         // The accumulators are not read before the walk ends: without this the compiler

@@ -219,13 +219,15 @@ __global__ __launch_bounds__(kWave * kTaprowWaves, WPE) void k_rows_taprow_filte
             for (int r = 0; r < R; ++r)
 #pragma unroll
                 for (int e = 0; e < VX; ++e) {
-                    const A gx = elem<T>(gw[ST][r], e) * row[r].at(e + j * D - HX);
+                    const A gv = elem<T>(gw[ST][r], e), xv = row[r].at(e + j * D - HX);
                     if constexpr (MUL) {
+                        const A gx = gv * xv;
                         acc_sf[r][j][e] = fma_(gx, w[j], acc_sf[r][j][e]);
                         pcf[j] = fma_(gx, elem<T>(sfw[r][j], e), pcf[j]);
                     } else {
-                        acc_sf[r][j][e] += gx;
-                        pcf[j] += gx;
+                        // (two multiply-adds instead of a product and two additions)
+                        acc_sf[r][j][e] = fma_(gv, xv, acc_sf[r][j][e]);
+                        pcf[j] = fma_(gv, xv, pcf[j]);
                     }
                 }
         // The accumulators are not read before the walk ends: without this the compiler
