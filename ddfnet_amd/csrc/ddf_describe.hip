@@ -9,6 +9,7 @@ namespace ddf {
 
 namespace {
 const char *layout_name(const RowsGeom &g) {
+    if (g.Hi != g.H) return g.lp > g.lpr ? "padded,stride 2" : "plain,stride 2";
     return g.segs > 0 ? "segments" : g.lp > g.lpr ? "padded" : "plain";
 }
 }  // namespace
@@ -41,7 +42,10 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
                            tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
                            rows_cover_backward(p, dtype);
     if (!tiled && !rows_both) { add("%s", "generic_backward"); return n; }
-    const bool fuse = tiled && (need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0 &&
+    const bool rows_filters_only = dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
+                                   rows_cover_stride2_filters(p, dtype);
+    const bool fuse = tiled && (need & DDF_NEED_DX) && fneed && !rows_both && !rows_filters_only &&
+                      tune_int("DDF_TUNE_FUSED", 1) != 0 &&
                       wave_geometry(p, dtype, kWaveFused, 0, &wg, &ps, &nv) &&
                       wave_geometry(p, dtype, kWaveFilters, 0, &gp, &pps, &pnv) && gp.TH == wg.TH &&
                       gp.csplit == wg.csplit;
@@ -59,7 +63,7 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
         return n;
     }
     if (need & DDF_NEED_DX) {
-        if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
+        if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 && p.s == 1 &&
             rows_geometry(p, dtype, 0, &rg, &vx, &r))
             add("k_rows<dX,VX=%d,R=%d,%s>", vx, r, layout_name(rg));
         else if (small_supported(p)) add("%s", "k_small<dX>");

@@ -42,7 +42,8 @@
 namespace ddf {
 
 struct RowsGeom {
-    int C, H, W;              // per sample (stride 1: the result plane has the same shape)
+    int C, H, W;              // per sample, of the result plane
+    int Hi, Wi;               // feature plane (stride 1: the same shape)
     int lpr, rg;              // lanes per image row, row groups per wave
     int lp;                   // lane pitch of a row group: lpr, or lpr + 1 (an idle lane after each row)
     unsigned lp_magic;        // ceil(2^32 / lp), 0 when lp == 1
@@ -157,6 +158,33 @@ struct Lane {
     }
 };
 
+// Stride 2, 3 x 3, one result row per lane: the lane's VX result pixels of row y
+// read the feature rows 2y-1 .. 2y+1, columns 2*x0-1 .. 2*x0+2*VX-1: a vector of
+// 2*VX elements per row at xoff (offsets inside the feature plane) and the last
+// element of the lane to the left.
+template <int VX>
+struct LaneStride2 {
+    static constexpr int ROWS = 3;
+    bool first, last;
+    int xoff[ROWS];
+    int ooff[1];
+    __host__ __device__ __forceinline__ void init(const RowsGeom &g, int strip, int lane, int = 0) {
+        const int grp = magic_div(lane, g.lp_magic);
+        const int v = lane - grp * g.lp;
+        const int y = strip * g.rps + grp;
+        const bool live = grp < g.rg && v < g.lpr && y < g.H;
+        const int x0 = v * VX;
+        first = v == 0;
+        last = v == g.lpr - 1;
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) {
+            const int yy = 2 * y - 1 + rr;
+            xoff[rr] = (live && yy >= 0 && yy < g.Hi) ? yy * g.Wi + 2 * x0 : -1;
+        }
+        ooff[0] = live ? y * g.W + x0 : -1;
+    }
+};
+
 // Window row rr (0 = HY rows above the lane's first row) is touched by some tap
 // of some of the lane's R rows: rr = r + i*D.  With dilation the window has
 // rows no tap lands on; they are neither loaded nor shifted.
@@ -187,11 +215,17 @@ __device__ __forceinline__ void load_words(__amdgpu_buffer_rsrc_t rsrc, uint32_t
     } else if constexpr (N == 2) {
         const auto v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)off, 0, 0);
         w[0] = v[0]; w[1] = v[1];
-    } else {
-        static_assert(N == 4, "vectors of 4, 8 or 16 bytes");
+    } else if constexpr (N == 4) {
         const auto v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0);
 #pragma unroll
         for (int k = 0; k < 4; ++k) w[k] = v[k];
+    } else {
+        static_assert(N == 8, "vectors of 4, 8, 16 or 32 bytes");
+        // (an offset outside the descriptor stays outside with 16 added)
+        const auto lo = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)off, 0, 0);
+        const auto hi = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)(off + 16u), 0, 0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) { w[k] = lo[k]; w[4 + k] = hi[k]; }
     }
 }
 
@@ -335,7 +369,10 @@ __device__ __forceinline__ double lane_broadcast<double>(double v, int src_lane)
 
 // BWD = false: out = forward(x, cf, sf).  BWD = true: x is dO and out is dX.
 // WPE: waves per SIMD the register allocation must leave room for.
-template <typename T, int K, int D, bool MUL, bool BWD, int VX, int R, bool PAD, int NST, int WPE>
+// S = 2 (forward, 3 x 3, one row per lane): g describes the result plane, the
+// lane's feature vectors are 2 * VX elements wide (LaneStride2).
+template <typename T, int K, int D, bool MUL, bool BWD, int VX, int R, bool PAD, int NST, int WPE,
+          int S = 1>
 __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const T *__restrict__ x,
                                                          const T *__restrict__ cf,
                                                          const T *__restrict__ sf,
@@ -343,21 +380,25 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RAD = K / 2, HX = RAD * D, HY = RAD * D;
     constexpr int ROWS = R + 2 * HY;
-    constexpr int NW = VX * sizeof(T) / 4;
-    using Row = ExtRow<T, VX, HX, PAD>;
+    constexpr int NW = VX * sizeof(T) / 4;   // words of a result vector
+    constexpr int NWX = S * NW;              // words of a feature vector
+    using Row = ExtRow<T, S * VX, HX, PAD>;
     static_assert(KK <= kWave, "one lane per channel-filter tap");
+    static_assert(S == 1 || (S == 2 && K == 3 && D == 1 && R == 1 && !BWD), "stride 2: forward, 3 x 3");
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     Work wk;
     if (!wk.init(g, blockIdx.x, wave) || wk.c_end <= wk.c_begin) return;
     const int nch = wk.c_end - wk.c_begin;
-    const int64_t plane = (int64_t)g.H * g.W;
+    const int64_t plane = (int64_t)g.H * g.W;   // result plane
     const uint32_t plane_bytes = (uint32_t)plane * (uint32_t)sizeof(T);
-    Lane<R, HY, VX> ln;
+    const int64_t xplane = S == 1 ? plane : (int64_t)g.Hi * g.Wi;
+    const uint32_t xplane_bytes = S == 1 ? plane_bytes : (uint32_t)xplane * (uint32_t)sizeof(T);
+    std::conditional_t<S == 1, Lane<R, HY, VX>, LaneStride2<VX>> ln;
     ln.init(g, wk.strip, lane);
 
-    const T *xs = x + (wk.n * g.C + wk.c_begin) * plane;
+    const T *xs = x + (wk.n * g.C + wk.c_begin) * xplane;
     T *os = out + (wk.n * g.C + wk.c_begin) * plane;
     // byte offsets of the lane's vectors inside a plane; kOutside: reads as zero, is not written
     uint32_t xb[ROWS], ob[R];
@@ -409,15 +450,15 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
 
     // feature rows and channel taps of channel ci, stage ST; a channel past the
     // wave's last one reads zeros (empty descriptor)
-    uint32_t xw[NST][ROWS][NW];
+    uint32_t xw[NST][ROWS][NWX];
     T cfl[NST];
     A cfu[NST][kScalarTaps ? KK : 1];
     auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
-        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * plane, ci < nch ? plane_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * xplane, ci < nch ? xplane_bytes : 0u);
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr)
-            if (row_needed<R, K, D>(rr)) load_words<NW>(pr, xb[rr], xw[ST][rr]);
+            if (row_needed<R, K, D>(rr)) load_words<NWX>(pr, xb[rr], xw[ST][rr]);
         const int cc = ci < nch ? ci : nch - 1;   // (the taps are read through plain pointers: stay inside)
         if constexpr (kScalarTaps) {
 #pragma unroll
@@ -458,7 +499,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
         for (int rr = 0; rr < ROWS; ++rr) {
             if (!row_needed<R, K, D>(rr)) continue;
 #pragma unroll
-            for (int k = 0; k < NW; ++k) row[rr].own[k] = xw[ST][rr][k];
+            for (int k = 0; k < NWX; ++k) row[rr].own[k] = xw[ST][rr][k];
             row[rr].sides(ln.first, ln.last);
         }
         A w[KK];
@@ -485,7 +526,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
                 for (int r = 0; r < R; ++r)
 #pragma unroll
                     for (int e = 0; e < VX; ++e) {
-                        const A xv = row[r + i * D].at(e + j * D - HX);
+                        const A xv = row[r + i * D].at(S * e + j * D - HX);
                         const A sv = elem<T>(sfw[r][i * K + j], e);
                         if constexpr (MUL) {
                             acc[r][e] = fma_(w[i * K + j], fma_(xv, sv, A(0)), acc[r][e]);

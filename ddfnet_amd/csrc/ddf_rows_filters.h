@@ -54,7 +54,10 @@ __device__ __forceinline__ void wave_sync() {
 // second set of spatial taps (those of the pixels its dO values come from),
 // and every channel ends with the store of its dX rows.  One launch for the
 // whole backward pass; dO, CF and SF are read once.
-template <typename T, int K, int D, bool MUL, int VX, int R, bool PAD, bool DX, int NST, int WPE>
+// S = 2 (3 x 3, one row per lane, filter gradients only): g describes the dO
+// plane, the lane's feature vectors are 2 * VX elements wide (LaneStride2).
+template <typename T, int K, int D, bool MUL, int VX, int R, bool PAD, bool DX, int NST, int WPE,
+          int S = 1>
 __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     RowsGeom g, const T *__restrict__ go, const T *__restrict__ x, const T *__restrict__ cf,
     const T *__restrict__ sf, T *__restrict__ dx, T *__restrict__ dcf, T *__restrict__ dsf,
@@ -66,10 +69,12 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     constexpr int GROWS = DX ? ROWS : R;       // dO rows a lane loads per channel
     constexpr int GOWN = DX ? HY : 0;          // its own first row among them
     constexpr bool kFilters = MUL || DX;       // CF and SF values are needed at all
-    constexpr int NW = VX * sizeof(T) / 4;
+    constexpr int NW = VX * sizeof(T) / 4;   // words of a dO / filter vector
+    constexpr int NWX = S * NW;              // words of a feature vector
     constexpr int G = kFlushChannels;
-    using Row = ExtRow<T, VX, HX, PAD>;
+    using Row = ExtRow<T, S * VX, HX, PAD>;
     static_assert(G * KK <= kWave, "one lane per (channel, tap) of a flush group");
+    static_assert(S == 1 || (S == 2 && K == 3 && D == 1 && R == 1 && !DX), "stride 2: 3 x 3, filters only");
     extern __shared__ __align__(16) unsigned char smem[];
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -81,15 +86,17 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     const int c0 = min(wk.c_begin + wave * g.cpw, wk.c_end);
     const int nch = min(g.cpw, wk.c_end - c0);
     const int c_first = min(c0, g.C - 1);   // (pointers of a wave without channels stay inside)
-    const int64_t plane = (int64_t)g.H * g.W;
+    const int64_t plane = (int64_t)g.H * g.W;   // dO plane
     const uint32_t plane_bytes = (uint32_t)plane * (uint32_t)sizeof(T);
-    Lane<R, HY, VX> ln;
+    const int64_t xplane = S == 1 ? plane : (int64_t)g.Hi * g.Wi;
+    const uint32_t xplane_bytes = S == 1 ? plane_bytes : (uint32_t)xplane * (uint32_t)sizeof(T);
+    std::conditional_t<S == 1, Lane<R, HY, VX>, LaneStride2<VX>> ln;
     ln.init(g, wk.strip, lane);
 
     // x_mod != 0: the batch is several groups of x_mod samples that share one set of
     // features (the sub-pixel branches of the up-sampling operator's gradient)
     const int64_t xn = x_mod ? wk.n % x_mod : wk.n;
-    const T *xs = x + (xn * g.C + c_first) * plane;
+    const T *xs = x + (xn * g.C + c_first) * xplane;
     const T *gs = go + (wk.n * g.C + c_first) * plane;
     T *ds = DX ? dx + (wk.n * g.C + c_first) * plane : nullptr;
     uint32_t xb[ROWS], ob[R];
@@ -106,18 +113,18 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     // past the wave's last one reads zeros (empty descriptors) and so adds nothing;
     // idle lanes and rows outside the image read zeros as well.
     constexpr bool kScalarTaps = sizeof(T) >= 4;   // (see k_rows)
-    uint32_t xw[NST][ROWS][NW], gw[NST][GROWS][NW];
+    uint32_t xw[NST][ROWS][NWX], gw[NST][GROWS][NW];
     T cfl[NST];
     A cfu[NST][kScalarTaps && kFilters ? KK : 1];
     auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         const uint32_t bytes = ci < nch ? plane_bytes : 0u;
-        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * plane, bytes);
+        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * xplane, ci < nch ? xplane_bytes : 0u);
         const __amdgpu_buffer_rsrc_t gr = plane_rsrc(gs + (int64_t)ci * plane, bytes);
         // (with dilation the window has rows no tap lands on: see row_needed)
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr)
-            if (row_needed<R, K, D>(rr)) load_words<NW>(pr, xb[rr], xw[ST][rr]);
+            if (row_needed<R, K, D>(rr)) load_words<NWX>(pr, xb[rr], xw[ST][rr]);
 #pragma unroll
         for (int r = 0; r < GROWS; ++r)
             if (!DX || row_needed<R, K, D>(r)) load_words<NW>(gr, DX ? xb[r] : ob[r], gw[ST][r]);
@@ -237,7 +244,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
         for (int rr = 0; rr < ROWS; ++rr) {
             if (!row_needed<R, K, D>(rr)) continue;
 #pragma unroll
-            for (int k = 0; k < NW; ++k) row[rr].own[k] = xw[ST][rr][k];
+            for (int k = 0; k < NWX; ++k) row[rr].own[k] = xw[ST][rr][k];
             row[rr].sides(ln.first, ln.last);
         }
         // dO at the lane's own pixels.  (DX loads dO through the window offsets, so a
@@ -274,7 +281,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
                     for (int e = 0; e < VX; ++e) {
                         const int t = i * K + j;
-                        const A xv = row[r + i * D].at(e + j * D - HX);
+                        const A xv = row[r + i * D].at(S * e + j * D - HX);
                         if constexpr (MUL) {
                             const A gx = gval[r][e] * xv;
                             acc_sf[r][t][e] = fma_(gx, w[t], acc_sf[r][t][e]);

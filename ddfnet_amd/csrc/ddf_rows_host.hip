@@ -52,6 +52,100 @@ void lay_out_lanes(RowsGeom *t, int H, int W, int vx, int R) {
     t->rps = t->rg * R;
 }
 
+// Channels per wave of k_rows: enough waves to fill the machine (and to even out
+// its SIMDs), walks long enough to amortise the spatial-filter registers.  The
+// kernels walk whole rounds of `nst` channels, so the count is a multiple of
+// that.  `plane`: pixels of a result plane.
+bool cut_channels_forward(RowsGeom &t, int64_t N, int C, int nst, int64_t plane) {
+    const int64_t base = N * t.nstrips;
+    const int target = tune_int("DDF_TUNE_ROWS_WAVES", 8192);
+    const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
+    int cpw = (int)(C / want_split);
+    const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", 2 * nst);
+    cpw = std::max(cpw / nst * nst, min_cpw);
+    const int forced = tune_int("DDF_TUNE_ROWS_CPW", 0);
+    if (forced) cpw = forced;
+    t.cpw = std::max(1, std::min(cpw, C));
+    t.cpb = t.cpw;
+    t.csplit = (C + t.cpw - 1) / t.cpw;
+    // (single-wave workgroups spread over the machine faster: what counts for the
+    // smallest launches)
+    t.wpb = std::max(1, std::min(tune_int("DDF_TUNE_ROWS_WPB", plane <= 256 ? 1 : 2), rows::kMaxWpb));
+    const int64_t nwork = base * t.csplit;
+    if (nwork > (1 << 30)) return false;
+    // magic-number division of the work id is exact while id * divisor < 2^32
+    if (nwork * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
+    t.csplit_magic = magic_of(t.csplit);
+    t.nstrips_magic = magic_of(t.nstrips);
+    const int64_t ngroups = (nwork + t.wpb - 1) / t.wpb;
+    t.xcd_per = (unsigned)((ngroups + rows::kXcd - 1) / rows::kXcd);
+    t.nwork = (int)nwork;
+    return true;
+}
+
+// Channels per wave of k_rows_filters: the four waves of a workgroup cover cpb =
+// 4 * cpw channels; enough workgroups to fill the machine, as few channel splits
+// (dSF partial sums through the workspace) as that allows.
+bool cut_channels_filters(RowsGeom &t, int64_t N, int C) {
+    const int64_t base = N * t.nstrips;
+    const int target = tune_int("DDF_TUNE_ROWSF_WAVES", 2048);
+    const int64_t want_split = std::max<int64_t>(1, (target + base * rows::kFilterWaves - 1) /
+                                                        (base * rows::kFilterWaves));
+    int cpb = (int)((C + want_split - 1) / want_split);
+    int cpw = (cpb + rows::kFilterWaves - 1) / rows::kFilterWaves;
+    // whole rounds of the kernel's channel pipeline and whole dCF flush groups
+    cpw = (cpw + rows::kFlushChannels - 1) / rows::kFlushChannels * rows::kFlushChannels;
+    cpw = std::max(cpw, tune_int("DDF_TUNE_ROWSF_MIN_CPW", 2 * rows::kFlushChannels));
+    const int forced = tune_int("DDF_TUNE_ROWSF_CPW", 0);
+    if (forced) cpw = std::min(forced, C);
+    t.cpw = std::max(1, cpw);
+    t.cpb = t.cpw * rows::kFilterWaves;
+    t.csplit = (C + t.cpb - 1) / t.cpb;
+    t.wpb = 1;
+    const int64_t nwork = base * t.csplit;
+    if (nwork > (1 << 30)) return false;
+    if (nwork * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
+    t.csplit_magic = magic_of(t.csplit);
+    t.nstrips_magic = magic_of(t.nstrips);
+    t.xcd_per = (unsigned)((nwork + rows::kXcd - 1) / rows::kXcd);
+    t.nwork = (int)nwork;
+    return true;
+}
+
+// Stride 2 (3 x 3, fp16 / fp32): lanes over the result plane, one row per lane,
+// vx result pixels per lane from feature vectors of 2 * vx elements.  Rows of
+// the feature plane must keep those vectors aligned (W a multiple of 2 * vx) and
+// a result row must fit the lanes of a wave.  filters: the cut of
+// k_rows_filters, else of k_rows.
+bool stride2_geometry(const Problem &p, int dtype, bool filters, RowsGeom *g, int *vx_out,
+                      int *r_out) {
+    if (!(p.s == 2 && p.k == 3 && p.d == 1)) return false;
+    if (dtype != DDF_F16 && dtype != DDF_F32) return false;
+    if (p.N <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0) return false;
+    if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
+    const int esz = dtype == DDF_F16 ? 2 : 4;
+    const int H = (int)p.H, W = (int)p.W, Ho = (int)p.Ho, Wo = (int)p.Wo, C = (int)p.C;
+    if ((int64_t)H * W * 8 >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
+    int vx = 0;
+    for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
+        if (cand > tune_int("DDF_TUNE_ROWS_VX", 16)) continue;
+        if (W % (2 * cand) != 0) continue;
+        vx = cand;
+        break;
+    }
+    if (vx == 0 || Wo / vx > kMaxRowLanes) return false;
+    RowsGeom t{};
+    t.C = C; t.H = Ho; t.W = Wo; t.Hi = H; t.Wi = W;
+    lay_out_lanes(&t, Ho, Wo, vx, 1);
+    if (filters ? !cut_channels_filters(t, p.N, C)
+                : !cut_channels_forward(t, p.N, C, kRowsStages, (int64_t)Ho * Wo))
+        return false;
+    *g = t;
+    *vx_out = vx;
+    *r_out = 1;
+    return true;
+}
+
 }  // namespace
 
 // Instantiated (elements per lane and row, rows per lane) per element size.
@@ -61,10 +155,14 @@ bool rows_variant_built(int esz, int vx, int r) {
     return false;
 }
 
-bool rows_shape_built(int k, int d, int s) { return s == 1 && (k == 3 || k == 5) && (d == 1 || d == 2); }
+// (stride 2: the forward pass only)
+bool rows_shape_built(int k, int d, int s) {
+    return (s == 1 && (k == 3 || k == 5) && (d == 1 || d == 2)) || (s == 2 && k == 3 && d == 1);
+}
 
 bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx_out, int *r_out) {
     if (!rows_shape_built(p.k, p.d, p.s)) return false;
+    if (p.s == 2) return max_vx <= 0 && stride2_geometry(p, dtype, false, g, vx_out, r_out);
     if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
     if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
     const int esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
@@ -98,37 +196,10 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     if (!rows_variant_built(esz, vx, R)) return false;
 
     RowsGeom t{};
-    t.C = C; t.H = H; t.W = W;
+    t.C = C; t.H = t.Hi = H; t.W = t.Wi = W;
     lay_out_lanes(&t, H, W, vx, R);
 
-    // Channels per wave: enough waves to fill the machine (and to even out its
-    // SIMDs), walks long enough to amortise the spatial-filter registers.  The
-    // kernels walk whole rounds of kRowsStages channels, so the count is a
-    // multiple of that.
-    const int64_t base = p.N * t.nstrips;
-    const int target = tune_int("DDF_TUNE_ROWS_WAVES", 8192);
-    const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
-    int cpw = (int)(C / want_split);
-    const int nst = p.k == 5 ? 2 : kRowsStages;
-    const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", 2 * nst);
-    cpw = std::max(cpw / nst * nst, min_cpw);
-    const int forced = tune_int("DDF_TUNE_ROWS_CPW", 0);
-    if (forced) cpw = forced;
-    t.cpw = std::max(1, std::min(cpw, C));
-    t.cpb = t.cpw;
-    t.csplit = (C + t.cpw - 1) / t.cpw;
-    // (single-wave workgroups spread over the machine faster: what counts for the
-    // smallest launches)
-    t.wpb = std::max(1, std::min(tune_int("DDF_TUNE_ROWS_WPB", H * W <= 256 ? 1 : 2), rows::kMaxWpb));
-    const int64_t nwork = base * t.csplit;
-    if (nwork > (1 << 30)) return false;
-    // magic-number division of the work id is exact while id * divisor < 2^32
-    if (nwork * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
-    t.csplit_magic = magic_of(t.csplit);
-    t.nstrips_magic = magic_of(t.nstrips);
-    const int64_t ngroups = (nwork + t.wpb - 1) / t.wpb;
-    t.xcd_per = (unsigned)((ngroups + rows::kXcd - 1) / rows::kXcd);
-    t.nwork = (int)nwork;
+    if (!cut_channels_forward(t, p.N, C, p.k == 5 ? 2 : kRowsStages, (int64_t)H * W)) return false;
     *g = t;
     *vx_out = vx;
     *r_out = R;
@@ -146,6 +217,7 @@ bool rows_filters_variant_built(int esz, int vx, int r, bool fused) {
 
 bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g, int *vx_out,
                            int *r_out) {
+    if (p.s == 2) return !fused && stride2_geometry(p, dtype, true, g, vx_out, r_out);
     if (!(p.s == 1 && p.k == 3 && (p.d == 1 || p.d == 2))) return false;
     if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
     if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
@@ -172,34 +244,10 @@ bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g,
     if (vx == 0) return false;
 
     RowsGeom t{};
-    t.C = C; t.H = H; t.W = W;
+    t.C = C; t.H = t.Hi = H; t.W = t.Wi = W;
     lay_out_lanes(&t, H, W, vx, R);
 
-    // Channels per wave: the four waves of a workgroup cover cpb = 4 * cpw
-    // channels; enough workgroups to fill the machine, as few channel splits
-    // (dSF partial sums through the workspace) as that allows.
-    const int64_t base = p.N * t.nstrips;
-    const int target = tune_int("DDF_TUNE_ROWSF_WAVES", 2048);
-    const int64_t want_split = std::max<int64_t>(1, (target + base * rows::kFilterWaves - 1) /
-                                                        (base * rows::kFilterWaves));
-    int cpb = (int)((C + want_split - 1) / want_split);
-    int cpw = (cpb + rows::kFilterWaves - 1) / rows::kFilterWaves;
-    // whole rounds of the kernel's channel pipeline and whole dCF flush groups
-    cpw = (cpw + rows::kFlushChannels - 1) / rows::kFlushChannels * rows::kFlushChannels;
-    cpw = std::max(cpw, tune_int("DDF_TUNE_ROWSF_MIN_CPW", 2 * rows::kFlushChannels));
-    const int forced = tune_int("DDF_TUNE_ROWSF_CPW", 0);
-    if (forced) cpw = std::min(forced, C);
-    t.cpw = std::max(1, cpw);
-    t.cpb = t.cpw * rows::kFilterWaves;
-    t.csplit = (C + t.cpb - 1) / t.cpb;
-    t.wpb = 1;
-    const int64_t nwork = base * t.csplit;
-    if (nwork > (1 << 30)) return false;
-    if (nwork * std::max(t.csplit, t.nstrips) >= (1ll << 32)) return false;
-    t.csplit_magic = magic_of(t.csplit);
-    t.nstrips_magic = magic_of(t.nstrips);
-    t.xcd_per = (unsigned)((nwork + rows::kXcd - 1) / rows::kXcd);
-    t.nwork = (int)nwork;
+    if (!cut_channels_filters(t, p.N, C)) return false;
     *g = t;
     *vx_out = vx;
     *r_out = R;
@@ -231,7 +279,7 @@ bool rows_taprow_geometry(const Problem &p, int dtype, RowsGeom *g, int *vx_out,
         if (cand > tune_int("DDF_TUNE_TAPROW_VX", 16)) continue;
         if (W % cand != 0 || cand < hx || cand < 2) continue;
         RowsGeom c{};
-        c.C = C; c.H = H; c.W = W;
+        c.C = C; c.H = c.Hi = H; c.W = c.Wi = W;
         lay_out_lanes(&c, H, W, cand, 1);
         t = c;
         vx = cand;
@@ -266,9 +314,14 @@ bool rows_taprow_geometry(const Problem &p, int dtype, RowsGeom *g, int *vx_out,
 
 bool rows_cover_backward(const Problem &p, int dtype) {
     RowsGeom g; int vx, r;
-    return rows_geometry(p, dtype, 0, &g, &vx, &r) &&
+    return p.s == 1 && rows_geometry(p, dtype, 0, &g, &vx, &r) &&
            (rows_taprow_geometry(p, dtype, &g, &vx, &r) ||
             rows_filters_geometry(p, dtype, false, &g, &vx, &r));
+}
+
+bool rows_cover_stride2_filters(const Problem &p, int dtype) {
+    RowsGeom g; int vx, r;
+    return p.s == 2 && rows_filters_geometry(p, dtype, false, &g, &vx, &r);
 }
 
 size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need) {
@@ -284,7 +337,7 @@ size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need) {
             continue;
         size_t bytes = 0;
         if ((need & DDF_NEED_DSF) && g.csplit > 1)
-            bytes += ((size_t)p.N * g.csplit * p.kk * p.H * p.W * asz + 255) / 256 * 256;
+            bytes += ((size_t)p.N * g.csplit * p.kk * p.Ho * p.Wo * asz + 255) / 256 * 256;
         if ((need & DDF_NEED_DCF) && g.nstrips > 1)
             bytes += ((size_t)p.N * p.C * g.nstrips * p.kk * asz + 255) / 256 * 256;
         most = std::max(most, bytes);

@@ -1,6 +1,8 @@
 // Launch code of the row-register kernels, instantiated once per element type.
 #pragma once
 
+#include <algorithm>
+
 #include "ddf_rows_taprow.h"
 #include "ddf_wave.h"
 
@@ -44,6 +46,27 @@ hipError_t launch_kdv(const Problem &p, const RowsGeom &g, bool backward, const 
     return hipGetLastError();
 }
 
+// Stride 2, forward.
+template <typename T, int VX>
+hipError_t launch_stride2_v(const Problem &p, const RowsGeom &g, const T *x, const T *cf,
+                            const T *sf, T *out, hipStream_t st) {
+    const dim3 grid(g.xcd_per * kXcd), block(kWave * g.wpb);
+    const bool pad = rows_shift_in_as_is(g);
+    constexpr int kWpe = sizeof(T) == 2 && VX >= 8 ? 2 : 3;
+#define DDF_ROWS_CASE(MUL_, PAD_)                                                               \
+    hipLaunchKernelGGL((k_rows<T, 3, 1, MUL_, false, VX, 1, PAD_, kStages, kWpe, 2>), grid,     \
+                       block, 0, st, g, x, cf, sf, out)
+    if (p.mul) {
+        if (pad) DDF_ROWS_CASE(true, true);
+        else DDF_ROWS_CASE(true, false);
+    } else {
+        if (pad) DDF_ROWS_CASE(false, true);
+        else DDF_ROWS_CASE(false, false);
+    }
+#undef DDF_ROWS_CASE
+    return hipGetLastError();
+}
+
 template <typename T, int VX, int R>
 hipError_t launch_v(const Problem &p, const RowsGeom &g, bool backward, const T *x, const T *cf,
                     const T *sf, T *out, hipStream_t st) {
@@ -76,6 +99,22 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
     if (!rows_geometry(p, dtype, 0, &g, &vx, &r)) return hipErrorNotSupported;
     const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
     if ((((uintptr_t)x | (uintptr_t)sf | (uintptr_t)out) & mask) != 0) return hipErrorNotSupported;
+    if (p.s == 2) {
+        // (feature vectors are twice as long and come in pieces of at most 16 bytes)
+        if (backward || ((uintptr_t)x & (std::min<uintptr_t>(2 * vx * sizeof(T), 16) - 1)) != 0)
+            return hipErrorNotSupported;
+        if constexpr (sizeof(T) == 2) {
+            if (vx == 8) return rows::launch_stride2_v<T, 8>(p, g, x, cf, sf, out, st);
+        }
+        if constexpr (sizeof(T) == 4) {
+            if (vx == 1) return rows::launch_stride2_v<T, 1>(p, g, x, cf, sf, out, st);
+        }
+        if constexpr (sizeof(T) != 8) {
+            if (vx == 4) return rows::launch_stride2_v<T, 4>(p, g, x, cf, sf, out, st);
+            if (vx == 2) return rows::launch_stride2_v<T, 2>(p, g, x, cf, sf, out, st);
+        }
+        return hipErrorNotSupported;
+    }
     if constexpr (sizeof(T) == 2) {
         if (vx == 8 && r == 1) return rows::launch_v<T, 8, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
@@ -127,6 +166,33 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
         if constexpr (VX >= 2 && R == 1) { DDF_ROWSF_D(2) } else { return hipErrorNotSupported; }
     }
 #undef DDF_ROWSF_D
+#undef DDF_ROWSF_CASE
+    return hipGetLastError();
+}
+
+// Stride 2: filter gradients (the feature gradient is a launch of its own).
+template <typename T, int VX>
+hipError_t launch_filters_stride2_v(const Problem &p, const RowsGeom &g, const T *go, const T *x,
+                                    const T *cf, const T *sf, T *dcf, T *dsf,
+                                    typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
+                                    unsigned need, hipStream_t st) {
+    using A = typename Acc<T>::type;
+    // (channels in flight per wave: 32-byte feature vectors of fp16 leave room for two)
+    constexpr int kStagesS2 = sizeof(T) == 2 && VX >= 8 ? 2 : 4, kWpe = 2;
+    const dim3 grid(g.xcd_per * kXcd), block(kWave * kFilterWaves);
+    const int lds = filters_lds_bytes<9>((int)sizeof(A), 1, VX);
+    const bool pad = rows_shift_in_as_is(g);
+#define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
+    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, 1, PAD_, false, kStagesS2, kWpe, 2>),  \
+                       grid, block, lds, st, g, go, x, cf, sf, (T *)nullptr, dcf, dsf, ws_sf,    \
+                       ws_cf, need, 0)
+    if (p.mul) {
+        if (pad) DDF_ROWSF_CASE(true, true);
+        else DDF_ROWSF_CASE(true, false);
+    } else {
+        if (pad) DDF_ROWSF_CASE(false, true);
+        else DDF_ROWSF_CASE(false, false);
+    }
 #undef DDF_ROWSF_CASE
     return hipGetLastError();
 }
@@ -193,9 +259,11 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
     if ((((uintptr_t)x | (uintptr_t)go | (uintptr_t)sf | (uintptr_t)dsf | (uintptr_t)dx) & mask) != 0)
         return hipErrorNotSupported;
+    if (p.s == 2 && (x_mod != 0 || ((uintptr_t)x & (std::min<uintptr_t>(2 * vx * sizeof(T), 16) - 1)) != 0))
+        return hipErrorNotSupported;
     unsigned char *wp = static_cast<unsigned char *>(ws);
     A *ws_sf = nullptr, *ws_cf = nullptr;
-    const int64_t n_sf = p.N * p.kk * p.H * p.W;
+    const int64_t n_sf = p.N * p.kk * p.Ho * p.Wo;
     if ((need & DDF_NEED_DSF) && g.csplit > 1) {
         ws_sf = reinterpret_cast<A *>(wp);
         wp += ((size_t)n_sf * g.csplit * sizeof(A) + 255) / 256 * 256;
@@ -203,7 +271,19 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     if ((need & DDF_NEED_DCF) && g.nstrips > 1) ws_cf = reinterpret_cast<A *>(wp);
     hipError_t err = hipErrorNotSupported;
     if constexpr (sizeof(T) != 8) {
-        if (taprow) {
+        if (p.s == 2) {
+            if (vx == 4)
+                err = rows::launch_filters_stride2_v<T, 4>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            else if (vx == 2)
+                err = rows::launch_filters_stride2_v<T, 2>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            if constexpr (sizeof(T) == 2) {
+                if (vx == 8)
+                    err = rows::launch_filters_stride2_v<T, 8>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            } else {
+                if (vx == 1)
+                    err = rows::launch_filters_stride2_v<T, 1>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+            }
+        } else if (taprow) {
             if (vx == 4)
                 err = rows::launch_taprow_v<T, 4>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             else if (vx == 2)
@@ -233,7 +313,7 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     }
     if (err != hipSuccess) return err;
     if (ws_sf) {
-        err = wave::sum_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.H * p.W, st);
+        err = wave::sum_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, st);
         if (err != hipSuccess) return err;
     }
     if (ws_cf) err = wave::sum_partials<T>(ws_cf, dcf, p.N * p.C, g.nstrips, (int64_t)p.kk, st);

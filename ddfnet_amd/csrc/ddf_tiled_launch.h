@@ -194,7 +194,13 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
         rows_both = tune_int("DDF_TUNE_ROWS", 1) != 0 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
                     rows_cover_backward(p, dtype);
     }
-    if ((need & DDF_NEED_DX) && fneed && !rows_both && tune_int("DDF_TUNE_FUSED", 1) != 0) {
+    // (stride 2: the row-register kernels do the filter gradients, the tile kernel dX)
+    bool rows_filters_only = false;
+    if constexpr (sizeof(T) != 8) {
+        rows_filters_only = tune_int("DDF_TUNE_ROWSF", 1) != 0 && rows_cover_stride2_filters(p, dtype);
+    }
+    if ((need & DDF_NEED_DX) && fneed && !rows_both && !rows_filters_only &&
+        tune_int("DDF_TUNE_FUSED", 1) != 0) {
         WaveGeom gp; int pps, pnv;
         fuse = wave_plan<T>(p, kWaveFused, {go, x, sf, dx}, &g, &ps, &nv) &&
                wave_geometry(p, dtype, kWaveFilters, 0, &gp, &pps, &pnv) && gp.TH == g.TH &&
