@@ -8,6 +8,11 @@
 namespace ddf {
 
 namespace {
+// The launch that adds up what a filter-gradient kernel leaves in the workspace.
+const char *sums_name(unsigned fneed, int csplit, int nstrips) {
+    const bool sf = (fneed & DDF_NEED_DSF) && csplit > 1, cf = (fneed & DDF_NEED_DCF) && nstrips > 1;
+    return sf && cf ? " + k_sum_partials_pair" : (sf || cf) ? " + k_sum_partials" : "";
+}
 const char *layout_name(const RowsGeom &g) {
     if (g.Hi != g.H) return g.lp > g.lpr ? "padded,stride 2" : "plain,stride 2";
     return g.segs > 0 ? "segments" : g.lp > g.lpr ? "padded" : "plain";
@@ -52,14 +57,12 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
     if ((need & DDF_NEED_DX) && fneed && dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
         rows_filters_geometry(p, dtype, true, &rg, &vx, &r)) {
         add("k_rows_filters<dX,VX=%d,R=%d,%s>", vx, r, layout_name(rg));
-        if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
-        if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
+        add("%s", sums_name(fneed, rg.csplit, rg.nstrips));
         return n;
     }
     if (fuse) {
         add("%s", "k_backward_filters<DX>");
-        if ((fneed & DDF_NEED_DSF) && wg.csplit > 1) add("%s", " + k_sum_partials");
-        if ((fneed & DDF_NEED_DCF) && wg.nstrips > 1) add("%s", " + k_sum_partials");
+        add("%s", sums_name(fneed, wg.csplit, wg.nstrips));
         return n;
     }
     if (need & DDF_NEED_DX) {
@@ -74,18 +77,15 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
         if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
             rows_taprow_geometry(p, dtype, &rg, &vx, &r)) {
             add("k_rows_taprow_filters<VX=%d,%s>", vx, layout_name(rg));
-            if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
-            if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
+            add("%s", sums_name(fneed, rg.csplit, rg.nstrips));
         } else if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWSF", 1) != 0 &&
             rows_filters_geometry(p, dtype, false, &rg, &vx, &r)) {
             add("k_rows_filters<VX=%d,R=%d,%s>", vx, r, layout_name(rg));
-            if ((fneed & DDF_NEED_DSF) && rg.csplit > 1) add("%s", " + k_sum_partials");
-            if ((fneed & DDF_NEED_DCF) && rg.nstrips > 1) add("%s", " + k_sum_partials");
+            add("%s", sums_name(fneed, rg.csplit, rg.nstrips));
         } else {
             wave_geometry(p, dtype, kWaveFilters, 0, &wg, &ps, &nv);
             add("%s", "k_backward_filters");
-            if ((fneed & DDF_NEED_DSF) && wg.csplit > 1) add("%s", " + k_sum_partials");
-            if ((fneed & DDF_NEED_DCF) && wg.nstrips > 1) add("%s", " + k_sum_partials");
+            add("%s", sums_name(fneed, wg.csplit, wg.nstrips));
         }
     }
     return n;

@@ -312,12 +312,8 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
         }
     }
     if (err != hipSuccess) return err;
-    if (ws_sf) {
-        err = wave::sum_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, st);
-        if (err != hipSuccess) return err;
-    }
-    if (ws_cf) err = wave::sum_partials<T>(ws_cf, dcf, p.N * p.C, g.nstrips, (int64_t)p.kk, st);
-    return err;
+    return wave::sum_filter_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, ws_cf, dcf,
+                                        p.N * p.C, g.nstrips, (int64_t)p.kk, st);
 }
 
 template <typename T>

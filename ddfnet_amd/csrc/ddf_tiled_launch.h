@@ -254,16 +254,10 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
                                     p, g, ps, nv, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, fneed,
                                     st));
         if (err != hipSuccess) return err;
-        if (ws_sf) {
-            // dSF[n, t, pix] = sum over channel splits
-            err = wave::sum_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, st);
-            if (err != hipSuccess) return err;
-        }
-        if (ws_cf) {
-            // dCF[nc, t] = sum over strips
-            err = wave::sum_partials<T>(ws_cf, dcf, p.N * p.C, g.nstrips, (int64_t)p.kk, st);
-            if (err != hipSuccess) return err;
-        }
+        // dSF[n, t, pix] = sum over channel splits, dCF[nc, t] = sum over strips
+        err = wave::sum_filter_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, ws_cf, dcf,
+                                           p.N * p.C, g.nstrips, (int64_t)p.kk, st);
+        if (err != hipSuccess) return err;
     }
     return err;
 }

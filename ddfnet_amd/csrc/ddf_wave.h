@@ -1108,12 +1108,12 @@ __global__ __launch_bounds__(kWave * kFilterWaves) void k_backward_filters(
 // thread adds up VEC neighbouring i (inner % VEC == 0) and keeps 8 loads in
 // flight; the order of the additions is fixed, so results are reproducible.
 template <typename T, int VEC>
-__global__ __launch_bounds__(256) void k_sum_partials(
-    const typename Acc<T>::type *__restrict__ part, T *__restrict__ out, int64_t outer,
-    int parts, int64_t inner) {
+__device__ __forceinline__ void sum_partials_block(const typename Acc<T>::type *__restrict__ part,
+                                                   T *__restrict__ out, int64_t outer, int parts,
+                                                   int64_t inner, unsigned block) {
     using A = typename Acc<T>::type;
     const int64_t iv = inner / VEC;
-    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t idx = (int64_t)block * 256 + threadIdx.x;
     if (idx >= outer * iv) return;
     const int64_t o = idx / iv, i = (idx - o * iv) * VEC;
     const A *src = part + o * parts * inner + i;
@@ -1140,20 +1140,75 @@ __global__ __launch_bounds__(256) void k_sum_partials(
     for (int k = 0; k < VEC; ++k) st(out + o * inner + i + k, tot[k]);
 }
 
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void k_sum_partials(
+    const typename Acc<T>::type *__restrict__ part, T *__restrict__ out, int64_t outer,
+    int parts, int64_t inner) {
+    sum_partials_block<T, VEC>(part, out, outer, parts, inner, blockIdx.x);
+}
+
+// One sum of partials: the arguments of k_sum_partials and the blocks it takes.
+template <typename T>
+struct SumJob {
+    const typename Acc<T>::type *part;
+    T *out;
+    int64_t outer, inner;
+    int parts;
+    bool wide;         // four neighbouring elements per thread
+    unsigned blocks;
+};
+template <typename T>
+inline SumJob<T> sum_job(const typename Acc<T>::type *part, T *out, int64_t outer, int parts,
+                         int64_t inner) {
+    using A = typename Acc<T>::type;
+    SumJob<T> j{part, out, outer, inner, parts, sizeof(A) == 4 && inner % 4 == 0, 0};
+    const int64_t threads = outer * (j.wide ? inner / 4 : inner);
+    j.blocks = (unsigned)((threads + 255) / 256);
+    return j;
+}
+
+// Two independent sums in one launch: the first a.blocks workgroups take a,
+// the others b.
+template <typename T>
+__global__ __launch_bounds__(256) void k_sum_partials_pair(SumJob<T> a, SumJob<T> b) {
+    const bool second = blockIdx.x >= a.blocks;
+    const SumJob<T> &j = second ? b : a;
+    const unsigned block = second ? blockIdx.x - a.blocks : blockIdx.x;
+    if (j.wide) sum_partials_block<T, 4>(j.part, j.out, j.outer, j.parts, j.inner, block);
+    else sum_partials_block<T, 1>(j.part, j.out, j.outer, j.parts, j.inner, block);
+}
+
 // Launches k_sum_partials with the widest access the sizes allow (the
 // workspace is 256-byte aligned).
 template <typename T>
 inline hipError_t sum_partials(const typename Acc<T>::type *part, T *out, int64_t outer,
                                int parts, int64_t inner, hipStream_t st) {
-    using A = typename Acc<T>::type;
-    const bool wide = sizeof(A) == 4 && inner % 4 == 0;
-    const int64_t threads = outer * (wide ? inner / 4 : inner);
-    const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
-    if (wide)
+    const SumJob<T> j = sum_job<T>(part, out, outer, parts, inner);
+    const dim3 grid(j.blocks), block(256);
+    if (j.wide)
         hipLaunchKernelGGL((k_sum_partials<T, 4>), grid, block, 0, st, part, out, outer, parts, inner);
     else
         hipLaunchKernelGGL((k_sum_partials<T, 1>), grid, block, 0, st, part, out, outer, parts, inner);
     return hipGetLastError();
+}
+
+// The partial sums a filter-gradient launch leaves behind: dSF over `csplit`
+// channel splits and / or dCF over `nstrips` strips (null: nothing to add), in
+// one launch.
+template <typename T>
+inline hipError_t sum_filter_partials(const typename Acc<T>::type *ws_sf, T *dsf, int64_t n,
+                                      int csplit, int64_t sf_inner,
+                                      const typename Acc<T>::type *ws_cf, T *dcf, int64_t nc,
+                                      int nstrips, int64_t kk, hipStream_t st) {
+    if (ws_sf && ws_cf) {
+        const SumJob<T> a = sum_job<T>(ws_sf, dsf, n, csplit, sf_inner);
+        const SumJob<T> b = sum_job<T>(ws_cf, dcf, nc, nstrips, kk);
+        hipLaunchKernelGGL((k_sum_partials_pair<T>), dim3(a.blocks + b.blocks), dim3(256), 0, st, a, b);
+        return hipGetLastError();
+    }
+    if (ws_sf) return sum_partials<T>(ws_sf, dsf, n, csplit, sf_inner, st);
+    if (ws_cf) return sum_partials<T>(ws_cf, dcf, nc, nstrips, kk, st);
+    return hipSuccess;
 }
 
 }  // namespace wave

@@ -178,6 +178,38 @@ static void check_geometry(int kind, long N, long C, long H, long W, int k, int 
     g_fails = 0;
 }
 
+// Every work item mapped to its own (sample, strip, channel range[, tap row]), the
+// channel ranges covering C, the workgroups dealt out evenly over the XCDs.
+static void check_work_items(const RowsGeom &g, long N, long C, int kind, int taps) {
+    const bool filters = kind == 1;
+    const int per = kind == 2 ? taps : 1;   // waves (one per filter row) per (sample, strip, channel range)
+    const long items = (long)N * g.nstrips * g.csplit * per;
+    CHECK(items == g.nwork, "work items %d", g.nwork);
+    CHECK((long)g.csplit * g.cpb >= C && (long)(g.csplit - 1) * g.cpb < C, "channel ranges");
+    if (filters) CHECK(g.cpb == g.cpw * rows::kFilterWaves && g.wpb == 1, "filter workgroup shape");
+    else if (kind == 2) CHECK(g.cpb == g.cpw && g.wpb == rows::kTaprowWaves, "tap-row workgroup shape");
+    else CHECK(g.cpb == g.cpw && g.wpb >= 1 && g.wpb <= rows::kMaxWpb, "waves per workgroup");
+    const long groups = (items + g.wpb - 1) / g.wpb;
+    CHECK((long)g.xcd_per * 8 >= groups && (long)(g.xcd_per - 1) * 8 < groups, "workgroups per XCD");
+    const long nblk = (long)g.xcd_per * 8;
+    std::vector<char> seen(items, 0);
+    const long stepb = nblk > 100000 ? 53 : 1;
+    for (long blk = 0; blk < nblk; blk += stepb)
+        for (int w = 0; w < g.wpb; ++w) {
+            rows::Work wk;
+            const int item = rows::Work::item_of(g, (int)blk, w);
+            if (item < 0) continue;
+            wk.decode(g, item / per);   // (as the kernels do)
+            const long id = (((long)wk.n * g.nstrips + wk.strip) * g.csplit + wk.cs) * per + item % per;
+            CHECK(wk.n < N && wk.strip < g.nstrips && wk.cs < g.csplit && id < items, "work item out of range");
+            if (id < items) { CHECK(!seen[id], "work item %ld handed out twice", id); seen[id] = 1; }
+            CHECK(wk.c_begin == wk.cs * g.cpb && wk.c_end <= C && wk.c_end > wk.c_begin, "channel range");
+        }
+    if (stepb == 1)
+        for (long i = 0; i < items; ++i)
+            if (!seen[i]) { CHECK(false, "work item %ld never handed out", i); break; }
+}
+
 // Row-register kernels (ddf_rows.h, ddf_rows_filters.h): the kernels ask rows::Lane and
 // rows::Work - the very code compiled here - where a lane's vectors are, so the model runs
 // that code for every lane of every strip and checks what the kernels rely on: offsets
@@ -248,33 +280,7 @@ static void replay_rows(const RowsGeom &g, long N, long C, int kind, int taps = 
         }
     for (long i = 0; i < plane; ++i)
         if (owner[i] != 1) { CHECK(false, "pixel %ld owned %d times", i, owner[i]); break; }
-    // work items
-    const int per = kind == 2 ? taps : 1;   // waves (one per filter row) per (sample, strip, channel range)
-    const long items = (long)N * g.nstrips * g.csplit * per;
-    CHECK(items == g.nwork, "work items %d", g.nwork);
-    CHECK((long)g.csplit * g.cpb >= C && (long)(g.csplit - 1) * g.cpb < C, "channel ranges");
-    if (filters) CHECK(g.cpb == g.cpw * rows::kFilterWaves && g.wpb == 1, "filter workgroup shape");
-    else if (kind == 2) CHECK(g.cpb == g.cpw && g.wpb == rows::kTaprowWaves, "tap-row workgroup shape");
-    else CHECK(g.cpb == g.cpw && g.wpb >= 1 && g.wpb <= rows::kMaxWpb, "waves per workgroup");
-    const long groups = (items + g.wpb - 1) / g.wpb;
-    CHECK((long)g.xcd_per * 8 >= groups && (long)(g.xcd_per - 1) * 8 < groups, "workgroups per XCD");
-    const long nblk = (long)g.xcd_per * 8;
-    std::vector<char> seen(items, 0);
-    const long stepb = nblk > 100000 ? 53 : 1;
-    for (long blk = 0; blk < nblk; blk += stepb)
-        for (int w = 0; w < g.wpb; ++w) {
-            rows::Work wk;
-            const int item = rows::Work::item_of(g, (int)blk, w);
-            if (item < 0) continue;
-            wk.decode(g, item / per);   // (as the kernels do)
-            const long id = (((long)wk.n * g.nstrips + wk.strip) * g.csplit + wk.cs) * per + item % per;
-            CHECK(wk.n < N && wk.strip < g.nstrips && wk.cs < g.csplit && id < items, "work item out of range");
-            if (id < items) { CHECK(!seen[id], "work item %ld handed out twice", id); seen[id] = 1; }
-            CHECK(wk.c_begin == wk.cs * g.cpb && wk.c_end <= C && wk.c_end > wk.c_begin, "channel range");
-        }
-    if (stepb == 1)
-        for (long i = 0; i < items; ++i)
-            if (!seen[i]) { CHECK(false, "work item %ld never handed out", i); break; }
+    check_work_items(g, N, C, kind, taps);
 }
 
 static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, bool filters, bool fused = false,
@@ -326,6 +332,76 @@ static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, 
     g_fails = 0;
 }
 
+// Stride 2 (3 x 3) on the row-register kernels: lanes are laid out over the result plane;
+// rows::LaneStride2 says where the lane's three feature vectors (2 * VX elements each) and
+// its VX result pixels are.
+template <int VX>
+static void replay_rows_stride2(const RowsGeom &g, long N, long C, int esz, bool filters) {
+    const long plane = (long)g.H * g.W, xplane = (long)g.Hi * g.Wi;
+    std::vector<int> owner(plane, 0);
+    CHECK(g.segs == 0 && g.lpr * VX == g.W && g.lpr <= 32, "lanes per result row");
+    CHECK(g.lp == g.lpr || g.lp == g.lpr + 1, "lane pitch %d for %d lanes per row", g.lp, g.lpr);
+    CHECK((long)(g.rg - 1) * g.lp + g.lpr <= 64, "row groups do not fit the wavefront");
+    CHECK(g.H == g.Hi / 2 && g.W == g.Wi / 2 && g.Wi % (2 * VX) == 0, "planes %dx%d -> %dx%d", g.Hi, g.Wi, g.H, g.W);
+    const int piece = 2 * VX * esz < 16 ? 2 * VX * esz : 16;   // bytes of one load instruction
+    for (int strip = 0; strip < g.nstrips; ++strip)
+        for (int lane = 0; lane < 64; ++lane) {
+            rows::LaneStride2<VX> ln;
+            ln.init(g, strip, lane);
+            const int grp = lane / g.lp, v = lane % g.lp;
+            const int y = strip * g.rps + grp, x0 = v * VX;
+            const bool live = grp < g.rg && v < g.lpr && y < g.H;
+            for (int rr = 0; rr < 3; ++rr) {
+                const int yy = 2 * y - 1 + rr, off = ln.xoff[rr];
+                if (!live || yy < 0) { CHECK(off < 0, "lane %d row %d should read nothing", lane, rr); continue; }
+                CHECK(yy < g.Hi, "feature row %d beyond the plane", yy);
+                CHECK(off == yy * g.Wi + 2 * x0 && off + 2 * VX <= xplane, "offset %d is not row %d column %d", off, yy, 2 * x0);
+                CHECK(((long)off * esz) % piece == 0, "offset %d misaligned", off);
+            }
+            if (live) {
+                CHECK(ln.ooff[0] == y * g.W + x0, "result offset");
+                for (int e = 0; e < VX; ++e) ++owner[ln.ooff[0] + e];
+            } else {
+                CHECK(ln.ooff[0] < 0, "idle lane %d writes", lane);
+            }
+            CHECK(ln.first == (v == 0) && ln.last == (v == g.lpr - 1), "row ends");
+        }
+    for (long i = 0; i < plane; ++i)
+        if (owner[i] != 1) { CHECK(false, "pixel %ld owned %d times", i, owner[i]); break; }
+    check_work_items(g, N, C, filters ? 1 : 0, 0);
+}
+
+static void check_rows_stride2(long N, long C, long H, long W, int dtype, bool filters) {
+    const Problem p = make_problem(N, C, H, W, 3, 1, 2, 0);
+    RowsGeom g;
+    int vx, r;
+    const bool ok = filters ? rows_filters_geometry(p, dtype, false, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r);
+    const char *name = filters ? "-filters" : "";
+    if (!ok) {
+        printf("kind rows%s stride 2 %ldx%ldx%ldx%ld dt%d: unsupported\n", name, N, C, H, W, dtype);
+        return;
+    }
+    printf("kind rows%s stride 2 %ldx%ldx%ldx%ld dt%d: vx=%d lpr=%d lp=%d rg=%d rps=%d nstrips=%d cpw=%d cpb=%d "
+           "csplit=%d wpb=%d nwork=%d\n", name, N, C, H, W, dtype, vx, g.lpr, g.lp, g.rg, g.rps, g.nstrips,
+           g.cpw, g.cpb, g.csplit, g.wpb, g.nwork);
+    const int esz = dtype == 0 ? 2 : 4;
+    CHECK(dtype != 2 && r == 1, "stride 2 variant");
+    CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4, "vector of %d bytes", vx * esz);
+    CHECK(!rows_filters_geometry(p, dtype, true, &g, &vx, &r), "no one-launch backward with stride 2");
+    (filters ? rows_filters_geometry(p, dtype, false, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r));
+    if (filters) {
+        CHECK(rows::filters_lds_bytes<9>(4, 1, vx) <= 64 * 1024, "filter kernel LDS");
+        CHECK(g.cpw % rows::kFlushChannels == 0, "channels per wave %d not whole flush groups", g.cpw);
+    }
+    if (vx == 1) replay_rows_stride2<1>(g, N, C, esz, filters);
+    else if (vx == 2) replay_rows_stride2<2>(g, N, C, esz, filters);
+    else if (vx == 4) replay_rows_stride2<4>(g, N, C, esz, filters);
+    else if (vx == 8) replay_rows_stride2<8>(g, N, C, esz, filters);
+    else CHECK(false, "no replay for vx=%d", vx);
+    if (g_fails) printf("  -> %d violations\n", g_fails);
+    g_fails = 0;
+}
+
 int main() {
     const long shapes[][4] = {
         {96, 64, 56, 56},   {64, 256, 14, 14}, {64, 128, 28, 28},  {64, 512, 7, 7},   {64, 64, 56, 56},
@@ -354,6 +430,10 @@ int main() {
                 check_rows(sh[0], sh[1], sh[2], sh[3], 5, d, dtype, true, false, true);
                 check_rows(sh[0], sh[1], sh[2], sh[3], 3, d, dtype, true, false, true);
             }
+    for (auto &sh : shapes)
+        for (int dtype = 0; dtype < 3; ++dtype)
+            for (int filters = 0; filters < 2; ++filters)
+                check_rows_stride2(sh[0], sh[1], sh[2], sh[3], dtype, filters != 0);
     // seeded random shapes on top of the fixed list
     unsigned long long state = 0x9E3779B97F4A7C15ull;
     auto next = [&](int lo, int hi) {
@@ -371,6 +451,8 @@ int main() {
         check_rows(N, C, H, (W / 8 + 1) * 8, 5, next(1, 2), next(0, 1), false);
         check_rows(N, C, H, (W / 8 + 1) * 8 * next(1, 6), 3, next(1, 2), next(0, 1), next(0, 1) != 0);
         check_rows(N, C, H, (W / 4 + 1) * 4, 5, next(1, 2), next(0, 1), true, false, true);
+        check_rows_stride2(N, C, H + 1, (W / 4 + 1) * 4, next(0, 1), next(0, 1) != 0);
+        check_rows_stride2(N, C, H + 1, (W / 16 + 1) * 16, next(0, 1), next(0, 1) != 0);
     }
     return 0;
 }

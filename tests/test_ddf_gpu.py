@@ -140,6 +140,36 @@ def test_wide_rows_fp16(case, combine):
     check_against_oracle(*tensors, k, d, s, combine, '', what=str(case))
 
 
+STRIDE2 = [
+    # N, C, H, W: 3x3, stride 2
+    (2, 10, 56, 56),    # four result pixels per lane (fp32), eight (fp16); four strips per plane
+    (2, 7, 28, 28),     # two / four result pixels per lane
+    (3, 9, 14, 14),     # 7 x 7 results: one pixel per lane (fp32)
+    (1, 5, 33, 64),     # odd height: the last feature row is never read
+    (2, 6, 15, 36),     # rows of 18 results, odd height
+    (1, 4, 40, 256),    # 32 lanes per result row: no idle lane between rows
+    (1, 3, 9, 250),     # result rows longer than a wave's lanes: the tile kernels
+    (2, 70, 12, 24),    # more channels than one wave walks
+]
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16], ids=_ids)
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('shape', STRIDE2, ids=_ids)
+def test_stride_two_on_the_row_kernels(shape, combine, dtype):
+    """Stride 2: forward and filter gradients run on the row-register kernels
+    where a result row fits the lanes of a wave and the feature rows keep their
+    vectors aligned; everything against the oracle."""
+    from ddfnet_amd import _lib
+    N, C, H, W = shape
+    if shape in ((2, 10, 56, 56), (2, 7, 28, 28)):
+        assert 'k_rows<' in _lib.describe(shape, 3, 1, 2, combine, dtype) and \
+            'stride 2' in _lib.describe(shape, 3, 1, 2, combine, dtype)
+        assert 'k_rows_filters<' in _lib.describe(shape, 3, 1, 2, combine, dtype, need=7)
+    tensors = random_case(N, C, H, W, 3, 2, dtype, seed=13)
+    check_against_oracle(*tensors, 3, 1, 2, combine, '', what=str(shape))
+
+
 @pytest.mark.parametrize('version', VERSIONS)
 @pytest.mark.parametrize('dtype', [torch.float64, torch.float32], ids=_ids)
 @pytest.mark.parametrize('case', EDGE, ids=_ids)
