@@ -138,33 +138,39 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             }
         }
     };
-    // spatial taps of the lane's pixels (needed for dCF under 'mul' only)
-    uint32_t sfw[MUL ? R : 1][KK][NW];
-    if constexpr (MUL) {
-        const T *sfn = sf + wk.n * KK * plane;
-#pragma unroll
-        for (int t = 0; t < KK; ++t) {
-            const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
-#pragma unroll
-            for (int r = 0; r < R; ++r) load_words<NW>(sr, ob[r], sfw[r][t]);
-        }
-    }
-    // (DX) spatial taps at the pixels the lane's dO values come from: slot (i, j)
+    // Spatial taps of the lane's pixels (sfw: needed for dCF under 'mul' only) and,
+    // with DX, at the pixels the lane's dO values come from: slot (i, j) of sfg
     // holds tap (K-1-i, K-1-j) of the pixel (i-RAD)*D rows and (j-RAD)*D columns
-    // away, zero where that pixel does not exist (see k_rows)
+    // away, zero where that pixel does not exist (see k_rows).  Both come out of
+    // the same window rows of a tap's plane, each loaded once.  (Through the
+    // window offsets a lane that only reads for its neighbours holds real taps in
+    // sfw as well; its dO is masked below, so they enter no sum.)
+    uint32_t sfw[MUL ? R : 1][KK][NW];
     uint32_t sfg[DX ? R : 1][KK][NW];
     if constexpr (DX) {
         const T *sfn = sf + wk.n * KK * plane;
 #pragma unroll
-        for (int i = 0; i < K; ++i)
+        for (int ti = 0; ti < K; ++ti)
 #pragma unroll
-            for (int j = 0; j < K; ++j) {
-                const __amdgpu_buffer_rsrc_t sr =
-                    plane_rsrc(sfn + ((K - 1 - i) * K + (K - 1 - j)) * plane, plane_bytes);
+            for (int tj = 0; tj < K; ++tj) {
+                const int t = ti * K + tj, i = K - 1 - ti, j = K - 1 - tj;
+                const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
+                uint32_t pw[ROWS][NW];
+#pragma unroll
+                for (int rr = 0; rr < ROWS; ++rr) {
+                    const bool for_grad = rr >= i * D && rr < i * D + R;
+                    const bool for_own = MUL && rr >= HY && rr < HY + R;
+                    if (for_grad || for_own) load_words<NW>(sr, xb[rr], pw[rr]);
+                }
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
+                    if constexpr (MUL) {
+#pragma unroll
+                        for (int k = 0; k < NW; ++k) sfw[r][t][k] = pw[HY + r][k];
+                    }
                     Row row;
-                    load_words<NW>(sr, xb[r + i * D], row.own);
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) row.own[k] = pw[r + i * D][k];
                     row.sides(ln.first, ln.last);
                     A v[VX];
 #pragma unroll
@@ -172,6 +178,14 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                     pack<T, VX, A>(v, sfg[r][i * K + j]);
                 }
             }
+    } else if constexpr (MUL) {
+        const T *sfn = sf + wk.n * KK * plane;
+#pragma unroll
+        for (int t = 0; t < KK; ++t) {
+            const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
+#pragma unroll
+            for (int r = 0; r < R; ++r) load_words<NW>(sr, ob[r], sfw[r][t]);
+        }
     }
     // first channels of the walk; then wait for the spatial taps, which were requested
     // before them: a wait inside the walk would drain the channel pipeline every round
