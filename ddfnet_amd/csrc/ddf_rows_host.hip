@@ -55,13 +55,14 @@ void lay_out_lanes(RowsGeom *t, int H, int W, int vx, int R) {
 // Channels per wave of k_rows: enough waves to fill the machine (and to even out
 // its SIMDs), walks long enough to amortise the spatial-filter registers.  The
 // kernels walk whole rounds of `nst` channels, so the count is a multiple of
-// that.  `plane`: pixels of a result plane.
-bool cut_channels_forward(RowsGeom &t, int64_t N, int C, int nst, int64_t plane) {
+// that.  `plane`: pixels of a result plane; `min_walk`: shortest walk worth the
+// prologue (0: two rounds).
+bool cut_channels_forward(RowsGeom &t, int64_t N, int C, int nst, int64_t plane, int min_walk = 0) {
     const int64_t base = N * t.nstrips;
     const int target = tune_int("DDF_TUNE_ROWS_WAVES", 8192);
     const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
     int cpw = (int)(C / want_split);
-    const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", 2 * nst);
+    const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", std::max(2 * nst, (min_walk + nst - 1) / nst * nst));
     cpw = std::max(cpw / nst * nst, min_cpw);
     const int forced = tune_int("DDF_TUNE_ROWS_CPW", 0);
     if (forced) cpw = forced;
@@ -199,7 +200,9 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     t.C = C; t.H = t.Hi = H; t.W = t.Wi = W;
     lay_out_lanes(&t, H, W, vx, R);
 
-    if (!cut_channels_forward(t, p.N, C, p.k == 5 ? 2 : kRowsStages, (int64_t)H * W)) return false;
+    // (25 spatial taps per pixel to load before the walk: 32 pixel-channels per lane at least)
+    if (!cut_channels_forward(t, p.N, C, p.k == 5 ? 2 : kRowsStages, (int64_t)H * W, p.k == 5 ? 32 / vx : 0))
+        return false;
     *g = t;
     *vx_out = vx;
     *r_out = R;
