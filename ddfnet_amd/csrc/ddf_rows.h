@@ -168,6 +168,7 @@ struct LaneStride2 {
     bool first, last;
     int xoff[ROWS];
     int ooff[1];
+    int onext;   // the lane's vector one result row further down (-1: past the last row)
     __host__ __device__ __forceinline__ void init(const RowsGeom &g, int strip, int lane, int = 0) {
         const int grp = magic_div(lane, g.lp_magic);
         const int v = lane - grp * g.lp;
@@ -182,6 +183,7 @@ struct LaneStride2 {
             xoff[rr] = (live && yy >= 0 && yy < g.Hi) ? yy * g.Wi + 2 * x0 : -1;
         }
         ooff[0] = live ? y * g.W + x0 : -1;
+        onext = (live && y + 1 < g.H) ? (y + 1) * g.W + x0 : -1;
     }
 };
 
@@ -248,10 +250,14 @@ __device__ __forceinline__ void store_words_nt(__amdgpu_buffer_rsrc_t rsrc, uint
         v2 v = {w[0], w[1]};
         __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, (int)off, 0, 2);
     } else {
-        static_assert(N == 4, "vectors of 4, 8 or 16 bytes");
+        static_assert(N == 4 || N == 8, "vectors of 4, 8, 16 or 32 bytes");
         typedef uint32_t v4 __attribute__((ext_vector_type(4)));
         v4 v = {w[0], w[1], w[2], w[3]};
         __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, (int)off, 0, 2);
+        if constexpr (N == 8) {
+            v4 u = {w[4], w[5], w[6], w[7]};
+            __builtin_amdgcn_raw_buffer_store_b128(u, rsrc, (int)(off + 16u), 0, 2);
+        }
     }
 }
 

@@ -66,15 +66,17 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RAD = K / 2, HX = RAD * D, HY = RAD * D;
     constexpr int ROWS = R + 2 * HY;
-    constexpr int GROWS = DX ? ROWS : R;       // dO rows a lane loads per channel
-    constexpr int GOWN = DX ? HY : 0;          // its own first row among them
+    // dO rows a lane loads per channel, and its own first row among them (DX:
+    // the whole window; with stride 2 its own row and the next)
+    constexpr int GROWS = DX ? (S == 2 ? 2 : ROWS) : R;
+    constexpr int GOWN = DX && S == 1 ? HY : 0;
     constexpr bool kFilters = MUL || DX;       // CF and SF values are needed at all
     constexpr int NW = VX * sizeof(T) / 4;   // words of a dO / filter vector
     constexpr int NWX = S * NW;              // words of a feature vector
     constexpr int G = kFlushChannels;
     using Row = ExtRow<T, S * VX, HX, PAD>;
     static_assert(G * KK <= kWave, "one lane per (channel, tap) of a flush group");
-    static_assert(S == 1 || (S == 2 && K == 3 && D == 1 && R == 1 && !DX), "stride 2: 3 x 3, filters only");
+    static_assert(S == 1 || (S == 2 && K == 3 && D == 1 && R == 1), "stride 2: 3 x 3, one row per lane");
     extern __shared__ __align__(16) unsigned char smem[];
 
     const int lane = threadIdx.x & (kWave - 1);
@@ -98,7 +100,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     const int64_t xn = x_mod ? wk.n % x_mod : wk.n;
     const T *xs = x + (xn * g.C + c_first) * xplane;
     const T *gs = go + (wk.n * g.C + c_first) * plane;
-    T *ds = DX ? dx + (wk.n * g.C + c_first) * plane : nullptr;
+    T *ds = DX ? dx + (wk.n * g.C + c_first) * xplane : nullptr;
     uint32_t xb[ROWS], ob[R];
 #pragma unroll
     for (int rr = 0; rr < ROWS; ++rr)
@@ -106,6 +108,15 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
     for (int r = 0; r < R; ++r)
         ob[r] = ln.ooff[r] < 0 ? kOutside : (uint32_t)ln.ooff[r] * (uint32_t)sizeof(T);
+    // where the lane's dO rows are
+    uint32_t gb[GROWS];
+    if constexpr (DX && S == 2) {
+        gb[0] = ob[0];
+        gb[1] = ln.onext < 0 ? kOutside : (uint32_t)ln.onext * (uint32_t)sizeof(T);
+    } else {
+#pragma unroll
+        for (int r = 0; r < GROWS; ++r) gb[r] = DX ? xb[r] : ob[r];
+    }
     const int tl = lane < KK ? lane : KK - 1;
     const T *cfs = cf + (wk.n * g.C + c_first) * KK;
 
@@ -127,7 +138,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             if (row_needed<R, K, D>(rr)) load_words<NWX>(pr, xb[rr], xw[ST][rr]);
 #pragma unroll
         for (int r = 0; r < GROWS; ++r)
-            if (!DX || row_needed<R, K, D>(r)) load_words<NW>(gr, DX ? xb[r] : ob[r], gw[ST][r]);
+            if (!DX || S == 2 || row_needed<R, K, D>(r)) load_words<NW>(gr, gb[r], gw[ST][r]);
         if constexpr (kFilters) {
             const int cc = ci < nch ? ci : (nch > 0 ? nch - 1 : 0);
             if constexpr (kScalarTaps) {
@@ -147,7 +158,44 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     // sfw as well; its dO is masked below, so they enter no sum.)
     uint32_t sfw[MUL ? R : 1][KK][NW];
     uint32_t sfg[DX ? R : 1][KK][NW];
-    if constexpr (DX) {
+    if constexpr (DX && S == 2) {
+        // Stride 2: result pixel (y, x) reaches feature pixel (2y + i - 1, 2x + j - 1)
+        // through tap (i, j).  Seen from the lane's 2 x 2 VX block of feature pixels
+        // (rows 2y and 2y + 1), tap row 0 belongs to the result row below and tap
+        // column 0 to the result pixel to the right: slot (i, j) holds that pixel's tap.
+        using SRow = ExtRow<T, VX, 1, PAD>;
+        const T *sfn = sf + wk.n * KK * plane;
+#pragma unroll
+        for (int i = 0; i < K; ++i)
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                const int t = i * K + j;
+                const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
+                uint32_t own[NW];
+                if (MUL || i > 0) load_words<NW>(sr, gb[0], own);
+                if constexpr (MUL) {
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) sfw[0][t][k] = own[k];
+                }
+                SRow row;
+                if (i == 0) {
+                    load_words<NW>(sr, gb[1], row.own);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) row.own[k] = own[k];
+                }
+                if (j == 0) {
+                    row.sides(ln.first, ln.last);
+                    A v[VX];
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) v[e] = row.at(e + 1);
+                    pack<T, VX, A>(v, sfg[0][t]);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) sfg[0][t][k] = row.own[k];
+                }
+            }
+    } else if constexpr (DX) {
         const T *sfn = sf + wk.n * KK * plane;
 #pragma unroll
         for (int ti = 0; ti < K; ++ti)
@@ -314,7 +362,45 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             for (int t = 0; t < KK; ++t)
 #pragma unroll
                 for (int e = 0; e < VX; ++e) asm volatile("" : "+v"(acc_sf[r][t][e]));
-        if constexpr (DX) {
+        if constexpr (DX && S == 2) {
+            // feature gradient of the lane's two feature rows: the four parity classes
+            // of a feature pixel see one, two, two and four taps
+            using GRow = ExtRow<T, VX, 1, PAD>;
+            GRow g0, g1;
+#pragma unroll
+            for (int k = 0; k < NW; ++k) { g0.own[k] = gw[ST][0][k]; g1.own[k] = gw[ST][1][k]; }
+            g0.sides(ln.first, ln.last);
+            g1.sides(ln.first, ln.last);
+            // dO * comb(CF[i][j], SF[i][j]) with the spatial tap of slot (i, j)
+            auto term = [&](A gv, int i, int j, int e, A acc) __attribute__((always_inline)) {
+                const int t = i * K + j;
+                const A sv = elem<T>(sfg[0][t], e);
+                if constexpr (MUL) return fma_(w[t], fma_(gv, sv, A(0)), acc);
+                else return fma_(gv, sv, fma_(gv, w[t], acc));
+            };
+            A top[2 * VX], bot[2 * VX];
+#pragma unroll
+            for (int e = 0; e < VX; ++e) {
+                const A g00 = g0.at(e), g01 = g0.at(e + 1), g10 = g1.at(e), g11 = g1.at(e + 1);
+                top[2 * e] = term(g00, 1, 1, e, A(0));
+                top[2 * e + 1] = term(g00, 1, 2, e, term(g01, 1, 0, e, A(0)));
+                bot[2 * e] = term(g00, 2, 1, e, term(g10, 0, 1, e, A(0)));
+                bot[2 * e + 1] = term(g00, 2, 2, e, term(g01, 2, 0, e, term(g10, 0, 2, e, term(g11, 0, 0, e, A(0)))));
+            }
+            const __amdgpu_buffer_rsrc_t dr = plane_rsrc(ds + (int64_t)ci * xplane, ci < nch ? xplane_bytes : 0u);
+            if constexpr (sizeof(T) == 2) {
+#pragma unroll
+                for (int e = 0; e < 2 * VX; ++e) {
+                    asm volatile("" : "+v"(top[e]));
+                    asm volatile("" : "+v"(bot[e]));
+                }
+            }
+            uint32_t ow[NWX];
+            pack<T, 2 * VX, A>(top, ow);
+            store_words_nt<NWX>(dr, xb[1], ow);
+            pack<T, 2 * VX, A>(bot, ow);
+            store_words_nt<NWX>(dr, xb[2], ow);
+        } else if constexpr (DX) {
             // feature gradient of the lane's pixels: dO at the flipped tap offsets
             Row grow[ROWS];
 #pragma unroll

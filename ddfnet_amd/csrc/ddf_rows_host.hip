@@ -118,8 +118,8 @@ bool cut_channels_filters(RowsGeom &t, int64_t N, int C) {
 // the feature plane must keep those vectors aligned (W a multiple of 2 * vx) and
 // a result row must fit the lanes of a wave.  filters: the cut of
 // k_rows_filters, else of k_rows.
-bool stride2_geometry(const Problem &p, int dtype, bool filters, RowsGeom *g, int *vx_out,
-                      int *r_out) {
+bool stride2_geometry(const Problem &p, int dtype, bool filters, int max_vx, RowsGeom *g,
+                      int *vx_out, int *r_out) {
     if (!(p.s == 2 && p.k == 3 && p.d == 1)) return false;
     if (dtype != DDF_F16 && dtype != DDF_F32) return false;
     if (p.N <= 0 || p.C <= 0 || p.Ho <= 0 || p.Wo <= 0) return false;
@@ -129,7 +129,7 @@ bool stride2_geometry(const Problem &p, int dtype, bool filters, RowsGeom *g, in
     if ((int64_t)H * W * 8 >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
     int vx = 0;
     for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
-        if (cand > tune_int("DDF_TUNE_ROWS_VX", 16)) continue;
+        if (cand > tune_int("DDF_TUNE_ROWS_VX", 16) || cand > max_vx) continue;
         if (W % (2 * cand) != 0) continue;
         vx = cand;
         break;
@@ -163,7 +163,7 @@ bool rows_shape_built(int k, int d, int s) {
 
 bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx_out, int *r_out) {
     if (!rows_shape_built(p.k, p.d, p.s)) return false;
-    if (p.s == 2) return max_vx <= 0 && stride2_geometry(p, dtype, false, g, vx_out, r_out);
+    if (p.s == 2) return max_vx <= 0 && stride2_geometry(p, dtype, false, 16, g, vx_out, r_out);
     if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
     if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;
     const int esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
@@ -220,7 +220,11 @@ bool rows_filters_variant_built(int esz, int vx, int r, bool fused) {
 
 bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g, int *vx_out,
                            int *r_out) {
-    if (p.s == 2) return !fused && stride2_geometry(p, dtype, true, g, vx_out, r_out);
+    // (stride 2, one launch for the whole backward pass: every feature row must be some
+    // lane's 2y or 2y + 1, so the height is even; the width already is)
+    if (p.s == 2)
+        return (!fused || (p.H % 2 == 0 && tune_int("DDF_TUNE_ROWSF_FUSED", 1) != 0)) &&
+               stride2_geometry(p, dtype, true, fused ? 4 : 16, g, vx_out, r_out);   // (registers)
     if (!(p.s == 1 && p.k == 3 && (p.d == 1 || p.d == 2))) return false;
     if (p.N <= 0 || p.C <= 0 || p.H <= 0 || p.W <= 0) return false;
     if (p.H > 16384 || p.W > 16384 || p.C > (1 << 24) || p.N > (1 << 24)) return false;

@@ -170,22 +170,22 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
     return hipGetLastError();
 }
 
-// Stride 2: filter gradients (the feature gradient is a launch of its own).
-template <typename T, int VX>
+// Stride 2: filter gradients and, with DX, the feature gradient in the same launch.
+template <typename T, int VX, bool DX>
 hipError_t launch_filters_stride2_v(const Problem &p, const RowsGeom &g, const T *go, const T *x,
-                                    const T *cf, const T *sf, T *dcf, T *dsf,
+                                    const T *cf, const T *sf, T *dx, T *dcf, T *dsf,
                                     typename Acc<T>::type *ws_sf, typename Acc<T>::type *ws_cf,
                                     unsigned need, hipStream_t st) {
     using A = typename Acc<T>::type;
-    // (channels in flight per wave: 32-byte feature vectors of fp16 leave room for two)
-    constexpr int kStagesS2 = sizeof(T) == 2 && VX >= 8 ? 2 : 4, kWpe = 2;
+    // (channels in flight per wave: 32-byte feature vectors of fp16 leave room for two,
+    // and so does the second set of spatial taps of the feature gradient)
+    constexpr int kStagesS2 = DX || (sizeof(T) == 2 && VX >= 8) ? 2 : 4, kWpe = 2;
     const dim3 grid(g.xcd_per * kXcd), block(kWave * kFilterWaves);
     const int lds = filters_lds_bytes<9>((int)sizeof(A), 1, VX);
     const bool pad = rows_shift_in_as_is(g);
 #define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
-    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, 1, PAD_, false, kStagesS2, kWpe, 2>),  \
-                       grid, block, lds, st, g, go, x, cf, sf, (T *)nullptr, dcf, dsf, ws_sf,    \
-                       ws_cf, need, 0)
+    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, 1, PAD_, DX, kStagesS2, kWpe, 2>),     \
+                       grid, block, lds, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, 0)
     if (p.mul) {
         if (pad) DDF_ROWSF_CASE(true, true);
         else DDF_ROWSF_CASE(true, false);
@@ -259,7 +259,8 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
     if ((((uintptr_t)x | (uintptr_t)go | (uintptr_t)sf | (uintptr_t)dsf | (uintptr_t)dx) & mask) != 0)
         return hipErrorNotSupported;
-    if (p.s == 2 && (x_mod != 0 || ((uintptr_t)x & (std::min<uintptr_t>(2 * vx * sizeof(T), 16) - 1)) != 0))
+    if (p.s == 2 && (x_mod != 0 || (((uintptr_t)x | (uintptr_t)dx) &
+                                    (std::min<uintptr_t>(2 * vx * sizeof(T), 16) - 1)) != 0))
         return hipErrorNotSupported;
     unsigned char *wp = static_cast<unsigned char *>(ws);
     A *ws_sf = nullptr, *ws_cf = nullptr;
@@ -272,17 +273,21 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     hipError_t err = hipErrorNotSupported;
     if constexpr (sizeof(T) != 8) {
         if (p.s == 2) {
-            if (vx == 4)
-                err = rows::launch_filters_stride2_v<T, 4>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
-            else if (vx == 2)
-                err = rows::launch_filters_stride2_v<T, 2>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+#define DDF_S2_CASE(VX_)                                                                          \
+    err = fused ? rows::launch_filters_stride2_v<T, VX_, true>(p, g, go, x, cf, sf, dx, dcf, dsf, \
+                                                               ws_sf, ws_cf, need, st)            \
+                : rows::launch_filters_stride2_v<T, VX_, false>(p, g, go, x, cf, sf, dx, dcf, dsf, \
+                                                                ws_sf, ws_cf, need, st)
+            if (vx == 4) DDF_S2_CASE(4);
+            else if (vx == 2) DDF_S2_CASE(2);
             if constexpr (sizeof(T) == 2) {
-                if (vx == 8)
-                    err = rows::launch_filters_stride2_v<T, 8>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+                if (vx == 8 && !fused)
+                    err = rows::launch_filters_stride2_v<T, 8, false>(p, g, go, x, cf, sf, dx, dcf, dsf,
+                                                                      ws_sf, ws_cf, need, st);
             } else {
-                if (vx == 1)
-                    err = rows::launch_filters_stride2_v<T, 1>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, st);
+                if (vx == 1) DDF_S2_CASE(1);
             }
+#undef DDF_S2_CASE
         } else if (taprow) {
             if (vx == 4)
                 err = rows::launch_taprow_v<T, 4>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);

@@ -360,9 +360,10 @@ static void replay_rows_stride2(const RowsGeom &g, long N, long C, int esz, bool
             }
             if (live) {
                 CHECK(ln.ooff[0] == y * g.W + x0, "result offset");
+                CHECK(ln.onext == (y + 1 < g.H ? (y + 1) * g.W + x0 : -1), "next result row");
                 for (int e = 0; e < VX; ++e) ++owner[ln.ooff[0] + e];
             } else {
-                CHECK(ln.ooff[0] < 0, "idle lane %d writes", lane);
+                CHECK(ln.ooff[0] < 0 && ln.onext < 0, "idle lane %d writes", lane);
             }
             CHECK(ln.first == (v == 0) && ln.last == (v == g.lpr - 1), "row ends");
         }
@@ -387,7 +388,8 @@ static void check_rows_stride2(long N, long C, long H, long W, int dtype, bool f
     const int esz = dtype == 0 ? 2 : 4;
     CHECK(dtype != 2 && r == 1, "stride 2 variant");
     CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4, "vector of %d bytes", vx * esz);
-    CHECK(!rows_filters_geometry(p, dtype, true, &g, &vx, &r), "no one-launch backward with stride 2");
+    // (the one-launch backward writes feature rows 2y and 2y + 1 of every result row y)
+    CHECK(rows_filters_geometry(p, dtype, true, &g, &vx, &r) == (H % 2 == 0), "one-launch backward with stride 2");
     (filters ? rows_filters_geometry(p, dtype, false, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r));
     if (filters) {
         CHECK(rows::filters_lds_bytes<9>(4, 1, vx) <= 64 * 1024, "filter kernel LDS");
