@@ -168,6 +168,16 @@ def test_stride_two_on_the_row_kernels(shape, combine, dtype):
         assert 'k_rows_filters<' in _lib.describe(shape, 3, 1, 2, combine, dtype, need=7)
     tensors = random_case(N, C, H, W, 3, 2, dtype, seed=13)
     check_against_oracle(*tensors, 3, 1, 2, combine, '', what=str(shape))
+    # all gradients together come from one launch where the height is even; asked for
+    # separately, the feature gradient is the tile kernel's: the routes agree to rounding
+    x, cf, sf, go = tensors
+    together = run_ddf(x, cf, sf, go, 3, 1, 2, combine)
+    only_dx = run_ddf(x, cf, sf, go, 3, 1, 2, combine, need=(True, False, False))
+    only_filters = run_ddf(x, cf, sf, go, 3, 1, 2, combine, need=(False, True, True))
+    tol = 1e-6 if dtype == torch.float32 else 2e-3
+    assert rel_err(only_dx[1], together[1].cpu()) <= tol
+    assert rel_err(only_filters[2], together[2].cpu()) <= tol
+    assert rel_err(only_filters[3], together[3].cpu()) <= tol
 
 
 @pytest.mark.parametrize('version', VERSIONS)
