@@ -372,12 +372,14 @@ static void replay_rows_stride2(const RowsGeom &g, long N, long C, int esz, bool
     check_work_items(g, N, C, filters ? 1 : 0, 0);
 }
 
-static void check_rows_stride2(long N, long C, long H, long W, int dtype, bool filters) {
+// fused: the cut of the launch that also writes the feature gradient (rows 2y and 2y + 1
+// of the feature plane from the lane of result row y: even heights only).
+static void check_rows_stride2(long N, long C, long H, long W, int dtype, bool filters, bool fused = false) {
     const Problem p = make_problem(N, C, H, W, 3, 1, 2, 0);
     RowsGeom g;
     int vx, r;
-    const bool ok = filters ? rows_filters_geometry(p, dtype, false, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r);
-    const char *name = filters ? "-filters" : "";
+    const bool ok = filters ? rows_filters_geometry(p, dtype, fused, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r);
+    const char *name = fused ? "-filters+dX" : filters ? "-filters" : "";
     if (!ok) {
         printf("kind rows%s stride 2 %ldx%ldx%ldx%ld dt%d: unsupported\n", name, N, C, H, W, dtype);
         return;
@@ -388,9 +390,7 @@ static void check_rows_stride2(long N, long C, long H, long W, int dtype, bool f
     const int esz = dtype == 0 ? 2 : 4;
     CHECK(dtype != 2 && r == 1, "stride 2 variant");
     CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4, "vector of %d bytes", vx * esz);
-    // (the one-launch backward writes feature rows 2y and 2y + 1 of every result row y)
-    CHECK(rows_filters_geometry(p, dtype, true, &g, &vx, &r) == (H % 2 == 0), "one-launch backward with stride 2");
-    (filters ? rows_filters_geometry(p, dtype, false, &g, &vx, &r) : rows_geometry(p, dtype, 0, &g, &vx, &r));
+    if (fused) CHECK(H % 2 == 0 && g.Hi == 2 * g.H && g.Wi == 2 * g.W, "one-launch backward leaves feature rows unwritten");
     if (filters) {
         CHECK(rows::filters_lds_bytes<9>(4, 1, vx) <= 64 * 1024, "filter kernel LDS");
         CHECK(g.cpw % rows::kFlushChannels == 0, "channels per wave %d not whole flush groups", g.cpw);
@@ -434,8 +434,8 @@ int main() {
             }
     for (auto &sh : shapes)
         for (int dtype = 0; dtype < 3; ++dtype)
-            for (int filters = 0; filters < 2; ++filters)
-                check_rows_stride2(sh[0], sh[1], sh[2], sh[3], dtype, filters != 0);
+            for (int filters = 0; filters < 3; ++filters)
+                check_rows_stride2(sh[0], sh[1], sh[2], sh[3], dtype, filters != 0, filters == 2);
     // seeded random shapes on top of the fixed list
     unsigned long long state = 0x9E3779B97F4A7C15ull;
     auto next = [&](int lo, int hi) {
@@ -455,6 +455,7 @@ int main() {
         check_rows(N, C, H, (W / 4 + 1) * 4, 5, next(1, 2), next(0, 1), true, false, true);
         check_rows_stride2(N, C, H + 1, (W / 4 + 1) * 4, next(0, 1), next(0, 1) != 0);
         check_rows_stride2(N, C, H + 1, (W / 16 + 1) * 16, next(0, 1), next(0, 1) != 0);
+        check_rows_stride2(N, C, H + 1, (W / 16 + 1) * 16, next(0, 1), true, true);
     }
     return 0;
 }
