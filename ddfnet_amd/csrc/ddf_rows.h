@@ -261,6 +261,22 @@ __device__ __forceinline__ void store_words_nt(__amdgpu_buffer_rsrc_t rsrc, uint
     }
 }
 
+// A lane's vector of BYTES bytes (2: one fp16 element, kept in the low half of a
+// word) <-> 32-bit words.
+constexpr int vec_words(int bytes) { return bytes >= 4 ? bytes / 4 : 1; }
+template <int BYTES>
+__device__ __forceinline__ void load_vec(__amdgpu_buffer_rsrc_t rsrc, uint32_t off,
+                                         uint32_t (&w)[vec_words(BYTES)]) {
+    if constexpr (BYTES == 2) w[0] = (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rsrc, (int)off, 0, 0);
+    else load_words<BYTES / 4>(rsrc, off, w);
+}
+template <int BYTES>
+__device__ __forceinline__ void store_vec_nt(__amdgpu_buffer_rsrc_t rsrc, uint32_t off,
+                                             const uint32_t (&w)[vec_words(BYTES)]) {
+    if constexpr (BYTES == 2) __builtin_amdgcn_raw_buffer_store_b16((short)w[0], rsrc, (int)off, 0, 2);
+    else store_words_nt<BYTES / 4>(rsrc, off, w);
+}
+
 // One accumulator-type value, rounded to the storage type, to byte offset off
 // of the buffer.
 template <typename T>
@@ -296,8 +312,11 @@ __device__ __forceinline__ typename Acc<T>::type elem(const uint32_t *w, int e) 
 
 // VX accumulator-type values -> storage-type words (round to nearest even).
 template <typename T, int VX, typename A>
-__device__ __forceinline__ void pack(const A (&v)[VX], uint32_t (&w)[VX * sizeof(T) / 4]) {
-    if constexpr (sizeof(T) == 2) {
+__device__ __forceinline__ void pack(const A (&v)[VX], uint32_t (&w)[vec_words(VX * sizeof(T))]) {
+    if constexpr (sizeof(T) == 2 && VX == 1) {
+        const _Float16 h = (_Float16)v[0];
+        w[0] = (uint32_t)__builtin_bit_cast(unsigned short, h);
+    } else if constexpr (sizeof(T) == 2) {
 #pragma unroll
         for (int k = 0; k < VX / 2; ++k) {
             half2_t h;
@@ -336,7 +355,7 @@ __device__ __forceinline__ double fma_(double a, double b, double c) { return __
 template <typename T, int VX, int HX, bool PAD>
 struct ExtRow {
     using A = typename Acc<T>::type;
-    static constexpr int NW = VX * sizeof(T) / 4;
+    static constexpr int NW = vec_words(VX * sizeof(T));
     static constexpr int SW = HX == 0 ? 1 : (HX * sizeof(T) + 3) / 4;   // words taken from each neighbour
     static constexpr int kLeftFirst = (NW - SW) * 4 / (int)sizeof(T);   // neighbour element in left[0]
     static_assert(HX <= VX, "taps reach beyond the neighbouring lane");
@@ -386,8 +405,8 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
     using A = typename Acc<T>::type;
     constexpr int KK = K * K, RAD = K / 2, HX = RAD * D, HY = RAD * D;
     constexpr int ROWS = R + 2 * HY;
-    constexpr int NW = VX * sizeof(T) / 4;   // words of a result vector
-    constexpr int NWX = S * NW;              // words of a feature vector
+    constexpr int kVB = VX * sizeof(T), kXB = S * kVB;   // bytes of a result / feature vector
+    constexpr int NW = vec_words(kVB), NWX = vec_words(kXB);
     using Row = ExtRow<T, S * VX, HX, PAD>;
     static_assert(KK <= kWave, "one lane per channel-filter tap");
     static_assert(S == 1 || (S == 2 && K == 3 && D == 1 && R == 1 && !BWD), "stride 2: forward, 3 x 3");
@@ -431,7 +450,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
             for (int t = 0; t < KK; ++t) {
                 const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
 #pragma unroll
-                for (int r = 0; r < R; ++r) load_words<NW>(sr, ob[r], sfw[r][t]);
+                for (int r = 0; r < R; ++r) load_vec<kVB>(sr, ob[r], sfw[r][t]);
             }
         } else {
 #pragma unroll
@@ -443,7 +462,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
 #pragma unroll
                     for (int r = 0; r < R; ++r) {
                         Row row;
-                        load_words<NW>(sr, xb[r + i * D], row.own);
+                        load_vec<kVB>(sr, xb[r + i * D], row.own);
                         row.sides(ln.first, ln.last);
                         A v[VX];
 #pragma unroll
@@ -464,7 +483,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
         const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * xplane, ci < nch ? xplane_bytes : 0u);
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr)
-            if (row_needed<R, K, D>(rr)) load_words<NWX>(pr, xb[rr], xw[ST][rr]);
+            if (row_needed<R, K, D>(rr)) load_vec<kXB>(pr, xb[rr], xw[ST][rr]);
         const int cc = ci < nch ? ci : nch - 1;   // (the taps are read through plain pointers: stay inside)
         if constexpr (kScalarTaps) {
 #pragma unroll
@@ -554,7 +573,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
             }
             uint32_t ow[NW];
             pack<T, VX, A>(acc[r], ow);
-            store_words_nt<NW>(orr, ob[r], ow);
+            store_vec_nt<kVB>(orr, ob[r], ow);
         }
     };
 

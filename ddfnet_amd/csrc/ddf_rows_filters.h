@@ -71,8 +71,8 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     constexpr int GROWS = DX ? (S == 2 ? 2 : ROWS) : R;
     constexpr int GOWN = DX && S == 1 ? HY : 0;
     constexpr bool kFilters = MUL || DX;       // CF and SF values are needed at all
-    constexpr int NW = VX * sizeof(T) / 4;   // words of a dO / filter vector
-    constexpr int NWX = S * NW;              // words of a feature vector
+    constexpr int kVB = VX * sizeof(T), kXB = S * kVB;   // bytes of a dO / filter vector, of a feature vector
+    constexpr int NW = vec_words(kVB), NWX = vec_words(kXB);
     constexpr int G = kFlushChannels;
     using Row = ExtRow<T, S * VX, HX, PAD>;
     static_assert(G * KK <= kWave, "one lane per (channel, tap) of a flush group");
@@ -135,10 +135,10 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
         // (with dilation the window has rows no tap lands on: see row_needed)
 #pragma unroll
         for (int rr = 0; rr < ROWS; ++rr)
-            if (row_needed<R, K, D>(rr)) load_words<NWX>(pr, xb[rr], xw[ST][rr]);
+            if (row_needed<R, K, D>(rr)) load_vec<kXB>(pr, xb[rr], xw[ST][rr]);
 #pragma unroll
         for (int r = 0; r < GROWS; ++r)
-            if (!DX || S == 2 || row_needed<R, K, D>(r)) load_words<NW>(gr, gb[r], gw[ST][r]);
+            if (!DX || S == 2 || row_needed<R, K, D>(r)) load_vec<kVB>(gr, gb[r], gw[ST][r]);
         if constexpr (kFilters) {
             const int cc = ci < nch ? ci : (nch > 0 ? nch - 1 : 0);
             if constexpr (kScalarTaps) {
@@ -172,14 +172,14 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                 const int t = i * K + j;
                 const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
                 uint32_t own[NW];
-                if (MUL || i > 0) load_words<NW>(sr, gb[0], own);
+                if (MUL || i > 0) load_vec<kVB>(sr, gb[0], own);
                 if constexpr (MUL) {
 #pragma unroll
                     for (int k = 0; k < NW; ++k) sfw[0][t][k] = own[k];
                 }
                 SRow row;
                 if (i == 0) {
-                    load_words<NW>(sr, gb[1], row.own);
+                    load_vec<kVB>(sr, gb[1], row.own);
                 } else {
 #pragma unroll
                     for (int k = 0; k < NW; ++k) row.own[k] = own[k];
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                 for (int rr = 0; rr < ROWS; ++rr) {
                     const bool for_grad = rr >= i * D && rr < i * D + R;
                     const bool for_own = MUL && rr >= HY && rr < HY + R;
-                    if (for_grad || for_own) load_words<NW>(sr, xb[rr], pw[rr]);
+                    if (for_grad || for_own) load_vec<kVB>(sr, xb[rr], pw[rr]);
                 }
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
         for (int t = 0; t < KK; ++t) {
             const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
 #pragma unroll
-            for (int r = 0; r < R; ++r) load_words<NW>(sr, ob[r], sfw[r][t]);
+            for (int r = 0; r < R; ++r) load_vec<kVB>(sr, ob[r], sfw[r][t]);
         }
     }
     // first channels of the walk; then wait for the spatial taps, which were requested
@@ -397,9 +397,9 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             }
             uint32_t ow[NWX];
             pack<T, 2 * VX, A>(top, ow);
-            store_words_nt<NWX>(dr, xb[1], ow);
+            store_vec_nt<kXB>(dr, xb[1], ow);
             pack<T, 2 * VX, A>(bot, ow);
-            store_words_nt<NWX>(dr, xb[2], ow);
+            store_vec_nt<kXB>(dr, xb[2], ow);
         } else if constexpr (DX) {
             // feature gradient of the lane's pixels: dO at the flipped tap offsets
             Row grow[ROWS];
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                 }
                 uint32_t ow[NW];
                 pack<T, VX, A>(accx, ow);
-                store_words_nt<NW>(dr, ob[r], ow);
+                store_vec_nt<kVB>(dr, ob[r], ow);
             }
         }
         if (want_cf && ci < nch) {
@@ -502,7 +502,7 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
             if (g.csplit == 1) {
                 uint32_t ow[NW];
                 pack<T, VX, A>(tot, ow);
-                store_words_nt<NW>(plane_rsrc(dsf + (wk.n * KK + t) * plane, plane_bytes), off_r, ow);
+                store_vec_nt<kVB>(plane_rsrc(dsf + (wk.n * KK + t) * plane, plane_bytes), off_r, ow);
             } else {
                 // partial sums in the accumulator type, same plane shape
                 constexpr int AW = VX * sizeof(A) / 4;

@@ -128,7 +128,7 @@ bool stride2_geometry(const Problem &p, int dtype, bool filters, int max_vx, Row
     const int H = (int)p.H, W = (int)p.W, Ho = (int)p.Ho, Wo = (int)p.Wo, C = (int)p.C;
     if ((int64_t)H * W * 8 >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
     int vx = 0;
-    for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
+    for (int cand = 16 / esz; cand >= 1; cand /= 2) {
         if (cand > tune_int("DDF_TUNE_ROWS_VX", 16) || cand > max_vx) continue;
         if (W % (2 * cand) != 0) continue;
         vx = cand;
@@ -151,7 +151,7 @@ bool stride2_geometry(const Problem &p, int dtype, bool filters, int max_vx, Row
 
 // Instantiated (elements per lane and row, rows per lane) per element size.
 bool rows_variant_built(int esz, int vx, int r) {
-    if (esz == 2) return (r == 1 && (vx == 8 || vx == 4 || vx == 2)) || (r == 2 && vx == 8);
+    if (esz == 2) return (r == 1 && (vx == 8 || vx == 4 || vx == 2 || vx == 1)) || (r == 2 && vx == 8);
     if (esz == 4) return (r == 1 && (vx == 4 || vx == 2 || vx == 1)) || (r == 2 && (vx == 2 || vx == 4));
     return false;
 }
@@ -172,7 +172,7 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
     if ((int64_t)H * W * esz >= (1ll << 31)) return false;   // byte offsets inside a plane are 32-bit
     // widest vector the row length allows, at most 32 lanes per image row
     int vx = 0;
-    for (int cand = 16 / esz; cand * esz >= 4; cand /= 2) {
+    for (int cand = 16 / esz; cand >= 1; cand /= 2) {
         if (max_vx > 0 && cand > max_vx) continue;
         if (cand > tune_int("DDF_TUNE_ROWS_VX", 16)) continue;
         if (W % cand != 0 || cand < hx) continue;
@@ -213,7 +213,7 @@ bool rows_geometry(const Problem &p, int dtype, int max_vx, RowsGeom *g, int *vx
 // fused: of the variant that also writes the feature gradient.
 bool rows_filters_variant_built(int esz, int vx, int r, bool fused) {
     if (esz != 2 && esz != 4) return false;
-    if (vx == 1) return esz == 4 && r == 1;   // odd row lengths, fp32: one pixel per lane
+    if (vx == 1) return r == 1;   // odd row lengths: one pixel per lane
     if (fused) return (vx == 2 && r == 2) || (vx == 4 && r == 1);
     return r == 1 && (vx == 4 || vx == 2);
 }
@@ -238,7 +238,7 @@ bool rows_filters_geometry(const Problem &p, int dtype, bool fused, RowsGeom *g,
                   tune_int("DDF_TUNE_ROWSF_FUSED", 1) == 0))
         return false;
     int vx = 0, R = 1;
-    for (int cand = std::min(16 / esz, 4); cand * esz >= 4; cand /= 2) {
+    for (int cand = std::min(16 / esz, 4); cand >= 1; cand /= 2) {
         if (cand > tune_int("DDF_TUNE_ROWSF_VX", 16)) continue;
         if (W % cand != 0 || cand < hx) continue;
         // two rows per lane where a row is a few 2-pixel vectors (14 x 14: one strip per plane)

@@ -106,10 +106,8 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
         if constexpr (sizeof(T) == 2) {
             if (vx == 8) return rows::launch_stride2_v<T, 8>(p, g, x, cf, sf, out, st);
         }
-        if constexpr (sizeof(T) == 4) {
-            if (vx == 1) return rows::launch_stride2_v<T, 1>(p, g, x, cf, sf, out, st);
-        }
         if constexpr (sizeof(T) != 8) {
+            if (vx == 1) return rows::launch_stride2_v<T, 1>(p, g, x, cf, sf, out, st);
             if (vx == 4) return rows::launch_stride2_v<T, 4>(p, g, x, cf, sf, out, st);
             if (vx == 2) return rows::launch_stride2_v<T, 2>(p, g, x, cf, sf, out, st);
         }
@@ -119,6 +117,7 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
         if (vx == 8 && r == 1) return rows::launch_v<T, 8, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 4 && r == 1) return rows::launch_v<T, 4, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 1 && r == 1) return rows::launch_v<T, 1, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 8 && r == 2) return rows::launch_v<T, 8, 2>(p, g, backward, x, cf, sf, out, st);
     } else if constexpr (sizeof(T) == 4) {
         if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
@@ -280,12 +279,11 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
                                                                 ws_sf, ws_cf, need, st)
             if (vx == 4) DDF_S2_CASE(4);
             else if (vx == 2) DDF_S2_CASE(2);
+            else if (vx == 1) DDF_S2_CASE(1);
             if constexpr (sizeof(T) == 2) {
                 if (vx == 8 && !fused)
                     err = rows::launch_filters_stride2_v<T, 8, false>(p, g, go, x, cf, sf, dx, dcf, dsf,
                                                                       ws_sf, ws_cf, need, st);
-            } else {
-                if (vx == 1) DDF_S2_CASE(1);
             }
 #undef DDF_S2_CASE
         } else if (taprow) {
@@ -298,12 +296,10 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
                     err = rows::launch_taprow_v<T, 8>(p, g, go, x, cf, sf, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
             }
         } else if (vx == 1) {
-            if constexpr (sizeof(T) == 4) {
-                if (fused)
-                    err = rows::launch_filters_v<T, 1, 1, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
-                else
-                    err = rows::launch_filters_v<T, 1, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
-            }
+            if (fused)
+                err = rows::launch_filters_v<T, 1, 1, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
+            else
+                err = rows::launch_filters_v<T, 1, 1, false>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);
         } else if (fused) {
             if (vx == 2 && r == 2)
                 err = rows::launch_filters_v<T, 2, 2, true>(p, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod, st);

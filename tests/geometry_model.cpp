@@ -312,7 +312,7 @@ static void check_rows(long N, long C, long H, long W, int k, int d, int dtype, 
         return;
     }
     const int esz = dtype == 0 ? 2 : dtype == 1 ? 4 : 8;
-    CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4, "vector of %d bytes", vx * esz);
+    CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4 || vx * esz == 2, "vector of %d bytes", vx * esz);
     CHECK((k / 2) * d <= vx, "taps reach beyond the neighbouring lane");
     CHECK((long)H * W * 8 < (1l << 31), "plane beyond 32-bit byte offsets");
     if (filters) {
@@ -389,7 +389,7 @@ static void check_rows_stride2(long N, long C, long H, long W, int dtype, bool f
            g.cpw, g.cpb, g.csplit, g.wpb, g.nwork);
     const int esz = dtype == 0 ? 2 : 4;
     CHECK(dtype != 2 && r == 1, "stride 2 variant");
-    CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4, "vector of %d bytes", vx * esz);
+    CHECK(vx * esz == 16 || vx * esz == 8 || vx * esz == 4 || vx * esz == 2, "vector of %d bytes", vx * esz);
     if (fused) CHECK(H % 2 == 0 && g.Hi == 2 * g.H && g.Wi == 2 * g.W, "one-launch backward leaves feature rows unwritten");
     if (filters) {
         CHECK(rows::filters_lds_bytes<9>(4, 1, vx) <= 64 * 1024, "filter kernel LDS");

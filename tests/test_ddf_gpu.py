@@ -569,6 +569,28 @@ def test_tiny_planes(N, C, H, W, d, combine, dtype):
     check_against_oracle(*case, 3, d, 1, combine, 'f', what='tiny plane, tiled forced')
 
 
+@pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('N,C,H,W,s', [
+    (3, 37, 7, 7, 1), (2, 20, 15, 15, 1), (1, 9, 6, 31, 1), (2, 6, 33, 57, 1),   # odd row lengths
+    (3, 20, 14, 14, 2), (2, 9, 12, 30, 2), (1, 5, 11, 14, 2),                     # odd result rows
+])
+def test_fp16_rows_of_odd_length(N, C, H, W, s, combine):
+    """fp16 rows with an odd number of pixels: one pixel (two bytes) per lane on the
+    row-register kernels."""
+    from ddfnet_amd import _lib
+    assert 'k_rows<VX=1' in _lib.describe((N, C, H, W), 3, 1, s, combine, torch.float16)
+    assert 'k_rows_filters<' in _lib.describe((N, C, H, W), 3, 1, s, combine, torch.float16, need=7)
+    case = random_case(N, C, H, W, 3, s, torch.float16, seed=N + C + W)
+    check_against_oracle(*case, 3, 1, s, combine, '', what='fp16, odd rows')
+    x, cf, sf, go = case
+    together = run_ddf(x, cf, sf, go, 3, 1, s, combine)
+    only_dx = run_ddf(x, cf, sf, go, 3, 1, s, combine, need=(True, False, False))
+    only_filters = run_ddf(x, cf, sf, go, 3, 1, s, combine, need=(False, True, True))
+    assert rel_err(only_dx[1], together[1].cpu()) <= 2e-3
+    assert rel_err(only_filters[2], together[2].cpu()) <= 2e-3
+    assert rel_err(only_filters[3], together[3].cpu()) <= 2e-3
+
+
 def test_cpp_operator_equals_python_operator():
     """ddf is the C++ autograd function of the torch extension where that is
     built; DDFFunction is the Python one.  Same checks, same library calls:
