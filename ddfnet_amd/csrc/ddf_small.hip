@@ -18,21 +18,15 @@
 // (ddf/src/cuda/ddf_mul_cuda_kernel.cu:85-165 and :198-290 of the reference).
 #include <algorithm>
 
-#include "ddf_common.h"
+#include "ddf_chunks.h"
 
 namespace ddf {
 int tune_int(const char *name, int fallback);
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kMaxPlane = 64;        // G >= 4 channel planes per pass
-constexpr int kStageChannels = 128;  // channels whose taps are staged in LDS at a time
-
-__device__ __forceinline__ unsigned xcd_order(unsigned bid, unsigned nblocks) {
-    if (nblocks % 8u != 0) return bid;
-    return (bid % 8u) * (nblocks / 8u) + bid / 8u;
-}
+using chunks::kThreads;
+constexpr int kMaxPlane = chunks::kSmallMaxPlane;   // G >= 4 channel planes per pass
 
 // Up to UU channels (G apart) of one pixel; `valid` of them exist (the others
 // repeat the last one and store nothing, so the loads need no branch).  `xb` /
@@ -75,18 +69,16 @@ __global__ __launch_bounds__(kThreads) void k_small(
     extern __shared__ __align__(16) unsigned char small_smem[];
     A *taps = reinterpret_cast<A *>(small_smem);   // [channel][tap]
 
-    const unsigned bid = xcd_order(blockIdx.x, gridDim.x);
-    const int chunk = (int)(bid % (unsigned)csplit);
-    const int64_t n = bid / (unsigned)csplit;
-    const int c0 = chunk * cpb;
-    const int nch = min(cpb, C - c0);
+    chunks::Block blk;
+    blk.init(blockIdx.x, gridDim.x, csplit, 1, cpb, C);
+    const int64_t n = blk.n;
+    const int c0 = blk.c0, nch = blk.nch;
     const int plane = H * W;
 
     // threads past the G planes idle on slot 0 / pixel 0 and store nothing
-    const int q_raw = (int)threadIdx.x / plane;
-    const bool live = q_raw < G;
-    const int q = live ? q_raw : 0;
-    const int pix = live ? (int)threadIdx.x - q_raw * plane : 0;
+    chunks::SmallThread th;
+    th.init((int)threadIdx.x, plane, G);
+    const int q = th.q, pix = th.pix;
     const int y = pix / W, xx = pix - y * W;
 
     // neighbours: offset from the pixel, whether inside; the spatial tap that
@@ -127,7 +119,7 @@ __global__ __launch_bounds__(kThreads) void k_small(
         }
         __syncthreads();
         // this thread's channels of the stage: q, q + G, q + 2G, ...
-        const int mine = live && ns > q ? (ns - q + G - 1) / G : 0;
+        const int mine = th.channels(ns, G);
         const T *xs = xc + (int64_t)s0 * plane;
         T *os = oc + (int64_t)s0 * plane;
         const A *w = taps + q * KK;
@@ -143,22 +135,13 @@ template <typename T, bool BWD>
 hipError_t launch(const Problem &p, const T *x, const T *cf, const T *sf, T *out,
                   hipStream_t stream) {
     using A = typename Acc<T>::type;
-    const int plane = (int)(p.H * p.W);
-    const int G = kThreads / plane;
-    // about two blocks per CU (more, shorter blocks measured slower), at least
-    // 2 passes of G channels per block
-    const int64_t target = tune_int("DDF_TUNE_SMALL_BLOCKS", 1024);
-    int csplit = 1;
-    while (p.N * csplit * 2 <= target && p.C / (csplit * 2) >= 2 * G) csplit *= 2;
-    const int cpb = (int)cdiv(p.C, csplit);
-    csplit = (int)cdiv(p.C, cpb);
-    const int64_t blocks = p.N * csplit;
-    if (blocks > 2147483647) return hipErrorInvalidConfiguration;
-    const int stage = std::min(cpb, kStageChannels);
-    const size_t lds = (size_t)stage * 9 * sizeof(A);
+    chunks::ChunkGeom g;
+    if (!chunks::small_chunks(p.N, p.C, (int)(p.H * p.W), (int)sizeof(A),
+                              tune_int("DDF_TUNE_SMALL_BLOCKS", 1024), &g))
+        return hipErrorInvalidConfiguration;
     auto kern = p.mul ? k_small<T, 3, true, BWD> : k_small<T, 3, false, BWD>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), lds, stream, x, cf, sf, out,
-                       (int)p.C, (int)p.H, (int)p.W, p.d, G, cpb, csplit, stage);
+    hipLaunchKernelGGL(kern, dim3((unsigned)g.blocks), dim3(kThreads), g.lds, stream, x, cf, sf, out,
+                       (int)p.C, (int)p.H, (int)p.W, p.d, g.G, g.cpb, g.csplit, g.stage);
     return hipGetLastError();
 }
 

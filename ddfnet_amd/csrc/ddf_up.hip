@@ -14,16 +14,17 @@
 // with wave-uniform (broadcast) addresses.
 #include <algorithm>
 #include <atomic>
-#include <cstdlib>
 
-#include "ddf_common.h"
+#include "ddf_chunks.h"
 
 namespace ddf {
+int tune_int(const char *name, int fallback);
+
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kStageChannels = 32;     // channels whose taps are staged in LDS at a time
-constexpr int kStageBytes = 32 * 1024;  // and the LDS they may take
+using chunks::kThreads;
+constexpr int kStageChannels = chunks::kUpStageChannels;   // channels whose taps are staged in LDS at a time
+constexpr int kStageBytes = chunks::kUpStageBytes;         // and the LDS they may take
 
 template <typename T>
 struct UpFilters {
@@ -42,14 +43,6 @@ template <> struct RowBits<4> { using type = uint32_t; };
 template <> struct RowBits<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
 template <> struct RowBits<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
 template <> struct RowBits<32> { typedef uint32_t type __attribute__((ext_vector_type(8))); };
-
-// Workgroups reach the 8 XCDs round-robin; renumber so that consecutive
-// logical blocks (same sample and pixel block, neighbouring channel chunks,
-// hence the same spatial taps) run on one XCD and share its L2.
-__device__ __forceinline__ unsigned xcd_order(unsigned bid, unsigned nblocks) {
-    if (nblocks % 8u != 0) return bid;
-    return (bid % 8u) * (nblocks / 8u) + bid / 8u;
-}
 
 // UU channels of one pixel: every load is issued before the first result is
 // needed (a wave keeps UU*K*K loads in flight), then R rows of R results per
@@ -116,13 +109,13 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
     extern __shared__ __align__(16) unsigned char up_smem[];
     A *taps = reinterpret_cast<A *>(up_smem);   // [channel][branch][tap]
 
-    const unsigned bid = xcd_order(blockIdx.x, gridDim.x);
-    const int chunk = (int)(bid % (unsigned)csplit);
-    const unsigned rest = bid / (unsigned)csplit;
-    const int pb = (int)(rest % (unsigned)pblocks);
-    const int64_t n = rest / (unsigned)pblocks;
-    const int c0 = chunk * cpb;
-    const int nch = min(cpb, C - c0);
+    // (consecutive logical blocks - same sample and pixel block, neighbouring channel
+    // chunks, hence the same spatial taps - run on one XCD and share its L2)
+    chunks::Block blk;
+    blk.init(blockIdx.x, gridDim.x, csplit, pblocks, cpb, C);
+    const int pb = blk.pb;
+    const int64_t n = blk.n;
+    const int c0 = blk.c0, nch = blk.nch;
     const int plane = H * W;
 
     // Lanes past the end of the plane work on its last pixel and store nothing:
@@ -196,17 +189,10 @@ __global__ __launch_bounds__(kThreads) void k_up_forward(
     }
 }
 
-// Tuning knob from the environment (experiments only; results do not change).
-int up_tune(const char *name, int fallback) {
-    const char *v = std::getenv(name);
-    return (v && *v) ? std::atoi(v) : fallback;
-}
-
 template <typename T, int K, int R>
 hipError_t launch(bool mul, const UpFilters<T> &f, const T *x, T *out, int64_t N, int C, int H,
                   int W, int D, hipStream_t stream) {
     using A = typename Acc<T>::type;
-    const int64_t pblocks = cdiv((int64_t)H * W, kThreads);
     const int per_channel = R * R * K * K * (int)sizeof(A);
     // Split the channels over blocks until the chip is full once: as many
     // blocks as can be resident together (a second round of blocks would start
@@ -230,19 +216,14 @@ hipError_t launch(bool mul, const UpFilters<T> &f, const T *x, T *out, int64_t N
         (void)hipGetLastError();
         cus = 256;
     }
-    const int64_t target = up_tune("DDF_TUNE_UP_BLOCKS", per_cu * cus);
-    const int min_chunk = std::max(1, up_tune("DDF_TUNE_UP_MIN_CHUNK", 8));
-    int csplit = 1;
-    while (N * pblocks * csplit * 2 <= target && C / (csplit * 2) >= min_chunk) csplit *= 2;
-    const int cpb = (int)cdiv(C, csplit);
-    csplit = (int)cdiv(C, cpb);
-    const int64_t blocks = N * pblocks * csplit;
-    if (blocks > 2147483647) return hipErrorInvalidConfiguration;
-    const int stage = std::max(1, std::min({cpb, kStageChannels, kStageBytes / per_channel}));
-    const size_t lds = (size_t)stage * per_channel;
+    const int64_t target = tune_int("DDF_TUNE_UP_BLOCKS", per_cu * cus);
+    const int min_chunk = std::max(1, tune_int("DDF_TUNE_UP_MIN_CHUNK", 8));
+    chunks::ChunkGeom g;
+    if (!chunks::up_chunks(N, C, (int64_t)H * W, R * R * K * K, (int)sizeof(A), target, min_chunk, &g))
+        return hipErrorInvalidConfiguration;
     const int vec_ok = ((uintptr_t)out % (sizeof(T) * R)) == 0;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), lds, stream, f, x, out, C, H,
-                       W, D, cpb, csplit, (int)pblocks, stage, vec_ok);
+    hipLaunchKernelGGL(kern, dim3((unsigned)g.blocks), dim3(kThreads), g.lds, stream, f, x, out, C, H,
+                       W, D, g.cpb, g.csplit, g.pblocks, g.stage, vec_ok);
     return hipGetLastError();
 }
 

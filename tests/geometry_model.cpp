@@ -12,6 +12,7 @@
 
 #include "ddf_tiled_host.hip"
 #include "ddf_rows_host.hip"
+#include "ddf_chunks.h"
 
 using namespace ddf;
 
@@ -404,6 +405,104 @@ static void check_rows_stride2(long N, long C, long H, long W, int dtype, bool f
     g_fails = 0;
 }
 
+// k_small and k_up_forward (ddf_small.hip, ddf_up.hip): a workgroup takes one chunk of a
+// sample's channels [and one block of 256 pixels], stages the chunk's channel taps in LDS
+// `stage` channels at a time and walks the channels.  The model asks chunks::small_chunks /
+// up_chunks - the launchers' own code - for the cut and replays chunks::Block and
+// chunks::SmallThread - the kernels' own code - for every workgroup [and thread]: every
+// (sample, pixel block, chunk) handed out exactly once, chunks covering C, LDS within the
+// stage, tap indices inside the staged range, every (channel, pixel) of a chunk written once,
+// element offsets inside the chunk's planes and below 2^32.
+static void check_chunk_blocks(const chunks::ChunkGeom &g, long N, long C) {
+    CHECK(g.cpb >= 1 && (long)g.csplit * g.cpb >= C && (long)(g.csplit - 1) * g.cpb < C, "chunks do not tile C");
+    CHECK(g.blocks == N * g.pblocks * g.csplit, "block count");
+    CHECK(g.stage >= 1 && g.stage <= g.cpb, "stage of %d channels for chunks of %d", g.stage, g.cpb);
+    CHECK(g.lds <= 64 * 1024, "LDS %zu", g.lds);
+    if (g.blocks > 400000) return;   // (the numbering is checked on the smaller cases)
+    std::vector<char> seen(g.blocks, 0);
+    for (long raw = 0; raw < g.blocks; ++raw) {
+        chunks::Block b;
+        b.init((unsigned)raw, (unsigned)g.blocks, g.csplit, g.pblocks, g.cpb, (int)C);
+        CHECK(b.n >= 0 && b.n < N && b.pb >= 0 && b.pb < g.pblocks && b.chunk >= 0 && b.chunk < g.csplit, "block out of range");
+        CHECK(b.c0 == b.chunk * g.cpb && b.nch >= 1 && b.c0 + b.nch <= C, "channels %d+%d of %ld", b.c0, b.nch, C);
+        const long id = (b.n * g.pblocks + b.pb) * g.csplit + b.chunk;
+        if (id >= 0 && id < g.blocks) { CHECK(!seen[id], "block %ld handed out twice", id); seen[id] = 1; }
+    }
+    for (long i = 0; i < g.blocks; ++i)
+        if (!seen[i]) { CHECK(false, "block %ld never handed out", i); break; }
+}
+
+static void check_small(long N, long C, int H, int W, int dtype, long target) {
+    const int plane = H * W, asz = dtype == 2 ? 8 : 4;
+    chunks::ChunkGeom g;
+    if (!chunks::small_chunks(N, C, plane, asz, target, &g)) {
+        printf("kind small %ldx%ldx%dx%d dt%d: unsupported\n", N, C, H, W, dtype);
+        return;
+    }
+    printf("kind small %ldx%ldx%dx%d dt%d: G=%d cpb=%d csplit=%d stage=%d blocks=%ld lds=%zu\n", N, C, H, W, dtype,
+           g.G, g.cpb, g.csplit, g.stage, (long)g.blocks, g.lds);
+    CHECK(g.G >= 4 && g.G * plane <= chunks::kThreads && g.pblocks == 1, "G=%d planes of %d pixels", g.G, plane);
+    CHECK(g.lds == (size_t)g.stage * 9 * asz, "LDS bytes");
+    check_chunk_blocks(g, N, C);
+    // one chunk of every length that occurs: the full one and the last one
+    const int lens[2] = {g.cpb, (int)(C - (long)(g.csplit - 1) * g.cpb)};
+    for (int which = 0; which < 2; ++which) {
+        const int nch = lens[which];
+        CHECK((long)nch * plane < (1l << 32), "32-bit offsets inside a chunk");
+        std::vector<int> owner((size_t)nch * plane, 0);
+        for (int s0 = 0; s0 < nch; s0 += g.stage) {
+            const int ns = std::min(g.stage, nch - s0);
+            CHECK(ns * 9 <= g.stage * 9, "taps staged beyond LDS");
+            for (int tid = 0; tid < chunks::kThreads; ++tid) {
+                chunks::SmallThread th;
+                th.init(tid, plane, g.G);
+                CHECK(th.q >= 0 && th.q < g.G && th.pix >= 0 && th.pix < plane, "thread %d -> slot %d pixel %d", tid, th.q, th.pix);
+                const int mine = th.channels(ns, g.G);
+                CHECK(th.live || mine == 0, "idle thread %d works", tid);
+                for (int m = 0; m < mine; ++m) {
+                    const int ch = th.q + m * g.G;   // channel of the stage, as the kernel's `at` and `w` walk it
+                    CHECK(ch < ns, "thread %d channel %d of %d", tid, ch, ns);
+                    CHECK((ch + 1) * 9 <= ns * 9, "tap index beyond the staged taps");
+                    if (ch < ns) ++owner[(size_t)(s0 + ch) * plane + th.pix];
+                }
+            }
+        }
+        for (size_t i = 0; i < owner.size(); ++i)
+            if (owner[i] != 1) { CHECK(false, "chunk element %zu written %d times", i, owner[i]); break; }
+    }
+    if (g_fails) printf("  -> %d violations\n", g_fails);
+    g_fails = 0;
+}
+
+static void check_up(long N, long C, long H, long W, int k, int scale, int dtype, long target, int min_chunk) {
+    const int asz = dtype == 2 ? 8 : 4, taps = k * k * scale * scale;
+    chunks::ChunkGeom g;
+    if (!chunks::up_chunks(N, C, H * W, taps, asz, target, min_chunk, &g)) {
+        printf("kind up %ldx%ldx%ldx%ld k%d x%d dt%d: unsupported\n", N, C, H, W, k, scale, dtype);
+        return;
+    }
+    printf("kind up %ldx%ldx%ldx%ld k%d x%d dt%d: cpb=%d csplit=%d pblocks=%d stage=%d blocks=%ld lds=%zu\n", N, C, H, W,
+           k, scale, dtype, g.cpb, g.csplit, g.pblocks, g.stage, (long)g.blocks, g.lds);
+    CHECK((long)g.pblocks * chunks::kThreads >= H * W && (long)(g.pblocks - 1) * chunks::kThreads < H * W, "pixel blocks");
+    CHECK(g.lds == (size_t)g.stage * taps * asz && g.lds <= (size_t)chunks::kUpStageBytes + (size_t)taps * asz, "LDS bytes");
+    CHECK(g.stage <= chunks::kUpStageChannels, "stage");
+    check_chunk_blocks(g, N, C);
+    // staging of a stage's taps: element e of RR*ns*KK -> (branch, channel, tap) -> LDS slot
+    const int KK = k * k, RR = scale * scale;
+    for (int ns : {1, g.stage}) {
+        const int per = ns * KK, total = RR * per;
+        std::vector<char> slot((size_t)g.stage * RR * KK, 0);
+        for (int e = 0; e < total; ++e) {
+            const int b = e / per, r = e - b * per, ch = r / KK, t = r - ch * KK;
+            const long at = ((long)ch * RR + b) * KK + t;
+            CHECK(b < RR && ch < ns && at >= 0 && at < (long)slot.size(), "tap %d staged outside LDS", e);
+            if (at >= 0 && at < (long)slot.size()) { CHECK(!slot[at], "LDS slot %ld written twice", at); slot[at] = 1; }
+        }
+    }
+    if (g_fails) printf("  -> %d violations\n", g_fails);
+    g_fails = 0;
+}
+
 int main() {
     const long shapes[][4] = {
         {96, 64, 56, 56},   {64, 256, 14, 14}, {64, 128, 28, 28},  {64, 512, 7, 7},   {64, 64, 56, 56},
@@ -436,6 +535,22 @@ int main() {
         for (int dtype = 0; dtype < 3; ++dtype)
             for (int filters = 0; filters < 3; ++filters)
                 check_rows_stride2(sh[0], sh[1], sh[2], sh[3], dtype, filters != 0, filters == 2);
+    // tiny planes (k_small): every plane size 1..64, ragged C, C below G, fp64 stages
+    for (int H = 1; H <= 8; ++H)
+        for (int W = 1; W <= 64 / H; W += (W < 9 ? 1 : 5))
+            for (long C : {1l, 3l, 37l, 130l, 512l, 2048l})
+                for (int dtype = 1; dtype < 3; ++dtype)
+                    check_small(H == 7 ? 64 : 3, C, H, W, dtype, C == 130 ? 64 : 1024);
+    check_small(1, 1 << 24, 8, 8, 1, 1024);
+    // up-sampling forward: every (k, scale) pair that is built, ragged C, fp64 stage sizing
+    const int up_pairs[][2] = {{1, 2}, {1, 3}, {1, 4}, {3, 2}, {3, 3}, {3, 4}, {5, 2}};
+    for (auto &ks : up_pairs)
+        for (long C : {1l, 7l, 64l, 100l, 513l})
+            for (int dtype = 1; dtype < 3; ++dtype) {
+                check_up(8, C, 64, 64, ks[0], ks[1], dtype, 512, 8);
+                check_up(1, C, 5, 7, ks[0], ks[1], dtype, 2048, 1);
+                check_up(3, C, 33, 100, ks[0], ks[1], dtype, 256, 8);
+            }
     // seeded random shapes on top of the fixed list
     unsigned long long state = 0x9E3779B97F4A7C15ull;
     auto next = [&](int lo, int hi) {

@@ -3,7 +3,9 @@
 tests/geometry_model.cpp includes the library's geometry code and replays the
 kernels' address arithmetic on the CPU for many shapes (the benchmark shapes,
 ragged ones, 1-pixel planes, wide images; every kernel size / dilation / stride
-the tuned family is built for; aligned and scalar-access plans).  A launch
+the tuned families are built for; aligned and scalar-access plans; the chunked
+kernels for tiny planes and for the up-sampling forward at every plane size,
+kernel size and scale they take).  A launch
 geometry that would make a kernel read or write out of bounds - the kind of
 mistake that faults a GPU - shows up here as a VIOLATION line instead."""
 import os
