@@ -333,11 +333,19 @@ def model_inference(batch=128, steps=10, warmup=3):
             model(x)
         ms = timed_blocks(lambda i: model(x), steps)[1]
         layers = ddf_resnet.time_ddf_layers(model, x)
+        # the same network with the BatchNorms that follow convolutions folded into them
+        folded = ddf_resnet.fold_batchnorm(model)
+        for _ in range(warmup):
+            folded(x)
+        ms_folded = timed_blocks(lambda i: folded(x), steps)[1]
+        del folded
     ddf_ms = sum(l['ms'] for l in layers)
     ddf_bytes = sum(l['bytes'] for l in layers)
     return {'model': 'ddf_mul_resnet50', 'batch': batch, 'dtype': 'f16', 'input': [batch, 3, 224, 224],
             'weights': 'random (Kaiming normal, BatchNorm at default init)',
             'images_per_s': round(batch / (ms * 1e-3), 1), 'ms_per_batch': round(ms, 3),
+            'images_per_s_folded_batchnorm': round(batch / (ms_folded * 1e-3), 1),
+            'ms_per_batch_folded_batchnorm': round(ms_folded, 3),
             'ddf_ms_per_batch': round(ddf_ms, 3),
             'ddf_gbps': round(ddf_bytes / (ddf_ms * 1e-3) / 1e9, 1) if ddf_ms else None,
             'ddf_layers': layers}

@@ -122,6 +122,27 @@ ddf_add_resnet101 = _make([3, 4, 23, 3], 'add')
 ddf_add_resnet152 = _make([3, 8, 36, 3], 'add')
 
 
+def fold_batchnorm(model):
+    """A copy of an eval-mode ``DDFResNet`` for inference with every BatchNorm
+    that directly follows a convolution folded into that convolution's weights and
+    bias (the stem's, ``bn1`` and ``bn3`` of each block, the shortcut's).  In eval
+    mode BatchNorm is a per-channel affine map, so the network computes the same
+    function; ``bn2`` follows the dynamic filter and stays."""
+    import copy
+    from torch.nn.utils.fusion import fuse_conv_bn_eval
+    assert not model.training, 'fold_batchnorm is for eval-mode models'
+    model = copy.deepcopy(model)
+    model.conv1, model.bn1 = fuse_conv_bn_eval(model.conv1, model.bn1), nn.Identity()
+    for block in model.modules():
+        if isinstance(block, DDFBottleneck):
+            block.conv1, block.bn1 = fuse_conv_bn_eval(block.conv1, block.bn1), nn.Identity()
+            block.conv3, block.bn3 = fuse_conv_bn_eval(block.conv3, block.bn3), nn.Identity()
+            if block.downsample is not None:
+                block.downsample = nn.Sequential(
+                    fuse_conv_bn_eval(block.downsample[0], block.downsample[1]))
+    return model
+
+
 def time_ddf_layers(model, x, iters=20):
     """Run ``model(x)`` once, record the operands of every ``ddf`` call made by
     its DDFPacks, then time each call on its own.  Returns one dict per layer

@@ -232,6 +232,30 @@ def test_resnet50_fp16_inference_and_layer_timing():
     assert shapes == want
 
 
+def test_resnet50_with_folded_batchnorm_computes_the_same_function():
+    """fold_batchnorm folds the eval-mode BatchNorms that follow convolutions into
+    them: same logits (fp32, non-trivial running statistics), fewer modules."""
+    from ddfnet_amd import ddf_resnet
+    torch.manual_seed(5)
+    model = ddf_resnet.ddf_mul_resnet50(num_classes=10, zero_init_last_bn=False).cuda()
+    for m in model.modules():
+        if isinstance(m, torch.nn.BatchNorm2d):
+            torch.nn.init.uniform_(m.weight, 0.5, 1.5)
+            torch.nn.init.uniform_(m.bias, -0.2, 0.2)
+            m.running_mean.uniform_(-0.1, 0.1)
+            m.running_var.uniform_(0.5, 1.5)
+    model.eval()
+    folded = ddf_resnet.fold_batchnorm(model)
+    n_bn = lambda net: sum(isinstance(m, torch.nn.BatchNorm2d) for m in net.modules())
+    assert n_bn(model) == 53 and n_bn(folded) == 16   # one per block remains (after the DDF layer)
+    x = torch.randn(2, 3, 64, 64, device='cuda')
+    with torch.no_grad():
+        want, got = model(x), folded(x)
+    assert (got - want).abs().max().item() <= 1e-4 * want.abs().max().item()
+    with pytest.raises(AssertionError):
+        ddf_resnet.fold_batchnorm(model.train())
+
+
 # ---------------------------------------------------------------------------
 # fused filter normalisation
 # ---------------------------------------------------------------------------
