@@ -11,7 +11,7 @@
 //     cf[n, c, t] = norm_t( b2[c*KK + t] + sum_m w2[c*KK + t, m] * relu(b1[m] + sum_c' w1[m, c'] * v[n, c']) )
 //   the two 1x1 convolutions on the pooled (n, c) vector are small matrix
 //   products; one workgroup computes the hidden vector of its sample and 64
-//   channels' filters, and normalises them in place.
+//   (wide layers: 128) channels' filters, and normalises them in place.
 //
 // norm_t(u) = gain_t * (u_t - mean(u)) / (std(u) + 1e-10) + offset_t with the
 // unbiased standard deviation over the KK taps, as in ddf_filter_norm.hip.
@@ -22,6 +22,8 @@
 #include "ddf_common.h"
 
 namespace ddf {
+int tune_int(const char *name, int fallback);
+
 namespace {
 
 constexpr int kChunk = 256;   // channels whose weights sit in LDS at a time (64 per wave)
@@ -270,106 +272,124 @@ __global__ __launch_bounds__(4 * kWave) void k_spatial_branch_tiles(
     }
 }
 
-// Sum over the 64 lanes (the same value in every lane): four butterfly steps
-// inside each row of 16 lanes through the VALU's lane-permute path, then the
-// four row sums through scalar registers.  (Shuffles through the LDS crossbar
-// cost a round trip each and made these kernels several times slower.)
+// Butterfly steps through the VALU's lane-permute path.  (Shuffles through the
+// LDS crossbar cost a round trip each and made these kernels several times slower.)
 template <int CTRL>
 __device__ __forceinline__ float add_permuted(float x) {
     return x + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float wave_sum(float v) {
+// Sum over each row of 16 lanes (the same value in every lane of the row).
+__device__ __forceinline__ float row_sum(float v) {
     v = add_permuted<0xB1>(v);    // quad_perm [1,0,3,2]
     v = add_permuted<0x4E>(v);    // quad_perm [2,3,0,1]
     v = add_permuted<0x141>(v);   // row_half_mirror
-    v = add_permuted<0x140>(v);   // row_mirror
-    const int b = __float_as_int(v);
-    return (__int_as_float(__builtin_amdgcn_readlane(b, 0)) + __int_as_float(__builtin_amdgcn_readlane(b, 16))) +
-           (__int_as_float(__builtin_amdgcn_readlane(b, 32)) + __int_as_float(__builtin_amdgcn_readlane(b, 48)));
+    return add_permuted<0x140>(v);   // row_mirror
 }
 
-constexpr int kChannelBlock = 64;     // channels whose filters one workgroup makes
 constexpr int kChannelThreads = 1024;  // sixteen waves: the rows of a block's taps are dealt out to them
 constexpr int kChannelWaves = kChannelThreads / kWave;
 
-// grid (channel blocks of kChannelBlock, N).  LDS: the pooled vector (C floats),
-// the hidden vector (mid floats), the block's un-normalised taps.  Every dot
-// product has the lanes of a wave along the weight row (coalesced) and ends in
-// a wave reduction; several rows are in flight per wave.  Every workgroup of a
-// sample recomputes the hidden vector, so the blocks are large: smaller ones
-// had all compute units read the same rows of w1 at once, which the L2 serves
-// one after the other.
-template <typename T, int KK>
+// grid (channel blocks of BLOCK channels, groups of NS samples).  LDS: the pooled
+// vectors (NS * C floats), the hidden vectors (NS * mid floats), the block's
+// un-normalised taps (NS * BLOCK * KK).  Every weight a lane loads serves the NS
+// samples of its workgroup (the weights are the same for all samples; re-read
+// per sample they cost more L2 bandwidth than anything else here).  Every
+// workgroup of a sample recomputes the hidden vector, so the blocks are large:
+// smaller ones had all compute units read the same rows of w1 at once, which
+// the L2 serves one after the other.
+template <typename T, int KK, int BLOCK, int NS>
 __global__ __launch_bounds__(kChannelThreads) void k_channel_branch(
     const T *__restrict__ pooled, const T *__restrict__ w1, const T *__restrict__ b1,
-    const T *__restrict__ w2, const T *__restrict__ b2, T *__restrict__ cf, int C, int mid,
+    const T *__restrict__ w2, const T *__restrict__ b2, T *__restrict__ cf, int N, int C, int mid,
     float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
     extern __shared__ float branch_smem[];
-    float *v = branch_smem;            // [C]
-    float *h = v + C;                  // [mid]
-    float *f = h + mid;                // [kChannelBlock * KK]
+    float *v = branch_smem;            // [NS][C]
+    float *h = v + NS * C;             // [NS][mid]
+    float *f = h + NS * mid;           // [NS][BLOCK * KK]
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-    const int64_t n = blockIdx.y;
-    const int cb = blockIdx.x * kChannelBlock;
-    for (int c = threadIdx.x; c < C; c += kChannelThreads) v[c] = ld(pooled + n * C + c);
+    const int64_t n0 = (int64_t)blockIdx.y * NS;
+    const int ns = min(NS, N - (int)n0);   // samples of this workgroup (the others: copies of the last)
+    const int cb = blockIdx.x * BLOCK;
+    for (int i = threadIdx.x; i < NS * C; i += kChannelThreads) {
+        const int s = i / C, c = i - s * C;
+        v[i] = ld(pooled + (n0 + min(s, ns - 1)) * C + c);
+    }
     __syncthreads();
-    // hidden vector: four rows of w1 per wave at a time
-    constexpr int RH = 4;
-    for (int m0 = wave * RH; m0 < mid; m0 += kChannelWaves * RH) {
-        float p[RH];
+    // Dot products with sixteen lanes along a weight row and four rows per wave at a
+    // time: each ends in a reduction over a row of 16 lanes (four lane-permute
+    // additions for four results; a whole wave per row paid thirteen for one).
+    const int seg = lane >> 4, sl = lane & 15;
+    // hidden vectors: rows of w1
+    for (int m0 = wave * 4; m0 < mid; m0 += kChannelWaves * 4) {
+        const int m = min(m0 + seg, mid - 1);
+        const T *row = w1 + (int64_t)m * C;
+        float p[NS];
 #pragma unroll
-        for (int u = 0; u < RH; ++u) p[u] = 0.f;
-#pragma unroll 4   // (all of a 256-channel row's loads go out before the first is used)
-        for (int c = lane; c < C; c += kWave) {
-            const float vc = v[c];
+        for (int s = 0; s < NS; ++s) p[s] = 0.f;
+#pragma unroll 8
+        for (int c = sl; c < C; c += 16) {
+            const float wv = ld(row + c);
 #pragma unroll
-            for (int u = 0; u < RH; ++u) {
-                const int m = min(m0 + u, mid - 1);
-                p[u] = fmaf(ld(w1 + (int64_t)m * C + c), vc, p[u]);
-            }
+            for (int s = 0; s < NS; ++s) p[s] = fmaf(wv, v[s * C + c], p[s]);
         }
+        const float bias = b1 ? ld(b1 + m) : 0.f;
 #pragma unroll
-        for (int u = 0; u < RH; ++u) {
-            const float tot = wave_sum(p[u]);
-            if (lane == 0 && m0 + u < mid) h[m0 + u] = fmaxf(tot + (b1 ? ld(b1 + m0 + u) : 0.f), 0.f);
+        for (int s = 0; s < NS; ++s) {
+            const float tot = row_sum(p[s]);
+            if (sl == 0 && m0 + seg < mid) h[s * mid + m0 + seg] = fmaxf(tot + bias, 0.f);
         }
     }
     __syncthreads();
-    // the block's taps: rows (cb * KK + r) of w2, eighteen per wave at a time
-    constexpr int RT = 18;
-    const int rows = min(kChannelBlock, C - cb) * KK;
-    for (int r0 = wave * RT; r0 < rows; r0 += kChannelWaves * RT) {
-        float p[RT];
+    // the block's taps: rows (cb * KK + r) of w2, RT passes of four rows in flight per wave
+    constexpr int RT = NS >= 4 ? 1 : NS == 2 ? 2 : 3;
+    const int rows = min(BLOCK, C - cb) * KK;
+    for (int r0 = wave * 4 * RT; r0 < rows; r0 += kChannelWaves * 4 * RT) {
+        float p[RT][NS];
+        const T *wrow[RT];
 #pragma unroll
-        for (int u = 0; u < RT; ++u) p[u] = 0.f;
+        for (int u = 0; u < RT; ++u) {
+#pragma unroll
+            for (int s = 0; s < NS; ++s) p[u][s] = 0.f;
+            wrow[u] = w2 + ((int64_t)cb * KK + min(r0 + 4 * u + seg, rows - 1)) * mid;
+        }
 #pragma unroll 2
-        for (int m = lane; m < mid; m += kWave) {
-            const float hm = h[m];
+        for (int m = sl; m < mid; m += 16) {
+            float hm[NS];
+#pragma unroll
+            for (int s = 0; s < NS; ++s) hm[s] = h[s * mid + m];
 #pragma unroll
             for (int u = 0; u < RT; ++u) {
-                const int64_t row = (int64_t)cb * KK + min(r0 + u, rows - 1);
-                p[u] = fmaf(ld(w2 + row * mid + m), hm, p[u]);
+                const float wv = ld(wrow[u] + m);
+#pragma unroll
+                for (int s = 0; s < NS; ++s) p[u][s] = fmaf(wv, hm[s], p[u][s]);
             }
         }
 #pragma unroll
         for (int u = 0; u < RT; ++u) {
-            const float tot = wave_sum(p[u]);
-            if (lane == 0 && r0 + u < rows)
-                f[r0 + u] = tot + (b2 ? ld(b2 + (int64_t)cb * KK + r0 + u) : 0.f);
+            const int r = r0 + 4 * u + seg;
+            const float bias = (b2 && r < rows) ? ld(b2 + (int64_t)cb * KK + r) : 0.f;
+#pragma unroll
+            for (int s = 0; s < NS; ++s) {
+                const float tot = row_sum(p[u][s]);
+                if (sl == 0 && r < rows) f[s * BLOCK * KK + r] = tot + bias;
+            }
         }
     }
     __syncthreads();
-    const int i = threadIdx.x;
-    if (i >= kChannelBlock || cb + i >= C) return;
-    float u[KK];
+    // one thread per (sample, channel) normalises the KK taps
+    for (int i = threadIdx.x; i < NS * BLOCK; i += kChannelThreads) {
+        const int s = i / BLOCK, ch = i - s * BLOCK;
+        if (s >= ns || cb + ch >= C) continue;
+        float u[KK];
 #pragma unroll
-    for (int t = 0; t < KK; ++t) u[t] = f[i * KK + t];
-    TapParams<T, KK> params;
-    params.load(cb + i, gain, gain_vec, offset_vec, (const T *)nullptr);   // (b2 is in f already)
-    normalise<T, KK>(u, params);
-    T *op = cf + (n * C + cb + i) * KK;
+        for (int t = 0; t < KK; ++t) u[t] = f[(s * BLOCK + ch) * KK + t];
+        TapParams<T, KK> params;
+        params.load(cb + ch, gain, gain_vec, offset_vec, (const T *)nullptr);   // (b2 is in f already)
+        normalise<T, KK>(u, params);
+        T *op = cf + ((n0 + s) * C + cb + ch) * KK;
 #pragma unroll
-    for (int t = 0; t < KK; ++t) st(op + t, u[t]);
+        for (int t = 0; t < KK; ++t) st(op + t, u[t]);
+    }
 }
 
 }  // namespace
@@ -431,15 +451,33 @@ hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2
                           const T *gain_vec, const T *offset_vec, hipStream_t st) {
     if (N == 0 || C == 0) return hipSuccess;
     const int kk = k * k;
-    const size_t lds = ((size_t)C + (size_t)mid + (size_t)kChannelBlock * kk) * sizeof(float);
-    if (N > 65535 || mid < 1 || lds > 48 * 1024) return hipErrorNotSupported;
-    const dim3 grid((unsigned)cdiv(C, kChannelBlock), (unsigned)N);
-#define DDF_CHANNEL_CASE(KK_)                                                                    \
-    hipLaunchKernelGGL((k_channel_branch<T, KK_>), grid, dim3(kChannelThreads), lds, st, pooled, w1, \
-                       b1, w2, b2, cf, (int)C, (int)mid, (float)gain, gain_vec, offset_vec)
-    if (k == 3) DDF_CHANNEL_CASE(9);
-    else if (k == 5) DDF_CHANNEL_CASE(25);
+    // (wide layers: fewer, larger blocks, as every block of a sample recomputes the hidden vector)
+    const int block = C >= 512 ? 128 : 64;
+    // samples per workgroup: as many as keep every compute unit busy and fit the LDS
+    auto lds_of = [&](int ns) { return ((size_t)C + (size_t)mid + (size_t)block * kk) * ns * sizeof(float); };
+    int ns = 1;
+    const int forced = tune_int("DDF_TUNE_CHANNEL_NS", 0);
+    while (ns < 4 && cdiv(C, block) * cdiv(N, ns * 2) >= 256 && lds_of(ns * 2) <= 48 * 1024) ns *= 2;
+    if (forced == 1 || forced == 2 || forced == 4) ns = forced;
+    const size_t lds = lds_of(ns);
+    if (N > 65535 * ns || mid < 1 || lds > 48 * 1024) return hipErrorNotSupported;
+    const dim3 grid((unsigned)cdiv(C, block), (unsigned)cdiv(N, ns));
+#define DDF_CHANNEL_LAUNCH(KK_, BLOCK_, NS_)                                                     \
+    hipLaunchKernelGGL((k_channel_branch<T, KK_, BLOCK_, NS_>), grid, dim3(kChannelThreads), lds, \
+                       st, pooled, w1, b1, w2, b2, cf, (int)N, (int)C, (int)mid, (float)gain,    \
+                       gain_vec, offset_vec)
+#define DDF_CHANNEL_CASE(KK_, BLOCK_)                                                            \
+    do {                                                                                         \
+        if (ns == 4) DDF_CHANNEL_LAUNCH(KK_, BLOCK_, 4);                                         \
+        else if (ns == 2) DDF_CHANNEL_LAUNCH(KK_, BLOCK_, 2);                                    \
+        else DDF_CHANNEL_LAUNCH(KK_, BLOCK_, 1);                                                 \
+    } while (0)
+    if (k == 3 && block == 64) DDF_CHANNEL_CASE(9, 64);
+    else if (k == 3) DDF_CHANNEL_CASE(9, 128);
+    else if (k == 5 && block == 64) DDF_CHANNEL_CASE(25, 64);
+    else if (k == 5) DDF_CHANNEL_CASE(25, 128);
     else return hipErrorNotSupported;
+#undef DDF_CHANNEL_LAUNCH
 #undef DDF_CHANNEL_CASE
     return hipGetLastError();
 }
