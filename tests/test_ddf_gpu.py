@@ -454,18 +454,22 @@ def test_results_are_deterministic():
         assert torch.equal(u, v)
 
 
-def test_forward_and_backward_replay_in_a_hip_graph():
+@pytest.mark.parametrize('shape,stride,dtype', [
+    ((4, 32, 14, 14), 1, torch.float32),    # one-launch backward + one partial sum
+    ((2, 40, 56, 56), 2, torch.float32),    # stride 2: one-launch backward + both partial sums
+    ((3, 20, 7, 7), 1, torch.float16),      # two-byte vectors
+], ids=_ids)
+def test_forward_and_backward_replay_in_a_hip_graph(shape, stride, dtype):
     """The operator allocates nothing the capture cannot own and enqueues only
     kernels (no memset nodes), so forward + backward can be captured once and
     replayed.  Every replay - with ordinary eager work and synchronisation in
     between - must reproduce the eager result bit for bit."""
     from ddfnet_amd import ddf
-    shape = (4, 32, 14, 14)
-    host = [random_case(*shape, 3, 1, torch.float32, seed=s) for s in (21, 22, 23)]
+    host = [random_case(*shape, 3, stride, dtype, seed=s) for s in (21, 22, 23)]
     x, cf, sf, go = (t.clone().requires_grad_(i < 3) for i, t in enumerate(to_dev(*host[0])))
 
     def step():
-        out = ddf(x, cf, sf, 3, 1, 1, 'mul')
+        out = ddf(x, cf, sf, 3, 1, stride, 'mul')
         return (out,) + torch.autograd.grad(out, (x, cf, sf), go)
 
     side = torch.cuda.Stream()
