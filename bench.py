@@ -287,6 +287,25 @@ def profile_phase(name, phase, steps, warmup, lib):
             'copy_probe_bytes': 4 * a.numel() * 4}
 
 
+def profile_model(batches=5, warmup=4, batch=128):
+    """ddf_mul_resnet50 fp16 inference for runs under rocprofv3: warm-up batches (in which
+    the convolution library searches its kernels), half a second of silence, then `batches`
+    timed batches - the dispatches after the gap in the trace are the steady state."""
+    import time
+    from ddfnet_amd import ddf_resnet
+    torch.manual_seed(0)
+    model = ddf_resnet.ddf_mul_resnet50(zero_init_last_bn=False).cuda().half().eval()
+    x = torch.randn(batch, 3, 224, 224, device='cuda', dtype=torch.float16)
+    with torch.no_grad():
+        for _ in range(warmup):
+            model(x)
+        torch.cuda.synchronize()
+        time.sleep(0.5)
+        ms = timed(lambda i: model(x), batches)
+    return {'model': 'ddf_mul_resnet50', 'batch': batch, 'dtype': 'f16', 'batches': batches,
+            'ms_per_batch': round(ms, 3)}
+
+
 def cpu_baseline(name, budget_s=12.0):
     """The CPU oracle (a port of the reference's formulation; the reference has
     no CPU path of its own) timed on this host: fp32, forward + backward, on a
@@ -487,6 +506,9 @@ def main():
                     help='run only this library call of the workload (warm-up + steps calls, then the '
                          'copy probe) and print what was run: the unit the profiles/ summaries are '
                          'collected on')
+    ap.add_argument('--profile-model', action='store_true',
+                    help='run only the ResNet-50 inference (warm-up, a half-second gap, then --steps '
+                         'batches): the unit the model summary in profiles/ is collected on')
     ap.add_argument('--copy-probe', action='store_true',
                     help='also run a plain 256 MiB device copy (calibrates hardware counters)')
     args = ap.parse_args()
@@ -499,6 +521,9 @@ def main():
     from ddfnet_amd import _lib as lib
     lib.lib()
 
+    if args.profile_model:
+        print(json.dumps(profile_model(batches=args.steps)))
+        return
     if args.profile_phase:
         print(json.dumps(profile_phase(args.workload, args.profile_phase, args.steps, args.warmup, lib)))
         return
