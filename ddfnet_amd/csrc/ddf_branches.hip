@@ -409,7 +409,7 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
     const int chunk = (int)std::min<int64_t>(kChunk, (C + 8 * waves - 1) / (8 * waves) * (8 * waves));
     // Planes with many pixels: a wave per pixel tile, as wide a vector per lane as
     // rows and alignment allow while the waves still fill the machine.
-    if (stride == 1) {
+    if (stride == 1 && tune_int("DDF_TUNE_SPATIAL_TILES", 1) != 0) {
         for (int vp = 16 / (int)sizeof(T); vp >= 1; vp /= 2) {
             if (k == 5 && vp > 2) continue;   // (25 taps: the accumulators of two pixels per lane)
             if (W % vp != 0 || (((uintptr_t)x | (uintptr_t)sf) % (vp * sizeof(T))) != 0) continue;
@@ -438,7 +438,27 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
     hipLaunchKernelGGL((k_spatial_branch<T, KK_, WAVES_, VP_>), grid, dim3(WAVES_ * kWave), 0, st, x, \
                        w, bias, sf, (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, chunk,    \
                        (float)gain, gain_vec, offset_vec)
-    if (k == 3) DDF_SPATIAL_CASE(9, 8, 1);
+    // (vectors of pixels per lane where rows and alignment allow: fewer, wider loads)
+    int vp = 1;
+    // (two-byte elements; four-byte ones gain nothing from it)
+    if (stride == 1 && k == 3 && sizeof(T) == 2) {
+        for (int cand = tune_int("DDF_TUNE_SPATIAL_VP", 4); cand > 1; cand /= 2)
+            if (W % cand == 0 && (((uintptr_t)x | (uintptr_t)sf) % (cand * sizeof(T))) == 0 &&
+                N * head * cdiv(Ho * Wo, kWave * cand) >= 256) {
+                vp = cand;
+                break;
+            }
+    }
+    const dim3 grid_v((unsigned)cdiv(Ho * Wo, kWave * vp), (unsigned)head, (unsigned)N);
+    if (k == 3 && vp == 4) {
+        hipLaunchKernelGGL((k_spatial_branch<T, 9, 8, 4>), grid_v, dim3(8 * kWave), 0, st, x, w, bias, sf,
+                           (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, chunk, (float)gain, gain_vec,
+                           offset_vec);
+    } else if (k == 3 && vp == 2) {
+        hipLaunchKernelGGL((k_spatial_branch<T, 9, 8, 2>), grid_v, dim3(8 * kWave), 0, st, x, w, bias, sf,
+                           (int)C, (int)H, (int)W, (int)Ho, (int)Wo, stride, chunk, (float)gain, gain_vec,
+                           offset_vec);
+    } else if (k == 3) DDF_SPATIAL_CASE(9, 8, 1);
     else if (k == 5) DDF_SPATIAL_CASE(25, 4, 1);
     else return hipErrorNotSupported;
 #undef DDF_SPATIAL_CASE
