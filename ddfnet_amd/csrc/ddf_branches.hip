@@ -414,7 +414,7 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
             if (k == 5 && vp > 2) continue;   // (25 taps: the accumulators of two pixels per lane)
             if (W % vp != 0 || (((uintptr_t)x | (uintptr_t)sf) % (vp * sizeof(T))) != 0) continue;
             if (vp == 1 && sizeof(T) == 2) continue;   // (2-byte loads: the shared-pixel kernel does better)
-            if ((Ho * Wo) % vp != 0 || N * head * cdiv(Ho * Wo, kWave * vp) < 1024) continue;
+            if ((Ho * Wo) % vp != 0 || N * head * cdiv(Ho * Wo, kWave * vp) < tune_int("DDF_TUNE_SPATIAL_TILES_MIN", 1024)) continue;
             const dim3 grid((unsigned)cdiv(Ho * Wo, 4 * kWave * vp), (unsigned)head, (unsigned)N);
 #define DDF_TILES_CASE(KK_, VP_)                                                                \
     hipLaunchKernelGGL((k_spatial_branch_tiles<T, KK_, VP_>), grid, dim3(4 * kWave), 0, st, x, w, \
