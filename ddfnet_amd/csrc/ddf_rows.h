@@ -1,7 +1,9 @@
-// Row-register DDF kernels for gfx950 (stride 1): forward and feature gradient.
+// Row-register DDF kernels for gfx950: forward and feature gradient with stride 1,
+// the 3 x 3 forward also with stride 2 (LaneStride2, the S = 2 instantiations).
 //
-// A lane owns R consecutive rows of VX neighbouring pixels (one 16-, 8- or 4-byte
-// vector per row) of one sample and walks a range of channels.  Nothing of the
+// A lane owns R consecutive rows of VX neighbouring pixels (one 16-, 8-, 4- or -
+// a single fp16 pixel - 2-byte vector per row) of one sample and walks a range
+// of channels.  Nothing of the
 // feature map goes through LDS:
 //   * the R + 2*HY rows a lane needs per channel (its own and the HY = (K/2)*D
 //     rows above and below) come straight from global memory as whole vectors,

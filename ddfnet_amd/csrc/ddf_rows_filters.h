@@ -1,5 +1,6 @@
-// Row-register filter-gradient kernel for gfx950 (stride 1): dCF and dSF in one
-// walk, same lane layout and feature-row handling as ddf_rows.h.
+// Row-register filter-gradient kernel for gfx950 (stride 1; 3 x 3 also with
+// stride 2): dCF and dSF in one walk, same lane layout and feature-row handling
+// as ddf_rows.h.
 //
 // The kFilterWaves waves of a workgroup work on the same strip of the same
 // sample and walk consecutive channel ranges of g.cpw channels each.  Per
@@ -7,7 +8,8 @@
 // to both sums:
 //   dSF[t, pixel] += gx[t] * CF[c, t]      register accumulators over the walk
 //   dCF[c, t]      = sum over pixels of gx[t] * SF[t, pixel]
-// ('add' combine: both are sums of gx[t] itself.)  The per-lane dCF partials
+// ('add' combine: both are sums of gx[t] itself, formed by two multiply-adds
+// without the product in between.)  The per-lane dCF partials
 // of kFlushChannels channels are parked in LDS, lane-contiguous per (channel,
 // tap); then one lane per (channel, tap) adds up the 64 lane values with
 // 16-byte reads.  That costs a quarter of the vector instructions of a
@@ -54,8 +56,9 @@ __device__ __forceinline__ void wave_sync() {
 // second set of spatial taps (those of the pixels its dO values come from),
 // and every channel ends with the store of its dX rows.  One launch for the
 // whole backward pass; dO, CF and SF are read once.
-// S = 2 (3 x 3, one row per lane, filter gradients only): g describes the dO
-// plane, the lane's feature vectors are 2 * VX elements wide (LaneStride2).
+// S = 2 (3 x 3, one row per lane): g describes the dO plane, the lane's feature
+// vectors are 2 * VX elements wide (LaneStride2).  With DX the lane of result
+// row y also writes the feature gradient of feature rows 2y and 2y + 1.
 template <typename T, int K, int D, bool MUL, int VX, int R, bool PAD, bool DX, int NST, int WPE,
           int S = 1>
 __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
