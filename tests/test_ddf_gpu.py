@@ -376,6 +376,33 @@ def test_non_contiguous_inputs_are_accepted():
     assert out.is_contiguous() and rel_err(dx, want) <= 1e-5
 
 
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16], ids=_ids)
+@pytest.mark.parametrize('shape,stride', [((2, 16, 14, 14), 1), ((1, 33, 28, 56), 2), ((2, 3, 7, 7), 1),
+                                          ((1, 16, 8, 28), 2)])
+def test_tensors_that_start_at_odd_addresses(shape, stride, dtype):
+    """Contiguous tensors whose first element is one to three elements into an
+    allocation (views): the vector kernels turn such pointers down and the call
+    falls back to kernels with narrower accesses; results as always."""
+    from ddfnet_amd import ddf
+
+    def shifted(t, off):
+        base = torch.empty(t.numel() + 8, dtype=t.dtype, device='cuda')
+        view = base[off:off + t.numel()].view(t.shape)
+        view.copy_(t)
+        return view
+
+    for combine, offs in (('mul', (1, 0, 0, 0)), ('add', (0, 0, 1, 2)), ('mul', (3, 1, 2, 1))):
+        x, cf, sf, go = random_case(*shape, 3, stride, dtype, seed=sum(offs))
+        xd, cfd, sfd, god = (shifted(t.cuda(), o) for t, o in zip((x, cf, sf, go), offs))
+        leaves = [t.requires_grad_(True) for t in (xd, cfd, sfd)]
+        out = ddf(*leaves, 3, 1, stride, combine)
+        grads = torch.autograd.grad(out, leaves, god)
+        want = (oracle.forward(x, cf, sf, 3, 1, stride, combine),) + tuple(
+            oracle.backward(go, x, cf, sf, 3, 1, stride, combine))
+        for got, w in zip((out,) + tuple(grads), want):
+            assert rel_err(got.detach(), w) <= TOL[dtype]
+
+
 def test_runs_on_the_current_stream():
     from ddfnet_amd import ddf
     x, cf, sf, _ = random_case(4, 16, 14, 14, 3, 1, torch.float32, seed=12)
