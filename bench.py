@@ -287,6 +287,33 @@ def profile_phase(name, phase, steps, warmup, lib):
             'copy_probe_bytes': 4 * a.numel() * 4}
 
 
+def device_copy_ceiling(step_bytes):
+    """What a plain device-to-device copy reaches on this box: the practical
+    ceiling beside the 8 TB/s of the data sheet.  Once at 256 MiB, once moving as
+    many bytes as one forward call of the workload (read half, write half),
+    rotating over enough buffers to stay out of the last-level cache."""
+    big_a = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device='cuda')
+    big_b = torch.empty_like(big_a)
+    for _ in range(3):
+        big_b.copy_(big_a)
+    ms_big = timed(lambda i: big_b.copy_(big_a), 10)
+    big_bytes = 2 * big_a.numel() * 4
+    del big_a, big_b
+    half = max(1, step_bytes // 8)             # floats per side
+    pairs = int(max(2, 2 * LLC_BYTES // (half * 8) + 1))
+    src = [torch.empty(half, dtype=torch.float32, device='cuda') for _ in range(pairs)]
+    dst = [torch.empty(half, dtype=torch.float32, device='cuda') for _ in range(pairs)]
+    for i in range(pairs):
+        dst[i].copy_(src[i])
+    ms_small = timed(lambda i: dst[i % pairs].copy_(src[i % pairs]), 100)
+    out = {'bytes_large': big_bytes, 'gbps_large': round(big_bytes / (ms_big * 1e-3) / 1e9, 1),
+           'bytes_small': half * 8, 'us_small': round(ms_small * 1e3, 2),
+           'gbps_small': round(half * 8 / (ms_small * 1e-3) / 1e9, 1)}
+    del src, dst
+    torch.cuda.empty_cache()
+    return out
+
+
 def profile_model(batches=5, warmup=4, batch=128):
     """ddf_mul_resnet50 fp16 inference for runs under rocprofv3: warm-up batches (in which
     the convolution library searches its kernels), half a second of silence, then `batches`
@@ -553,6 +580,10 @@ def main():
     }
     if extra:
         line['other_workloads'] = {n: workload_summary(r) for n, r in extra.items()}
+    line['device_copy'] = device_copy_ceiling(res['bytes']['fwd'])
+    dc = line['device_copy']
+    log('[copy] device-to-device copy: %.0f GB/s moving %d MiB; %.0f GB/s (%.1f us) moving the %.1f MB of a forward call' % (
+        dc['gbps_large'], dc['bytes_large'] >> 20, dc['gbps_small'], dc['us_small'], dc['bytes_small'] / 1e6))
     if not args.only_headline:
         line['model_inference'] = model_inference()
         mi = line['model_inference']
