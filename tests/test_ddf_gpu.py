@@ -552,6 +552,29 @@ def test_random_shapes_against_oracle(chunk):
                              what='chunk %d case %d %s' % (chunk, i, (N, C, H, W, str(dtype))))
 
 
+@pytest.mark.parametrize('chunk', range(3))
+def test_random_stride_two_and_odd_rows_against_oracle(chunk):
+    """Seeded random 3x3 problems aimed at the stride-2 row kernels (all vector
+    widths, odd heights, rows too long for them) and at fp16 rows of odd length."""
+    import random
+    rng = random.Random(4000 + chunk)
+    done = 0
+    while done < 40:
+        s = rng.choice([1, 2, 2])
+        dtype = rng.choice([torch.float16, torch.float32, torch.float16])
+        N, C = rng.randint(1, 3), rng.choice([1, 2, 3, 7, 16, 33, 64, 65, 130])
+        H = rng.randint(1, 40)
+        W = rng.choice([1, 2, 3, 4, 6, 7, 8, 10, 12, 14, 15, 16, 20, 24, 28, 30, 32, 36, 48, 56, 57, 64, 66,
+                        128, 130, 256, 258])
+        if H // s == 0 or W // s == 0:
+            continue
+        combine = rng.choice(['mul', 'add'])
+        case = random_case(N, C, H, W, 3, s, dtype, seed=chunk * 1000 + done)
+        check_against_oracle(*case, 3, 1, s, combine, '',
+                             what=str((N, C, H, W, s, combine, dtype)))
+        done += 1
+
+
 def test_tensors_beyond_2_31_elements():
     """66 x 512 x 256 x 256 fp16 is 2.2e9 elements: offsets no longer fit 32
     bits (the reference indexes with int, ddf_mul_cuda_kernel.cu:28-33).  The
