@@ -25,7 +25,9 @@ using torch::autograd::AutogradContext;
 using torch::autograd::variable_list;
 
 // `assert cond, msg` of the Python front end.
+// (Also reached from the autograd engine's threads, which do not hold the GIL.)
 [[noreturn]] void assertion_error(const std::string &msg) {
+    py::gil_scoped_acquire gil;
     PyErr_SetString(PyExc_AssertionError, msg.c_str());
     throw py::error_already_set();
 }

@@ -183,12 +183,47 @@ class DDFFunction(Function):
 # The operator callers use: the C++ autograd function of the torch extension
 # (csrc/torch/ddf_torch.cpp: same checks, same messages, same library calls,
 # without the interpreter in between) where it has been built, else the Python
-# Function above.  Both enqueue the same kernels.
-try:
-    from . import _C
-except ImportError:      # extension (or the library it links) not built
-    _C = None
-ddf = _C.ddf if _C is not None else DDFFunction.apply
+# Function above.  Both enqueue the same kernels.  The extension is looked up at
+# the first call rather than at import, so a process that imports the package
+# and builds the extension afterwards still picks it up.
+_C = None
+_C_missing = False
+
+
+def extension(retry=False):
+    """The torch extension module ``ddfnet_amd._C``, or None where it (or the
+    library it links) has not been built.  ``retry`` looks again after a miss."""
+    global _C, _C_missing
+    if _C is None and (retry or not _C_missing):
+        try:
+            import importlib
+            importlib.invalidate_caches()
+            _C = importlib.import_module(__package__ + '._C')
+        except ImportError:      # extension (or the library it links) not built
+            _C_missing = True
+    return _C
+
+
+_DDF_ARGS = ('features', 'channel_filter', 'spatial_filter', 'kernel_size', 'dilation', 'stride',
+             'kernel_combine', 'version')
+_DDF_DEFAULTS = {'kernel_size': 3, 'dilation': 1, 'stride': 1, 'kernel_combine': 'mul', 'version': ''}
+
+
+def ddf(*args, **kwargs):
+    """The operator, ``DDFFunction.apply`` of ``ddf/ddf.py:122``; arguments may
+    also be given by the names of ``DDFFunction.forward``."""
+    ext = extension()
+    if ext is not None:
+        return ext.ddf(*args, **kwargs)
+    if kwargs:
+        named = dict(_DDF_DEFAULTS)
+        named.update(zip(_DDF_ARGS, args))
+        for name in kwargs:
+            if name not in _DDF_ARGS or name in _DDF_ARGS[:len(args)]:
+                raise TypeError("ddf() got an unexpected or repeated argument '%s'" % name)
+        named.update(kwargs)
+        args = tuple(named[name] for name in _DDF_ARGS)
+    return DDFFunction.apply(*args)
 
 
 class DDFUpFunction(Function):
@@ -269,8 +304,9 @@ def ddf_up(features, channel_filters, spatial_filters, kernel_size=3, dilation=1
     channel_filters, spatial_filters = tuple(channel_filters), tuple(spatial_filters)
     assert len(channel_filters) == len(spatial_filters) == scale_factor ** 2
     if _lib.up_forward_covers(kernel_size, scale_factor):
-        if _C is not None:   # the same operator as a C++ autograd function
-            return _C.ddf_up(features, list(channel_filters), list(spatial_filters), kernel_size,
+        ext = extension()
+        if ext is not None:   # the same operator as a C++ autograd function
+            return ext.ddf_up(features, list(channel_filters), list(spatial_filters), kernel_size,
                              dilation, scale_factor, kernel_combine)
         return DDFUpFunction.apply(features, kernel_size, dilation, scale_factor, kernel_combine,
                                    *(channel_filters + spatial_filters))

@@ -12,7 +12,8 @@ import torch.nn.functional as F
 from torch.nn.init import calculate_gain
 
 from . import _lib
-from .functional import _C, ddf, ddf_up
+from . import functional
+from .functional import ddf, ddf_up
 
 __all__ = ['FilterNorm', 'build_spatial_branch', 'build_channel_branch',
            'DDFPack', 'DDFUpPack']
@@ -221,6 +222,10 @@ class DDFPack(nn.Module):
                                         any(p.requires_grad for p in self.parameters())):
             return None
         k = self.kernel_size
+        # (a size the stride does not divide: the op-by-op path fails at its reshape, as the
+        # reference does at ddf/ddf.py:215-218, and so must this one)
+        if x.dim() == 4 and (x.size(2) % self.stride or x.size(3) % self.stride):
+            return None
         if not (x.is_cuda and x.dim() == 4 and _lib.branches_cover(k, x.dtype) and
                 self._stock_channel_branch() and self._stock_spatial_branch()):
             return None
@@ -234,9 +239,10 @@ class DDFPack(nn.Module):
             return None
         if ch_norm.in_channels != x.size(1) or fc1.in_channels != x.size(1):
             return None
-        if _C is not None:
+        ext = functional.extension()
+        if ext is not None:
             # the same four launches without the interpreter in between
-            return _C.ddf_pack_forward(
+            return ext.ddf_pack_forward(
                 x, conv.weight, conv.bias,
                 1.0 if sp_norm.runing_std else sp_norm.std, tensors[6], tensors[7],
                 fc1.weight, fc1.bias, fc2.weight, fc2.bias,

@@ -7,8 +7,10 @@
  * dense NCHW ("contiguous") and live on the device that is current when the
  * call is made.  Calls are asynchronous: they enqueue kernels on `stream`
  * (a hipStream_t passed as void*, NULL = the default stream) and return
- * without synchronising.  The library keeps no global state and is
- * re-entrant; the caller owns every buffer.
+ * without synchronising.  The caller owns every buffer and the entry points
+ * are re-entrant; the only state the library keeps is the per-device scratch
+ * array of ddf_hip_backward_static (calls of that one entry point share it)
+ * and a thread-local text of the last error.
  *
  * Operator (r = (k-1)/2, Ho = H / s, Wo = W / s with floor division,
  * t = i*k + j, comb(a,b) = a*b for DDF_MUL and a+b for DDF_ADD; a term whose

@@ -650,9 +650,8 @@ def test_cpp_operator_equals_python_operator():
     built; DDFFunction is the Python one.  Same checks, same library calls:
     results and gradients are bit-identical."""
     from ddfnet_amd import DDFFunction, ddf, functional
-    if functional._C is None:
+    if functional.extension() is None:
         pytest.skip('torch extension not built')
-    assert ddf is functional._C.ddf
     for dtype in (torch.float32, torch.float16):
         for (N, C, H, W, k, d, s, combine) in [(2, 16, 14, 14, 3, 1, 1, 'mul'), (2, 8, 9, 11, 3, 2, 2, 'add'),
                                                (1, 4, 12, 12, 5, 1, 1, 'mul')]:

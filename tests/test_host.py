@@ -266,3 +266,34 @@ def test_bench_refuses_more_than_one_gpu():
                           capture_output=True, text=True, timeout=300)
     assert proc.returncode == 2
     assert 'one GPU' in proc.stderr and proc.stdout.strip() == ''
+
+
+def test_extension_built_after_import_is_picked_up(tmp_path):
+    """A process that imports the package before the torch extension exists (a
+    clean checkout calling build()) finds it once it has been built: the lookup
+    happens at use, a miss is remembered until asked to look again."""
+    import glob
+    import shutil
+    import subprocess
+    import sys
+    here = os.path.dirname(os.path.abspath(ddfnet_amd.__file__))
+    built = glob.glob(os.path.join(here, '_C*.so'))
+    if not built or not _lib.is_built():
+        pytest.skip('library or torch extension not built')
+    pkg = tmp_path / 'ddfnet_amd'
+    pkg.mkdir()
+    for path in glob.glob(os.path.join(here, '*.py')):
+        shutil.copy(path, pkg)
+    script = (
+        'import shutil, sys\n'
+        'import ddfnet_amd\n'
+        'from ddfnet_amd import functional\n'
+        'assert functional.extension() is None\n'
+        'for path in sys.argv[1:]:\n'
+        '    shutil.copy(path, %r)\n'
+        'assert functional.extension() is None\n'
+        'ext = functional.extension(retry=True)\n'
+        'assert ext is not None and hasattr(ext, "ddf")\n' % str(pkg))
+    env = dict(os.environ, PYTHONPATH=str(tmp_path))
+    subprocess.run([sys.executable, '-c', script, _lib.LIB_PATH] + built, check=True, env=env,
+                   cwd=str(tmp_path))

@@ -70,7 +70,7 @@ def test_ddfpack_inference_path_matches_cpu_reference(k, stride, head, c, hw, dt
         assert pack._inference_filters(x) is not None       # the one-launch branches do run
         out = pack(x)
         # the ctypes route of the same launches (what runs without the torch extension)
-        monkeypatch.setattr(ddf_modules, '_C', None)
+        monkeypatch.setattr(ddf_modules.functional, 'extension', lambda retry=False: None)
         cf, sf = pack._inference_filters(x)
         monkeypatch.undo()
         g = head
@@ -101,6 +101,20 @@ def test_ddfpack_inference_path_only_for_stock_branches():
         pack = ddfnet_amd.DDFPack(16).cuda()
         out = pack(x.half())                                          # fp16 features, fp32 parameters
         assert torch.isfinite(out).all()
+
+
+def test_ddfpack_odd_size_under_stride_fails_in_both_modes():
+    """A 1x1 convolution of stride s yields ceil(H / s) rows and the operator
+    wants H // s: the reference fails at its reshape (ddf/ddf.py:215-218), with
+    and without gradients."""
+    pack = ddfnet_amd.DDFPack(16, stride=2).cuda()
+    x = torch.randn(2, 16, 9, 8, device='cuda')
+    with torch.no_grad():
+        assert pack._inference_filters(x) is None
+        with pytest.raises(RuntimeError):
+            pack(x)
+    with pytest.raises(RuntimeError):
+        pack(x)
 
 
 def test_ddfuppack_matches_cpu_reference(monkeypatch):

@@ -70,3 +70,45 @@ def test_static_backward_rejects_what_does_not_fit():
                                      k, d, s, 0, _lib.DTYPE[dtype], 7, 0, None)
     assert rc == 3   # DDF_ERR_WORKSPACE
     assert b'ddf_hip_backward_static holds' in lib.ddf_hip_last_error()
+
+
+def test_static_backward_allocates_nothing_and_replays_in_a_graph():
+    """The reason the entry point exists: a call leaves the device's free memory and
+    torch's allocator untouched, and it can be recorded into a HIP graph (which
+    forbids allocation) and replayed."""
+    shape, k, d, s, combine, dtype, need = (8, 64, 14, 14), 3, 1, 1, 'mul', torch.float32, 7
+    N, C, H, W = shape
+    assert _lib.backward_workspace_bytes(shape, k, d, s, combine, dtype, need) > 0
+    x, cf, sf, go = (t.cuda() for t in random_case(N, C, H, W, k, s, dtype, seed=5))
+    lib = _lib.lib()
+    tail = (N, C, H, W, k, d, s, _lib.COMBINE[combine], _lib.DTYPE[dtype])
+    got = [torch.full_like(t, float('nan')) for t in (x, cf, sf)]
+
+    def call(stream):
+        rc = lib.ddf_hip_backward_static(_ptr(go), _ptr(x), _ptr(cf), _ptr(sf), _ptr(got[0]),
+                                         _ptr(got[1]), _ptr(got[2]), *tail, need, 0,
+                                         ctypes.c_void_p(stream.cuda_stream))
+        assert rc == 0, lib.ddf_hip_last_error()
+
+    call(torch.cuda.current_stream())        # first call on the device: looks the array up
+    torch.cuda.synchronize()
+    eager = [t.clone() for t in got]
+    free_before, allocated_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated()
+    reserved_before = torch.cuda.memory_reserved()
+    call(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.cuda.memory_allocated() == allocated_before
+    assert torch.cuda.memory_reserved() == reserved_before
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream())    # (the capture stream)
+    for _ in range(3):
+        for t in got:
+            t.fill_(float('nan'))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(('dX', 'dCF', 'dSF'), eager, got):
+            assert torch.equal(a, b), name
