@@ -59,8 +59,10 @@ __device__ __forceinline__ void wave_sync() {
 // S = 2 (3 x 3, one row per lane): g describes the dO plane, the lane's feature
 // vectors are 2 * VX elements wide (LaneStride2).  With DX the lane of result
 // row y also writes the feature gradient of feature rows 2y and 2y + 1.
+// SEG (with DX): image rows are cut into segments, whose outer lanes hold dO
+// values they do not own; those are kept out of the filter sums.
 template <typename T, int K, int D, bool MUL, int VX, int R, bool PAD, bool DX, int NST, int WPE,
-          int S = 1>
+          int S = 1, bool SEG = true>
 __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     RowsGeom g, const T *__restrict__ go, const T *__restrict__ x, const T *__restrict__ cf,
     const T *__restrict__ sf, T *__restrict__ dx, T *__restrict__ dcf, T *__restrict__ dsf,
@@ -74,6 +76,8 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
     constexpr int GROWS = DX ? (S == 2 ? 2 : ROWS) : R;
     constexpr int GOWN = DX && S == 1 ? HY : 0;
     constexpr bool kFilters = MUL || DX;       // CF and SF values are needed at all
+    // fp16 feature gradient: comb(CF, SF) of a pixel pair is formed by one packed fp16 operation
+    constexpr bool kPackedComb = sizeof(T) == 2 && DX && S == 1 && VX >= 2;
     constexpr int kVB = VX * sizeof(T), kXB = S * kVB;   // bytes of a dO / filter vector, of a feature vector
     constexpr int NW = vec_words(kVB), NWX = vec_words(kXB);
     constexpr int G = kFlushChannels;
@@ -314,20 +318,32 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
         }
         // dO at the lane's own pixels.  (DX loads dO through the window offsets, so a
         // lane that only reads for its neighbours - the outer lanes of a row segment -
-        // holds real values here: they must not enter the filter sums twice.)
+        // holds real values here: they must not enter the filter sums twice.  Without
+        // segments every lane that owns nothing reads zeros anyway.)
         A gval[R][VX];
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
             for (int e = 0; e < VX; ++e) {
                 const A v = elem<T>(gw[ST][GOWN + r], e);
-                gval[r][e] = (DX && ob[r] == kOutside) ? A(0) : v;
+                gval[r][e] = (DX && SEG && ob[r] == kOutside) ? A(0) : v;
             }
+        // Channel taps.  fp16: tap t comes over from lane t in storage format, as a
+        // wave-uniform pair (t, t); it widens inside the mixed-precision multiply-adds.
         A w[KK];
+        uint32_t wpk[kPackedComb ? KK : 1];
         if constexpr (kFilters) {
             if constexpr (kScalarTaps) {
 #pragma unroll
                 for (int t = 0; t < KK; ++t) w[t] = cfu[ST][t];
+            } else if constexpr (kPackedComb) {
+                const uint32_t bits = (uint32_t)__builtin_bit_cast(unsigned short, cfl[ST]);
+#pragma unroll
+                for (int t = 0; t < KK; ++t) {
+                    const uint32_t b = (uint32_t)__builtin_amdgcn_readlane((int)bits, t);
+                    wpk[t] = b | (b << 16);
+                    w[t] = (A)__builtin_bit_cast(half2_t, wpk[t])[0];
+                }
             } else {
                 const A cfa = (A)ld(&cfl[ST]);
 #pragma unroll
@@ -340,15 +356,17 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
         for (int i = 0; i < K; ++i)
 #pragma unroll
-            for (int j = 0; j < K; ++j)
+            for (int j = 0; j < K; ++j) {
+                const int t = i * K + j;
 #pragma unroll
                 for (int r = 0; r < R; ++r)
 #pragma unroll
                     for (int e = 0; e < VX; ++e) {
-                        const int t = i * K + j;
                         const A xv = row[r + i * D].at(S * e + j * D - HX);
                         if constexpr (MUL) {
-                            const A gx = gval[r][e] * xv;
+                            // (fp16: as a multiply-add the product takes both factors in
+                            // storage format; a plain multiply would widen them first)
+                            const A gx = sizeof(T) == 2 ? fma_(gval[r][e], xv, A(0)) : gval[r][e] * xv;
                             acc_sf[r][t][e] = fma_(gx, w[t], acc_sf[r][t][e]);
                             pcf[t] = fma_(gx, elem<T>(sfw[r][t], e), pcf[t]);
                         } else {
@@ -357,14 +375,17 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                             pcf[t] = fma_(gval[r][e], xv, pcf[t]);
                         }
                     }
-        // The accumulators are not read before the walk ends: without this the compiler
-        // moves every update behind the flush branch and keeps (spills) the products.
+                // One tap at a time, so that its products die with it (left alone, the
+                // scheduler forms the products of all taps first: K*K*R*VX registers).
+                // The accumulators are not read before the walk ends: without the pin the
+                // compiler moves every update behind the flush branch and spills the products.
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+                for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int t = 0; t < KK; ++t)
-#pragma unroll
-                for (int e = 0; e < VX; ++e) asm volatile("" : "+v"(acc_sf[r][t][e]));
+                    for (int e = 0; e < VX; ++e) asm volatile("" : "+v"(acc_sf[r][t][e]));
+                asm volatile("" : "+v"(pcf[t]));
+                __builtin_amdgcn_sched_barrier(0);
+            }
         if constexpr (DX && S == 2) {
             // feature gradient of the lane's two feature rows: the four parity classes
             // of a feature pixel see one, two, two and four taps
@@ -422,7 +443,24 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
 #pragma unroll
                 for (int i = 0; i < K; ++i)
 #pragma unroll
-                    for (int j = 0; j < K; ++j)
+                    for (int j = 0; j < K; ++j) {
+                      if constexpr (kPackedComb) {
+                        // fp16: the combined filter of two pixels in one packed operation
+                        // (rounded to fp16 like the operands), then one multiply-add per pixel
+                        const int t = i * K + j;
+                        const half2_t wv = __builtin_bit_cast(half2_t, wpk[KK - 1 - t]);
+#pragma unroll
+                        for (int k = 0; k < NW; ++k) {
+                            const half2_t sv2 = __builtin_bit_cast(half2_t, sfg[r][t][k]);
+                            const half2_t cb = MUL ? wv * sv2 : wv + sv2;
+#pragma unroll
+                            for (int h = 0; h < 2; ++h) {
+                                const int e = 2 * k + h;
+                                const A gv = grow[r + i * D].at(e + j * D - HX);
+                                accx[e] = fma_(gv, (A)cb[h], accx[e]);
+                            }
+                        }
+                      } else {
 #pragma unroll
                         for (int e = 0; e < VX; ++e) {
                             const int t = i * K + j;
@@ -435,6 +473,8 @@ __global__ __launch_bounds__(kWave * kFilterWaves, WPE) void k_rows_filters(
                                 accx[e] = fma_(gv, sv, accx[e]);
                             }
                         }
+                      }
+                    }
                 if constexpr (sizeof(T) == 2) {
                     // round the complete fp32 sum, the same way in every unrolled copy (see k_rows)
 #pragma unroll

@@ -147,17 +147,21 @@ hipError_t launch_filters_v(const Problem &p, const RowsGeom &g, const T *go, co
     const int lds = filters_lds_bytes<9>((int)sizeof(A), R, VX);
     if (p.k != 3 || (p.d != 1 && p.d != 2)) return hipErrorNotSupported;
     const bool pad = rows_shift_in_as_is(g);
-#define DDF_ROWSF_CASE(D_, MUL_, PAD_)                                                           \
+    // (row segments: only the launch that also writes the feature gradient tells them apart)
+    const bool seg = DX && g.segs > 0;
+#define DDF_ROWSF_CASE(D_, MUL_, PAD_, SEG_)                                                     \
     hipLaunchKernelGGL((k_rows_filters<T, 3, D_, MUL_, VX, R, PAD_, DX, kFilterStages,           \
-                                       MUL_ ? WPE_MUL : WPE_ADD>),                               \
+                                       MUL_ ? WPE_MUL : WPE_ADD, 1, SEG_>),                      \
                        grid, block, lds, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, x_mod)
 #define DDF_ROWSF_D(D_)                                                                          \
     if (p.mul) {                                                                                 \
-        if (pad) DDF_ROWSF_CASE(D_, true, true);                                                 \
-        else DDF_ROWSF_CASE(D_, true, false);                                                    \
+        if (seg) DDF_ROWSF_CASE(D_, true, true, true);                                           \
+        else if (pad) DDF_ROWSF_CASE(D_, true, true, false);                                     \
+        else DDF_ROWSF_CASE(D_, true, false, false);                                             \
     } else {                                                                                     \
-        if (pad) DDF_ROWSF_CASE(D_, false, true);                                                \
-        else DDF_ROWSF_CASE(D_, false, false);                                                   \
+        if (seg) DDF_ROWSF_CASE(D_, false, true, true);                                          \
+        else if (pad) DDF_ROWSF_CASE(D_, false, true, false);                                    \
+        else DDF_ROWSF_CASE(D_, false, false, false);                                            \
     }
     if (p.d == 1) {
         DDF_ROWSF_D(1)
@@ -184,7 +188,7 @@ hipError_t launch_filters_stride2_v(const Problem &p, const RowsGeom &g, const T
     const int lds = filters_lds_bytes<9>((int)sizeof(A), 1, VX);
     const bool pad = rows_shift_in_as_is(g);
 #define DDF_ROWSF_CASE(MUL_, PAD_)                                                               \
-    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, 1, PAD_, DX, kStagesS2, kWpe, 2>),     \
+    hipLaunchKernelGGL((k_rows_filters<T, 3, 1, MUL_, VX, 1, PAD_, DX, kStagesS2, kWpe, 2, false>), \
                        grid, block, lds, st, g, go, x, cf, sf, dx, dcf, dsf, ws_sf, ws_cf, need, 0)
     if (p.mul) {
         if (pad) DDF_ROWSF_CASE(true, true);
