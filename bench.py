@@ -25,8 +25,10 @@ The same line carries the other benchmark configurations
 (``other_workloads``: the fp16 'add' stage-1 shape, the strided and the
 dilated 5x5 shapes, two more ResNet stages), ddf_mul_resnet50 inference
 (``model_inference``: fp16, batch 128, 224x224, random weights: images/s and
-per-layer GB/s of the DDF layers) and the CPU baseline; ``--only-headline``
-leaves the first two out.
+per-layer GB/s of the DDF layers, operands rotating beyond the last-level
+cache), a DDFPack layer as a training unit (``ddfpack_train``), the fused
+up-sampling forward (``up_forward``) and the CPU baseline; ``--only-headline``
+leaves all but the last out.
 
 Prints ONE JSON line on stdout; everything else goes to stderr.
 """
@@ -193,6 +195,26 @@ def profiled_traffic(workload, phase, kernels):
         for m in pat.finditer(text):
             if m.group(1) == workload and m.group(2) == phase and m.group(3) == kernels:
                 return int(m.group(4)), os.path.relpath(path, ROOT)
+    return None, None
+
+
+def profiled_kernel_us(workload, phase, kernels):
+    """Sum of the traced durations of the kernels of one library call, as recorded in
+    profiles/*.md by lines of the form
+        KERNELTIME workload=<name> phase=<fwd|bwd> kernels="<names>" us=<microseconds>
+    (rocprofv3 --kernel-trace --stats of the same call: average duration of each
+    kernel times its launches per call).  Returns (us, file name) or (None, None)."""
+    import glob
+    import re
+    pat = re.compile(r'KERNELTIME workload=(\S+) phase=(\S+) kernels="([^"]*)" us=([0-9.]+)')
+    for path in sorted(glob.glob(os.path.join(ROOT, 'profiles', '*.md'))):
+        try:
+            text = open(path).read()
+        except OSError:
+            continue
+        for m in pat.finditer(text):
+            if m.group(1) == workload and m.group(2) == phase and m.group(3) == kernels:
+                return float(m.group(4)), os.path.relpath(path, ROOT)
     return None, None
 
 
@@ -434,6 +456,63 @@ def test_time_table(iters=20, warmup=5):
     return rows
 
 
+def pack_train_table(iters=30, warmup=8):
+    """DDFPack (ddf/ddf.py:195-222) as a training unit: forward + backward (input and
+    parameter gradients) of one layer at the three stride-1 ResNet-50 stage shapes, fp32
+    and fp16.  `fused`: the spatial filter normalisation and the operator as one autograd
+    node whose backward pushes dSF through the normalisation inside the partial-sum
+    launch (the default); `op_by_op`: the normalisation as a module of its own in front
+    of the operator, as in the reference.  A step is host-bound at these sizes (about
+    thirty launches issued from Python), so beside the time per step the table gives the
+    launches per step and the summed durations of their kernels, both from torch's
+    profiler (null where that is not available)."""
+    from ddfnet_amd import DDFPack
+    shapes = [(64, 64, 56, 56), (64, 128, 28, 28), (64, 256, 14, 14)]
+    rows = []
+
+    def launches(step):
+        """(kernel launches, summed kernel durations in us) of one step."""
+        try:
+            from torch.profiler import profile, ProfilerActivity
+            with profile(activities=[ProfilerActivity.CUDA]) as prof:
+                step()
+                torch.cuda.synchronize()
+            kernels = [e for e in prof.events() if getattr(e, 'device_type', None) is not None and
+                       str(e.device_type).endswith('CUDA')]
+            return len(kernels), round(sum(e.time_range.elapsed_us() for e in kernels), 1)
+        except Exception:    # profiler back end missing on this box
+            return None, None
+
+    for dtype in (torch.float32, torch.float16):
+        for n, c, h, w in shapes:
+            torch.manual_seed(0)
+            layer = DDFPack(c).cuda().to(dtype).train()
+            x = torch.randn(n, c, h, w, device='cuda').to(dtype).requires_grad_(True)
+            go = torch.randn(n, c, h, w, device='cuda').to(dtype)
+            row = {'shape': [n, c, h, w], 'dtype': DTYPE_NAME[dtype]}
+            for name, fused in (('fused', True), ('op_by_op', False)):
+                layer.fuse_spatial_norm = fused
+
+                def step():
+                    layer.zero_grad(set_to_none=True)
+                    x.grad = None
+                    layer(x).backward(go)
+
+                for _ in range(warmup):
+                    step()
+                row[name + '_us'] = round(timed(lambda i: step(), iters) * 1e3, 1)
+                row[name + '_launches'], row[name + '_kernel_us'] = launches(step)
+            rows.append(row)
+            log('[pack-train] DDFPack(%d) %s %s: fused %.1f us per step (%s launches, %s us of kernels), '
+                'op by op %.1f us (%s launches, %s us of kernels)' % (
+                    c, row['shape'], row['dtype'], row['fused_us'], row['fused_launches'],
+                    row['fused_kernel_us'], row['op_by_op_us'], row['op_by_op_launches'],
+                    row['op_by_op_kernel_us']))
+            del layer, x, go
+            torch.cuda.empty_cache()
+    return rows
+
+
 def up_forward_table(lib, iters=50, warmup=10):
     """The up-sampling operator of DDFUpPack (ddf/ddf.py:264-272), forward only:
     one fused launch against the reference's composition (one ddf call per
@@ -491,11 +570,23 @@ def roofline_of(res):
     sec = res['phase_ms'][dominant] * 1e-3
     achieved = nbytes / sec / 1e9
     traffic, source = profiled_traffic(res['workload'], dominant, res['kernels'][dominant])
-    return {'bound': 'hbm', 'phase': dominant, 'kernel': res['kernels'][dominant],
-            'achieved': round(achieved, 2), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
-            'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': traffic,
-            'traffic_source': source, 'bytes_per_launch': nbytes,
-            'avg_launch_us': round(sec * 1e6, 3)}
+    out = {'bound': 'hbm', 'phase': dominant, 'kernel': res['kernels'][dominant],
+           'achieved': round(achieved, 2), 'peak': HBM_PEAK_GBPS, 'unit': 'GB/s',
+           'frac': round(achieved / HBM_PEAK_GBPS, 4), 'traffic': traffic,
+           'traffic_source': source, 'bytes_per_launch': nbytes,
+           'avg_launch_us': round(sec * 1e6, 3)}
+    # The same fraction from the committed kernel trace: algorithmic bytes / summed traced
+    # kernel durations.  It is lower than `frac` where a call is several kernels: the
+    # trace adds their durations up, while on the stream the next kernel's start
+    # overlaps the previous one's drain, which the events around the call see.
+    prof_us, prof_src = profiled_kernel_us(res['workload'], dominant, res['kernels'][dominant])
+    if prof_us:
+        out['profile_kernel_us'] = prof_us
+        out['frac_from_profile'] = round(nbytes / (prof_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+        out['profile_source'] = prof_src
+        out['frac_note'] = ('frac: events around back-to-back calls in this run; frac_from_profile: '
+                            'summed kernel durations of the committed rocprofv3 trace')
+    return out
 
 
 def workload_summary(r):
@@ -527,7 +618,8 @@ def main():
                     help="also run the reference's micro-benchmark table (conv, depthwise conv, "
                          "DDFPack, ddf at seven 256-channel shapes)")
     ap.add_argument('--up-pack', action='store_true',
-                    help='also time the fused up-sampling forward against its composition')
+                    help='with --only-headline: also time the fused up-sampling forward against its '
+                         'composition (part of the default line otherwise)')
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--profile-phase', choices=PHASES, default=None,
                     help='run only this library call of the workload (warm-up + steps calls, then the '
@@ -590,10 +682,13 @@ def main():
         log('[model] %s bs%d %s: %.1f images/s (%.2f ms/batch, DDF layers %.2f ms)' % (
             mi['model'], mi['batch'], mi['dtype'], mi['images_per_s'], mi['ms_per_batch'],
             mi['ddf_ms_per_batch']))
+    if not args.only_headline:
+        line['ddfpack_train'] = pack_train_table()
+        line['up_forward'] = up_forward_table(lib)
+    elif args.up_pack:
+        line['up_forward'] = up_forward_table(lib)
     if args.test_time:
         line['test_time'] = test_time_table()
-    if args.up_pack:
-        line['up_forward'] = up_forward_table(lib)
     if not args.no_cpu:
         line['cpu_baseline'] = cpu_baseline(args.workload)
         cb = line['cpu_baseline']

@@ -29,6 +29,9 @@ SYMBOLS = {
     'ddf_hip_backward_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u, _i]),
     'ddf_hip_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
     'ddf_hip_backward_static': (_i, [_vp] * 7 + [_i64] * 4 + [_i] * 5 + [_u, _i, _vp]),
+    'ddf_hip_backward_spatial_norm_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u, _i]),
+    'ddf_hip_backward_spatial_norm': (_i, [_vp] * 10 + [_sz] + [_i64] * 4 + [_i] * 5 +
+                                      [_u, _i, ctypes.c_double, _vp, _i, _vp]),
     'ddf_hip_filter_norm': (_i, [_vp] * 2 + [_i64] * 2 + [_i, _i64, ctypes.c_double] + [_vp] * 2 +
                             [_i, _vp]),
     'ddf_hip_filter_norm_backward': (_i, [_vp] * 4 + [_i64] * 2 + [_i, _i64, ctypes.c_double, _vp,
@@ -143,6 +146,23 @@ def backward(grad_output, features, channel_filter, spatial_filter, grad_feature
         _ptr(grad_features), _ptr(grad_channel_filter), _ptr(grad_spatial_filter),
         _ptr(workspace), ws_bytes, N, C, H, W, k, d, s, COMBINE[combine],
         DTYPE[features.dtype], need, VARIANT[variant], _stream()))
+
+
+def backward_spatial_norm(grad_output, features, channel_filter, spatial_filter, raw_spatial_filter,
+                          grad_features, grad_channel_filter, grad_raw_spatial_filter, gain_terms,
+                          k, d, s, combine, need, groups, gain, gain_vec=None, variant=''):
+    """``backward`` with the spatial filter normalisation behind dSF: writes the
+    gradient with respect to the raw (un-normalised) spatial filter.  Allocates
+    its workspace from torch's caching allocator."""
+    N, C, H, W = features.shape
+    tail = (N, C, H, W, k, d, s, COMBINE[combine], DTYPE[features.dtype])
+    nbytes = lib().ddf_hip_backward_spatial_norm_workspace_bytes(*tail, need, VARIANT[variant])
+    workspace = (torch.empty(nbytes, dtype=torch.uint8, device=features.device) if nbytes else None)
+    check(lib().ddf_hip_backward_spatial_norm(
+        _ptr(grad_output), _ptr(features), _ptr(channel_filter), _ptr(spatial_filter),
+        _ptr(raw_spatial_filter), _ptr(grad_features), _ptr(grad_channel_filter),
+        _ptr(grad_raw_spatial_filter), _ptr(gain_terms), _ptr(workspace), nbytes, *tail, need,
+        groups, float(gain), _ptr(gain_vec), VARIANT[variant], _stream()))
 
 
 def filter_norm(x, outer, groups, taps, inner, gain, gain_vec=None, offset_vec=None):

@@ -106,6 +106,47 @@ int backward_typed(const ddf::Problem &p, const void *go, const void *x, const v
 
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
+// ddf_hip_backward with the spatial filter normalisation behind dSF.  The
+// workspace starts with room for a complete dSF (storage type); the rest is the
+// backward pass's own.
+template <typename T>
+int backward_norm_typed(const ddf::Problem &p, const void *go, const void *x, const void *cf,
+                        const void *sf, const void *raw, void *dx, void *dcf, void *d_raw,
+                        void *terms, void *ws, size_t ws_bytes, int dtype, unsigned need,
+                        int groups, double gain, const void *gain_vec, int variant,
+                        hipStream_t stream) {
+    const size_t n_sf = (size_t)(p.N * p.kk * p.Ho * p.Wo);
+    const size_t tmp_bytes = (need & DDF_NEED_DSF) ? align256(n_sf * sizeof(T)) : 0;
+    const bool tiled = variant != DDF_VARIANT_GENERIC && ddf::tiled_backward_supported(p, dtype);
+    const size_t inner = tiled ? ddf::tiled_backward_workspace(p, dtype, need) : 0;
+    if (tmp_bytes + inner > 0 && (ws == nullptr || ws_bytes < tmp_bytes + inner))
+        return fail(DDF_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", tmp_bytes + inner,
+                    ws == nullptr ? (size_t)0 : ws_bytes);
+    if (tmp_bytes + inner > 0 && ((uintptr_t)ws & 255u) != 0)
+        return fail(DDF_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+    T *tmp = tmp_bytes ? static_cast<T *>(ws) : nullptr;
+    void *rest = inner ? static_cast<unsigned char *>(ws) + tmp_bytes : nullptr;
+    ddf::NormTail<T> tail{(const T *)raw, (T *)d_raw, (T *)terms, (const T *)gain_vec, groups, gain,
+                          false};
+    hipError_t err;
+    if (tiled)
+        err = ddf::tiled_backward<T>(p, (const T *)go, (const T *)x, (const T *)cf, (const T *)sf,
+                                     (T *)dx, (T *)dcf, tmp, rest, need, stream,
+                                     (need & DDF_NEED_DSF) ? &tail : nullptr);
+    else
+        err = ddf::generic_backward<T>(p, (const T *)go, (const T *)x, (const T *)cf, (const T *)sf,
+                                       (T *)dx, (T *)dcf, tmp, need, stream);
+    if (err != hipSuccess) return fail_hip(err, "ddf_hip_backward_spatial_norm launch");
+    if ((need & DDF_NEED_DSF) && !tail.applied) {
+        // (no pass over dSF to ride on: the normalisation's gradient as a launch of its own)
+        err = ddf::filter_norm_backward<T>(tmp, (const T *)raw, (T *)d_raw, (T *)terms,
+                                           p.N / groups, groups, p.kk, p.Ho * p.Wo, gain,
+                                           (const T *)gain_vec, stream);
+        if (err != hipSuccess) return fail_hip(err, "ddf_hip_backward_spatial_norm norm launch");
+    }
+    return DDF_OK;
+}
+
 // Address of `scratch` on the current device, looked up once per device (with
 // that device current) and kept.
 constexpr int kMaxDevices = 64;
@@ -263,6 +304,7 @@ int ddf_hip_describe(int64_t N, int64_t C, int64_t H, int64_t W, int kernel_size
     const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
     if (N * C * p.Ho * p.Wo == 0) { snprintf(buffer, buffer_len, "nothing"); return DDF_OK; }
     const unsigned need = need_mask & DDF_NEED_ALL;
+    const bool norm = (need_mask & DDF_DESCRIBE_SPATIAL_NORM) && (need & DDF_NEED_DSF);
     if (need == 0) {
         if (variant == DDF_VARIANT_GENERIC || !ddf::tiled_forward_supported(p, dtype))
             snprintf(buffer, buffer_len, "generic_forward");
@@ -270,9 +312,10 @@ int ddf_hip_describe(int64_t N, int64_t C, int64_t H, int64_t W, int kernel_size
             ddf::describe_forward(p, dtype, buffer, buffer_len);
     } else {
         if (variant == DDF_VARIANT_GENERIC || !ddf::tiled_backward_supported(p, dtype))
-            snprintf(buffer, buffer_len, "generic_backward");
+            snprintf(buffer, buffer_len, norm ? "generic_backward + k_filter_norm_backward" : "generic_backward");
         else
-            ddf::describe_backward(p, dtype, need, buffer, buffer_len);
+            ddf::describe_backward(p, dtype, need | (norm ? DDF_DESCRIBE_SPATIAL_NORM : 0u), buffer,
+                                   buffer_len);
     }
     return DDF_OK;
 }
@@ -355,6 +398,60 @@ int ddf_hip_backward(const void *grad_output, const void *features,
                                           grad_spatial_filter, workspace, workspace_bytes,
                                           dtype, need, variant, st);
     }
+}
+
+size_t ddf_hip_backward_spatial_norm_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W,
+                                                     int kernel_size, int dilation, int stride,
+                                                     int combine, int dtype, unsigned need_mask,
+                                                     int variant) {
+    if (check_problem(N, C, H, W, kernel_size, dilation, stride, combine, dtype, variant) != DDF_OK)
+        return 0;
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
+    const size_t esz = dtype == DDF_F16 ? 2 : dtype == DDF_F32 ? 4 : 8;
+    const size_t tmp = (need_mask & DDF_NEED_DSF) ? align256((size_t)(N * p.kk * p.Ho * p.Wo) * esz) : 0;
+    return tmp + ddf_hip_backward_workspace_bytes(N, C, H, W, kernel_size, dilation, stride, combine,
+                                                  dtype, need_mask, variant);
+}
+
+int ddf_hip_backward_spatial_norm(const void *grad_output, const void *features,
+                                  const void *channel_filter, const void *spatial_filter,
+                                  const void *raw_spatial_filter, void *grad_features,
+                                  void *grad_channel_filter, void *grad_raw_spatial_filter,
+                                  void *gain_terms, void *workspace, size_t workspace_bytes,
+                                  int64_t N, int64_t C, int64_t H, int64_t W, int kernel_size,
+                                  int dilation, int stride, int combine, int dtype,
+                                  unsigned need_mask, int groups, double gain, const void *gain_vec,
+                                  int variant, void *stream) {
+    int rc = check_problem(N, C, H, W, kernel_size, dilation, stride, combine, dtype, variant);
+    if (rc != DDF_OK) return rc;
+    const unsigned need = need_mask & DDF_NEED_ALL;
+    if (need == 0 || N == 0) return DDF_OK;
+    if (groups < 1 || N % groups != 0)
+        return fail(DDF_ERR_BAD_ARG, "groups must be >= 1 and divide N (got %d, N=%lld)", groups,
+                    (long long)N);
+    const ddf::Problem p = ddf::make_problem(N, C, H, W, kernel_size, dilation, stride, combine);
+    const int64_t n_x = N * C * H * W, n_o = N * C * p.Ho * p.Wo;
+    const int64_t n_cf = N * C * p.kk, n_sf = N * p.kk * p.Ho * p.Wo;
+    if ((!grad_output && n_o) || (!features && n_x) || (!channel_filter && n_cf) ||
+        (!spatial_filter && n_sf))
+        return fail(DDF_ERR_BAD_ARG, "null input tensor pointer");
+    if ((need & DDF_NEED_DSF) && n_sf && (!raw_spatial_filter || !grad_raw_spatial_filter))
+        return fail(DDF_ERR_BAD_ARG, "null pointer for the raw spatial filter or its gradient");
+    if (((need & DDF_NEED_DX) && !grad_features && n_x) ||
+        ((need & DDF_NEED_DCF) && !grad_channel_filter && n_cf))
+        return fail(DDF_ERR_BAD_ARG, "null pointer for a requested gradient");
+    hipStream_t st = (hipStream_t)stream;
+#define DDF_NORM_CASE(T_)                                                                          \
+    return backward_norm_typed<T_>(p, grad_output, features, channel_filter, spatial_filter,       \
+                                   raw_spatial_filter, grad_features, grad_channel_filter,         \
+                                   grad_raw_spatial_filter, gain_terms, workspace, workspace_bytes, \
+                                   dtype, need, groups, gain, gain_vec, variant, st)
+    switch (dtype) {
+        case DDF_F16: DDF_NORM_CASE(__half);
+        case DDF_F32: DDF_NORM_CASE(float);
+        default: DDF_NORM_CASE(double);
+    }
+#undef DDF_NORM_CASE
 }
 
 int ddf_hip_backward_static(const void *grad_output, const void *features,

@@ -45,6 +45,24 @@ __device__ __forceinline__ A comb(A a, A b) { return MUL ? a * b : a + b; }
 
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// The spatial filter normalisation behind the spatial-filter gradient (FilterNorm
+// of the spatial branch, ddf/ddf.py:146-157 of the reference: the operator's
+// spatial filter is gain * standardised(raw) over the k*k taps of a pixel).  A
+// backward pass that is handed one pushes dSF through the normalisation's
+// Jacobian in the pass that adds up its partial sums and writes d_raw instead;
+// `applied` tells the caller whether that happened (else dSF is complete where
+// the pass was told to put it, and the caller runs filter_norm_backward).
+template <typename T>
+struct NormTail {
+    const T *raw;          // (N, k*k, Ho, Wo), before the normalisation
+    T *d_raw;              // gradient with respect to raw
+    T *terms;              // nullable: dSF * standardised(raw), summed by the caller into the gain_vec gradient
+    const T *gain_vec;     // nullable: (groups, k*k); sample n uses group n % groups
+    int groups;
+    double gain;           // used when gain_vec is null
+    bool applied;
+};
+
 // Launchers.  Each returns a hipError_t from the launch (hipSuccess when the
 // tensor is empty and nothing was launched).  `supported` queries tell the
 // API layer whether the tiled family covers a problem.
@@ -147,7 +165,7 @@ bool rows_cover_stride2_filters(const Problem &p, int dtype);
 template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
                                T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st,
-                               int x_mod = 0);
+                               int x_mod = 0, NormTail<T> *norm = nullptr);
 // The whole backward pass of such a batch on the row-register kernels, or
 // hipErrorNotSupported before anything is launched (shape or alignment not
 // covered).  `ws`: rows_filters_workspace(p) bytes.
@@ -171,6 +189,6 @@ size_t tiled_backward_workspace(const Problem &p, int dtype, unsigned need);
 template <typename T>
 hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf,
                           const T *sf, T *dx, T *dcf, T *dsf, void *ws,
-                          unsigned need, hipStream_t st);
+                          unsigned need, hipStream_t st, NormTail<T> *norm = nullptr);
 
 }  // namespace ddf

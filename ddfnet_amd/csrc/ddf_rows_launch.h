@@ -251,7 +251,7 @@ hipError_t launch_taprow_v(const Problem &p, const RowsGeom &g, const T *go, con
 template <typename T>
 hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
                                T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st,
-                               int x_mod) {
+                               int x_mod, NormTail<T> *norm) {
     using A = typename Acc<T>::type;
     const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
     const bool fused = dx != nullptr;
@@ -319,7 +319,8 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
     }
     if (err != hipSuccess) return err;
     return wave::sum_filter_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, ws_cf, dcf,
-                                        p.N * p.C, g.nstrips, (int64_t)p.kk, st);
+                                        p.N * p.C, g.nstrips, (int64_t)p.kk, st,
+                                        (need & DDF_NEED_DSF) ? norm : nullptr);
 }
 
 template <typename T>
@@ -359,7 +360,7 @@ hipError_t rows_backward_shared_features(const Problem &p, int x_mod, const T *g
 #define DDF_INSTANTIATE_ROWS(T)                                                              \
     template hipError_t rows_filters_launch<T>(const Problem &, const T *, const T *, const T *, \
                                                const T *, T *, T *, T *, void *, unsigned,   \
-                                               hipStream_t, int);                             \
+                                               hipStream_t, int, NormTail<T> *);              \
     template hipError_t rows_launch<T>(const Problem &, bool, const T *, const T *, const T *, \
                                        T *, hipStream_t);                                     \
     template hipError_t rows_backward_shared_features<T>(const Problem &, int, const T *,    \

@@ -170,7 +170,8 @@ hipError_t tiled_forward(const Problem &p, const T *x, const T *cf, const T *sf,
 
 template <typename T>
 hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf, const T *sf,
-                          T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st) {
+                          T *dx, T *dcf, T *dsf, void *ws, unsigned need, hipStream_t st,
+                          NormTail<T> *norm) {
     using A = typename Acc<T>::type;
     const int dtype = sizeof(T) == 2 ? DDF_F16 : sizeof(T) == 4 ? DDF_F32 : DDF_F64;
     hipError_t err = hipSuccess;
@@ -180,7 +181,7 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     if constexpr (sizeof(T) != 8) {
         // the row-register kernel does the whole backward pass in one launch where it covers it
         if ((need & DDF_NEED_DX) && fneed && tune_int("DDF_TUNE_ROWSF", 1) != 0) {
-            err = rows_filters_launch<T>(p, go, x, cf, sf, dx, dcf, dsf, ws, fneed, st);
+            err = rows_filters_launch<T>(p, go, x, cf, sf, dx, dcf, dsf, ws, fneed, st, 0, norm);
             if (err != hipErrorNotSupported) return err;
             err = hipSuccess;
         }
@@ -227,7 +228,8 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
     if (fneed && !fuse) {
         if constexpr (sizeof(T) != 8) {
             if (tune_int("DDF_TUNE_ROWSF", 1) != 0) {
-                err = rows_filters_launch<T>(p, go, x, cf, sf, (T *)nullptr, dcf, dsf, ws, fneed, st);
+                err = rows_filters_launch<T>(p, go, x, cf, sf, (T *)nullptr, dcf, dsf, ws, fneed, st, 0,
+                                             norm);
                 if (err != hipErrorNotSupported) return err;
                 err = hipSuccess;
             }
@@ -256,7 +258,8 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
         if (err != hipSuccess) return err;
         // dSF[n, t, pix] = sum over channel splits, dCF[nc, t] = sum over strips
         err = wave::sum_filter_partials<T>(ws_sf, dsf, p.N, g.csplit, p.kk * p.Ho * p.Wo, ws_cf, dcf,
-                                           p.N * p.C, g.nstrips, (int64_t)p.kk, st);
+                                           p.N * p.C, g.nstrips, (int64_t)p.kk, st,
+                                           (fneed & DDF_NEED_DSF) ? norm : nullptr);
         if (err != hipSuccess) return err;
     }
     return err;
@@ -267,6 +270,6 @@ hipError_t tiled_backward(const Problem &p, const T *go, const T *x, const T *cf
                                          T *, hipStream_t);                               \
     template hipError_t tiled_backward<T>(const Problem &, const T *, const T *, const T *, \
                                           const T *, T *, T *, T *, void *, unsigned,     \
-                                          hipStream_t);
+                                          hipStream_t, NormTail<T> *);
 
 }  // namespace ddf

@@ -1147,6 +1147,62 @@ __global__ __launch_bounds__(256) void k_sum_partials(
     sum_partials_block<T, VEC>(part, out, outer, parts, inner, blockIdx.x);
 }
 
+// dSF of a pixel = sum of its partial sums (PT: the accumulator type, or - one
+// part, written by the filter kernel itself - the storage type), pushed through
+// the Jacobian of the spatial filter normalisation (see k_filter_norm_backward):
+// with c_t = raw_t - mean, inv = 1 / (sd + 1e-10), gy_t = dSF_t * gain_t,
+//   d_raw_t = inv * (gy_t - mean(gy)) - c_t * inv^2 * sum(gy * c) / (sd * (KK - 1)).
+// One thread per pixel of one sample; neighbouring threads are neighbouring
+// pixels, so every tap plane is read and written with coalesced accesses.
+template <typename T, typename PT, int KK>
+__device__ __forceinline__ void sum_norm_block(const PT *__restrict__ part, int parts, int64_t n_samples,
+                                               int64_t plane, const T *__restrict__ raw,
+                                               T *__restrict__ d_raw, T *__restrict__ terms,
+                                               const T *__restrict__ gain_vec, int groups,
+                                               typename Acc<T>::type gain, unsigned block) {
+    using A = typename Acc<T>::type;
+    const int64_t idx = (int64_t)block * 256 + threadIdx.x;
+    if (idx >= n_samples * plane) return;
+    const int64_t n = idx / plane, pix = idx - n * plane;
+    const PT *src = part + n * parts * KK * plane + pix;
+    A gy[KK];
+#pragma unroll
+    for (int t = 0; t < KK; ++t) gy[t] = 0;
+    for (int q = 0; q < parts; ++q) {
+        PT v[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) v[t] = src[((int64_t)q * KK + t) * plane];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) gy[t] += (A)v[t];
+    }
+    const int64_t base = n * KK * plane + pix;
+    A c[KK];
+    A sum = 0;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) { c[t] = (A)ld(raw + base + t * plane); sum += c[t]; }
+    const A mean = sum / (A)KK;
+    const int64_t grp = n % groups;
+    A sq = 0, s1 = 0, s2 = 0;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        c[t] -= mean;
+        const A w = gain_vec ? (A)ld(gain_vec + grp * KK + t) : gain;
+        sq += c[t] * c[t];
+        s1 += gy[t] * w;
+        s2 += gy[t] * w * c[t];
+    }
+    const A sd = sqrt(sq / (A)(KK - 1));
+    const A inv = (A)1 / (sd + (A)1e-10);
+    const A m1 = s1 / (A)KK;
+    const A k2 = inv * inv * s2 / (sd * (A)(KK - 1));
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        const A w = gain_vec ? (A)ld(gain_vec + grp * KK + t) : gain;
+        st(d_raw + base + t * plane, inv * (gy[t] * w - m1) - c[t] * k2);
+        if (terms) st(terms + base + t * plane, gy[t] * c[t] * inv);
+    }
+}
+
 // One sum of partials: the arguments of k_sum_partials and the blocks it takes.
 template <typename T>
 struct SumJob {
@@ -1192,14 +1248,64 @@ inline hipError_t sum_partials(const typename Acc<T>::type *part, T *out, int64_
     return hipGetLastError();
 }
 
+// The dSF sum with the spatial filter normalisation behind it (sum_norm_block) and,
+// in the same launch, the dCF sum b (b.blocks == 0: none).  The dSF parts are
+// `parts` partial sums in the accumulator type, or (part_t) one part in the
+// storage type.
+template <typename T, int KK>
+__global__ __launch_bounds__(256) void k_sum_norm_pair(
+    const typename Acc<T>::type *__restrict__ part_a, const T *__restrict__ part_t, int parts,
+    int64_t n_samples, int64_t plane, const T *__restrict__ raw, T *__restrict__ d_raw,
+    T *__restrict__ terms, const T *__restrict__ gain_vec, int groups,
+    typename Acc<T>::type gain, unsigned norm_blocks, SumJob<T> b) {
+    if (blockIdx.x >= norm_blocks) {
+        const unsigned block = blockIdx.x - norm_blocks;
+        if (b.wide) sum_partials_block<T, 4>(b.part, b.out, b.outer, b.parts, b.inner, block);
+        else sum_partials_block<T, 1>(b.part, b.out, b.outer, b.parts, b.inner, block);
+        return;
+    }
+    if (part_a)
+        sum_norm_block<T, typename Acc<T>::type, KK>(part_a, parts, n_samples, plane, raw, d_raw,
+                                                     terms, gain_vec, groups, gain, blockIdx.x);
+    else
+        sum_norm_block<T, T, KK>(part_t, 1, n_samples, plane, raw, d_raw, terms, gain_vec, groups,
+                                 gain, blockIdx.x);
+}
+
+template <typename T>
+bool norm_tail_kernel_built(int kk) { return kk == 9 || kk == 25; }
+
 // The partial sums a filter-gradient launch leaves behind: dSF over `csplit`
 // channel splits and / or dCF over `nstrips` strips (null: nothing to add), in
-// one launch.
+// one launch.  With `norm` (and a launch to be made anyway, and a kernel built
+// for this tap count) the dSF part of that launch also applies the spatial
+// filter normalisation's Jacobian and writes norm->d_raw: dsf is then where the
+// filter kernel put a complete dSF (no partial sums), and is not written here.
 template <typename T>
 inline hipError_t sum_filter_partials(const typename Acc<T>::type *ws_sf, T *dsf, int64_t n,
                                       int csplit, int64_t sf_inner,
                                       const typename Acc<T>::type *ws_cf, T *dcf, int64_t nc,
-                                      int nstrips, int64_t kk, hipStream_t st) {
+                                      int nstrips, int64_t kk, hipStream_t st,
+                                      NormTail<T> *norm = nullptr) {
+    using A = typename Acc<T>::type;
+    if (norm && dsf && (ws_sf || ws_cf) && norm_tail_kernel_built<T>((int)kk)) {
+        const int64_t plane = sf_inner / kk;
+        const int64_t threads = n * plane;
+        const unsigned norm_blocks = (unsigned)((threads + 255) / 256);
+        SumJob<T> b{};
+        if (ws_cf) b = sum_job<T>(ws_cf, dcf, nc, nstrips, kk);
+        const dim3 grid(norm_blocks + b.blocks), block(256);
+        const A gain = (A)norm->gain;
+#define DDF_SUM_NORM(KK_)                                                                         \
+    hipLaunchKernelGGL((k_sum_norm_pair<T, KK_>), grid, block, 0, st, ws_sf, ws_sf ? nullptr : dsf, \
+                       ws_sf ? csplit : 1, n, plane, norm->raw, norm->d_raw, norm->terms,         \
+                       norm->gain_vec, norm->groups, gain, norm_blocks, b)
+        if (kk == 9) DDF_SUM_NORM(9);
+        else DDF_SUM_NORM(25);
+#undef DDF_SUM_NORM
+        norm->applied = true;
+        return hipGetLastError();
+    }
     if (ws_sf && ws_cf) {
         const SumJob<T> a = sum_job<T>(ws_sf, dsf, n, csplit, sf_inner);
         const SumJob<T> b = sum_job<T>(ws_cf, dcf, nc, nstrips, kk);

@@ -22,7 +22,8 @@ from torch.autograd import Function
 
 from . import _lib
 
-__all__ = ['DDFFunction', 'ddf', 'OP_DICT', 'DDFUpFunction', 'ddf_up']
+__all__ = ['DDFFunction', 'ddf', 'OP_DICT', 'DDFUpFunction', 'ddf_up', 'DDFSpatialNormFunction',
+           'ddf_spatial_norm']
 
 
 def _require_device_contiguous(named_tensors):
@@ -224,6 +225,90 @@ def ddf(*args, **kwargs):
         named.update(kwargs)
         args = tuple(named[name] for name in _DDF_ARGS)
     return DDFFunction.apply(*args)
+
+
+class DDFSpatialNormFunction(Function):
+    """``ddf(features, channel_filter, FilterNorm(raw_spatial_filter), ...)`` as
+    one autograd node: the spatial filter normalisation of ``DDFPack``
+    (``ddf/ddf.py:146-157``, constant or learned per-tap gain, no offset) in
+    front of the operator (``ddf/ddf.py:217-221``).
+
+    Forward: the normalisation launch, then the operator's.  Backward: one
+    library call in which the launch that adds up the filter gradients' partial
+    sums also applies the normalisation's Jacobian, so the gradient of the
+    normalised filter is never written to memory and the normalisation's
+    gradient costs no launch of its own.
+
+    ``raw_spatial_filter`` is ``(b * groups, k*k, h // s, w // s)`` as the
+    operator takes it (``groups`` = the layer's ``head``: sample ``n`` uses row
+    ``n % groups`` of ``gain_vec``)."""
+
+    @staticmethod
+    def forward(ctx, features, channel_filter, raw_spatial_filter, gain_vec, kernel_size, dilation,
+                stride, kernel_combine, groups, gain):
+        assert features.is_cuda and channel_filter.is_cuda and raw_spatial_filter.is_cuda
+        assert kernel_combine in {'mul', 'add'}, \
+            'only support mul or add combination, instead of {}'.format(kernel_combine)
+        dtype = torch.promote_types(torch.promote_types(features.dtype, channel_filter.dtype),
+                                    raw_spatial_filter.dtype)
+        assert dtype in _lib.DTYPE, 'unsupported dtype {}'.format(dtype)
+        features = features.to(dtype).contiguous()
+        channel_filter = channel_filter.to(dtype).contiguous()
+        raw = raw_spatial_filter.to(dtype).contiguous()
+        gain_vec = None if gain_vec is None else gain_vec.to(dtype).contiguous()
+        b, c, h, w = features.size()
+        k = kernel_size
+        assert tuple(channel_filter.size()) == (b, c, k, k), \
+            "channel_filter size {} does not match feature size {}".format(
+                channel_filter.size(), features.size())
+        assert tuple(raw.size()) == (b, k * k, h // stride, w // stride), \
+            "spatial_filter size {} does not match feature size {}".format(
+                raw.size(), features.size())
+        assert groups >= 1 and b % groups == 0
+        ho, wo = h // stride, w // stride
+        with _lib.on_device_of(features):
+            spatial_filter = _lib.filter_norm(raw, b // groups, groups, k * k, ho * wo, gain, gain_vec)
+            output = features.new_empty((b, c, ho, wo))
+            _lib.forward(features, channel_filter, spatial_filter, output, k, dilation, stride,
+                         kernel_combine, '')
+        ctx.conf = (k, dilation, stride, kernel_combine, groups, gain)
+        if any(ctx.needs_input_grad):
+            ctx.save_for_backward(features, channel_filter, spatial_filter, raw, gain_vec)
+        return output
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_output):
+        features, channel_filter, spatial_filter, raw, gain_vec = ctx.saved_tensors
+        k, d, s, combine, groups, gain = ctx.conf
+        grad_output = grad_output.to(features.dtype).contiguous()
+        want = ctx.needs_input_grad
+        want_gain = gain_vec is not None and want[3]
+        need = ((_lib.NEED_DX if want[0] else 0) | (_lib.NEED_DCF if want[1] else 0) |
+                (_lib.NEED_DSF if (want[2] or want_gain) else 0))
+        gx = torch.empty_like(features) if want[0] else None
+        gcf = torch.empty_like(channel_filter) if want[1] else None
+        graw = torch.empty_like(raw) if need & _lib.NEED_DSF else None
+        terms = torch.empty_like(raw) if want_gain else None
+        if need:
+            with _lib.on_device_of(features):
+                _lib.backward_spatial_norm(grad_output, features, channel_filter, spatial_filter,
+                                           raw, gx, gcf, graw, terms, k, d, s, combine, need,
+                                           groups, gain, gain_vec)
+        ggain = None
+        if want_gain:
+            b, kk, ho, wo = raw.shape
+            ggain = terms.view(b // groups, groups, kk, ho * wo).sum(dim=(0, 3)).reshape(-1)
+        return gx, gcf, (graw if want[2] else None), ggain, None, None, None, None, None, None
+
+
+def ddf_spatial_norm(features, channel_filter, raw_spatial_filter, kernel_size=3, dilation=1,
+                     stride=1, kernel_combine='mul', groups=1, gain=1.0, gain_vec=None):
+    """``ddf`` on the spatial filter ``gain * standardised(raw_spatial_filter)``
+    (standardised over the ``kernel_size**2`` taps of every pixel; ``gain_vec``,
+    ``(groups * kernel_size**2,)``, replaces the scalar gain)."""
+    return DDFSpatialNormFunction.apply(features, channel_filter, raw_spatial_filter, gain_vec,
+                                        kernel_size, dilation, stride, kernel_combine, groups, gain)
 
 
 class DDFUpFunction(Function):

@@ -172,6 +172,8 @@ class DDFPack(nn.Module):
         self.dilation = dilation
         self.head = head
         self.kernel_combine = kernel_combine
+        # (training: normalisation + operator as one autograd node; off = op by op)
+        self.fuse_spatial_norm = True
         self.spatial_branch = build_spatial_branch(
             in_channels, kernel_size, head, nonlinearity, stride)
         self.channel_branch = build_channel_branch(
@@ -274,6 +276,18 @@ class DDFPack(nn.Module):
                       sf.reshape(b * g, k * k, ho, wo), k, self.dilation, s, self.kernel_combine)
             return out.reshape(b, c, ho, wo)
         cf = self._channel_filter(x).reshape(b * g, c // g, k, k)
+        if self.fuse_spatial_norm and x.is_cuda and self._stock_spatial_branch() and \
+                not self.spatial_branch[1].runing_mean and h % s == 0 and w % s == 0:
+            # Training: the spatial filter normalisation and the operator as one autograd
+            # node, whose backward pushes dSF through the normalisation in the launch that
+            # adds up the filter gradients' partial sums (no launch of its own for the
+            # normalisation's gradient, no round trip of dSF through memory).
+            conv, norm = self.spatial_branch
+            raw = conv(x).reshape(b * g, k * k, ho, wo)
+            out = functional.ddf_spatial_norm(
+                x.reshape(b * g, c // g, h, w), cf, raw, k, self.dilation, s, self.kernel_combine,
+                g, 1.0 if norm.runing_std else norm.std, norm.std if norm.runing_std else None)
+            return out.reshape(b, c, ho, wo)
         sf = self.spatial_branch(x).reshape(b * g, k * k, ho, wo)
         out = ddf(x.reshape(b * g, c // g, h, w), cf, sf,
                   k, self.dilation, s, self.kernel_combine)

@@ -72,6 +72,8 @@ typedef enum {
 #define DDF_NEED_DCF 2u
 #define DDF_NEED_DSF 4u
 #define DDF_NEED_ALL 7u
+/* ddf_hip_describe only: name the launches of ddf_hip_backward_spatial_norm */
+#define DDF_DESCRIBE_SPATIAL_NORM 8u
 
 /* Library version: major*10000 + minor*100 + patch. */
 int ddf_hip_version(void);
@@ -86,7 +88,8 @@ const char *ddf_hip_last_error(void);
  * Names of the kernels a call with these arguments launches, as text in
  * `buffer` (diagnostics for benchmarks and profiles; no counterpart in the
  * reference).  need_mask 0 describes ddf_hip_forward, anything else
- * ddf_hip_backward with that mask.  Pointer alignment, which can send a call
+ * ddf_hip_backward with that mask (with DDF_DESCRIBE_SPATIAL_NORM added:
+ * ddf_hip_backward_spatial_norm).  Pointer alignment, which can send a call
  * to the scalar-access kernels, is assumed to be 16 bytes.
  */
 int ddf_hip_describe(int64_t N, int64_t C, int64_t H, int64_t W,
@@ -196,6 +199,39 @@ int ddf_hip_filter_norm_backward(const void *grad_y, const void *x,
                                  int64_t groups, int taps, int64_t inner,
                                  double gain, const void *gain_vec, int dtype,
                                  void *stream);
+
+/*
+ * ddf_hip_backward with the spatial branch's filter normalisation behind it:
+ * what autograd runs, in the reference, for `ddf(x, cf, FilterNorm(raw), ...)`
+ * (DDFPack.forward, ddf/ddf.py:217-221, with FilterNorm 'spatial',
+ * ddf/ddf.py:146-157) - the operator's backward (ddf/src/ddf_mul_ext.cpp:36-55)
+ * followed by the gradient of the normalisation's op chain.
+ * `spatial_filter` is the normalised filter the forward pass used,
+ * `raw_spatial_filter` the (N, k*k, Ho, Wo) tensor it was normalised from with
+ * ddf_hip_filter_norm(raw, sf, N / groups, groups, k*k, Ho*Wo, gain, gain_vec,
+ * ...): sample n belongs to group n % groups.  DDF_NEED_DSF asks for
+ * `grad_raw_spatial_filter` (the gradient with respect to the raw filter; the
+ * gradient of the normalised one is not written anywhere the caller sees) and,
+ * unless `gain_terms` is NULL, for the per-element terms of the gain_vec
+ * gradient as in ddf_hip_filter_norm_backward.  Where the backward pass ends
+ * with a launch that adds up dSF or dCF partial sums, that launch applies the
+ * normalisation's Jacobian: one launch fewer than the two calls, and dSF makes
+ * no round trip through memory.  Workspace:
+ * ddf_hip_backward_spatial_norm_workspace_bytes(...), 256-byte aligned.
+ */
+size_t ddf_hip_backward_spatial_norm_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W,
+                                                     int kernel_size, int dilation, int stride,
+                                                     int combine, int dtype, unsigned need_mask,
+                                                     int variant);
+int ddf_hip_backward_spatial_norm(const void *grad_output, const void *features,
+                                  const void *channel_filter, const void *spatial_filter,
+                                  const void *raw_spatial_filter, void *grad_features,
+                                  void *grad_channel_filter, void *grad_raw_spatial_filter,
+                                  void *gain_terms, void *workspace, size_t workspace_bytes,
+                                  int64_t N, int64_t C, int64_t H, int64_t W, int kernel_size,
+                                  int dilation, int stride, int combine, int dtype,
+                                  unsigned need_mask, int groups, double gain, const void *gain_vec,
+                                  int variant, void *stream);
 
 /*
  * Spatial filter branch of DDFPack in one launch (build_spatial_branch,

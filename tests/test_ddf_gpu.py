@@ -226,6 +226,20 @@ def test_full_size_configs(name, version):
     print(name, version, errs)
 
 
+# The seven distinct DDF call shapes of ddf_mul_resnet50 (channels, input size, stride):
+# three per stage of 56 / 28 / 14 / 7 pixels, the first of stages 2-4 with stride 2.
+RESNET50_LAYERS = [(64, 56, 1), (128, 56, 2), (128, 28, 1), (256, 28, 2), (256, 14, 1),
+                   (512, 14, 2), (512, 7, 1)]
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.float32])
+@pytest.mark.parametrize('C,size,s', RESNET50_LAYERS)
+def test_resnet50_layer_shapes(C, size, s, dtype):
+    """'mul', 3 x 3, batch 8, in the precision the network runs in (fp16) and in fp32."""
+    case = random_case(8, C, size, size, 3, s, dtype, seed=21, standardize=True)
+    check_against_oracle(*case, 3, 1, s, 'mul', what='resnet50 layer C=%d %dx%d s=%d' % (C, size, size, s))
+
+
 @pytest.mark.parametrize('name', sorted(FULL))
 def test_full_size_invariants(name):
     """Size-independent properties on the device results alone.  mul is

@@ -37,14 +37,23 @@ def cpu_reference(module, monkeypatch, *inputs):
     return ref, ins, out
 
 
+@pytest.mark.parametrize('fused', [True, False])
 @pytest.mark.parametrize('combine', ['mul', 'add'])
 @pytest.mark.parametrize('stride,head', [(1, 1), (2, 1), (1, 4)])
-def test_ddfpack_matches_cpu_reference(stride, head, combine, monkeypatch):
+def test_ddfpack_matches_cpu_reference(stride, head, combine, fused, monkeypatch):
+    """fused: the spatial filter normalisation and the operator as one autograd node
+    (its gradient rides on the operator's partial-sum launch); else op by op."""
     torch.manual_seed(0)
     pack = ddfnet_amd.DDFPack(16, kernel_size=3, stride=stride, head=head,
                               kernel_combine=combine).cuda()
+    pack.fuse_spatial_norm = fused
+    calls = []
+    real = ddf_modules.functional.ddf_spatial_norm
+    monkeypatch.setattr(ddf_modules.functional, 'ddf_spatial_norm',
+                        lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
     x = torch.randn(2, 16, 12, 12, device='cuda', requires_grad=True)
     out = pack(x)
+    assert calls == ([1] if fused else [])
     assert out.shape == (2, 16, 12 // stride, 12 // stride)
     go = torch.randn_like(out)
     out.backward(go)
