@@ -157,9 +157,10 @@ size_t rows_filters_workspace(const Problem &p, int dtype, unsigned need);
 // The row-register kernels cover the feature gradient and, in a launch of its
 // own, the filter gradients of this problem (pointer alignment assumed).
 bool rows_cover_backward(const Problem &p, int dtype);
-// Stride 2: the row-register kernels cover the filter gradients (the feature
-// gradient stays with the tile kernels).
+// Stride 2: the row-register kernels cover the filter gradients, and (even feature
+// heights) the feature gradient asked for alone.
 bool rows_cover_stride2_filters(const Problem &p, int dtype);
+inline bool rows_stride2_feature_gradient(const Problem &p) { return p.s == 2 && p.H % 2 == 0; }
 // x_mod != 0: the batch p.N is several groups of x_mod samples sharing one set
 // of features x (x_mod samples long); everything else is indexed by the sample.
 template <typename T>

@@ -77,8 +77,8 @@ int describe_backward(const Problem &p, int dtype, unsigned need, char *buf, int
         return n;
     }
     if (need & DDF_NEED_DX) {
-        if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 && p.s == 1 &&
-            rows_geometry(p, dtype, 0, &rg, &vx, &r))
+        if (dtype != DDF_F64 && tune_int("DDF_TUNE_ROWS", 1) != 0 &&
+            (p.s == 1 || rows_stride2_feature_gradient(p)) && rows_geometry(p, dtype, 0, &rg, &vx, &r))
             add("k_rows<dX,VX=%d,R=%d,%s>", vx, r, layout_name(rg));
         else if (small_supported(p)) add("%s", "k_small<dX>");
         else add("%s", "k_backward_features");

@@ -411,7 +411,12 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
     constexpr int NW = vec_words(kVB), NWX = vec_words(kXB);
     using Row = ExtRow<T, S * VX, HX, PAD>;
     static_assert(KK <= kWave, "one lane per channel-filter tap");
-    static_assert(S == 1 || (S == 2 && K == 3 && D == 1 && R == 1 && !BWD), "stride 2: forward, 3 x 3");
+    static_assert(S == 1 || (S == 2 && K == 3 && D == 1 && R == 1), "stride 2: 3 x 3, one row per lane");
+    // Stride-2 feature gradient: the lane of result row y loads dO rows y and y + 1 and
+    // writes the feature rows 2y and 2y + 1 of its columns (even feature heights).
+    constexpr bool S2B = S == 2 && BWD;
+    constexpr int LROWS = S2B ? 2 : ROWS;                 // rows a lane loads per channel
+    constexpr int kLB = S2B ? kVB : kXB, LNW = vec_words(kLB);
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
@@ -425,8 +430,12 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
     std::conditional_t<S == 1, Lane<R, HY, VX>, LaneStride2<VX>> ln;
     ln.init(g, wk.strip, lane);
 
-    const T *xs = x + (wk.n * g.C + wk.c_begin) * xplane;
-    T *os = out + (wk.n * g.C + wk.c_begin) * plane;
+    // (the tensor read has the result plane's shape in the stride-2 gradient, and the one
+    // written the feature plane's)
+    const int64_t in_plane = S2B ? plane : xplane, out_plane = S2B ? xplane : plane;
+    const uint32_t in_bytes = S2B ? plane_bytes : xplane_bytes, out_bytes = S2B ? xplane_bytes : plane_bytes;
+    const T *xs = x + (wk.n * g.C + wk.c_begin) * in_plane;
+    T *os = out + (wk.n * g.C + wk.c_begin) * out_plane;
     // byte offsets of the lane's vectors inside a plane; kOutside: reads as zero, is not written
     uint32_t xb[ROWS], ob[R];
 #pragma unroll
@@ -437,8 +446,18 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
         ob[r] = ln.ooff[r] < 0 ? kOutside : (uint32_t)ln.ooff[r] * (uint32_t)sizeof(T);
     const T *cfs = cf + (wk.n * g.C + wk.c_begin) * KK;
     constexpr bool kScalarTaps = sizeof(T) >= 4;
+    constexpr bool kFlip = BWD && S == 1;       // (the stride-2 gradient names its taps itself)
     const int tl = lane < KK ? lane : KK - 1;   // lane t holds tap t of a channel (flipped for the gradient)
-    const int tsel = BWD ? KK - 1 - tl : tl;
+    const int tsel = kFlip ? KK - 1 - tl : tl;
+    // where the lane's loads are
+    uint32_t lb[LROWS];
+    if constexpr (S2B) {
+        lb[0] = ob[0];
+        lb[1] = ln.onext < 0 ? kOutside : (uint32_t)ln.onext * (uint32_t)sizeof(T);
+    } else {
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) lb[rr] = xb[rr];
+    }
 
     // Spatial taps of the lane's pixels, in storage format.  Forward: tap t at
     // the pixel itself.  Gradient: slot (i, j) holds tap (K-1-i, K-1-j) at the
@@ -447,7 +466,32 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
     uint32_t sfw[R][KK][NW];
     {
         const T *sfn = sf + wk.n * KK * plane;
-        if constexpr (!BWD) {
+        if constexpr (S2B) {
+            // Result pixel (y, x) reaches feature pixel (2y + i - 1, 2x + j - 1) through tap
+            // (i, j).  Seen from the lane's 2 x 2 VX block of feature pixels (rows 2y and
+            // 2y + 1), tap row 0 belongs to the result row below and tap column 0 to the
+            // result pixel to the right: slot (i, j) holds that pixel's tap.
+            using SRow = ExtRow<T, VX, 1, PAD>;
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    const int t = i * K + j;
+                    const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
+                    SRow row;
+                    load_vec<kVB>(sr, lb[i == 0 ? 1 : 0], row.own);
+                    if (j == 0) {
+                        row.sides(ln.first, ln.last);
+                        A v[VX];
+#pragma unroll
+                        for (int e = 0; e < VX; ++e) v[e] = row.at(e + 1);
+                        pack<T, VX, A>(v, sfw[0][t]);
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < NW; ++k) sfw[0][t][k] = row.own[k];
+                    }
+                }
+        } else if constexpr (!BWD) {
 #pragma unroll
             for (int t = 0; t < KK; ++t) {
                 const __amdgpu_buffer_rsrc_t sr = plane_rsrc(sfn + t * plane, plane_bytes);
@@ -477,19 +521,19 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
 
     // feature rows and channel taps of channel ci, stage ST; a channel past the
     // wave's last one reads zeros (empty descriptor)
-    uint32_t xw[NST][ROWS][NWX];
+    uint32_t xw[NST][LROWS][LNW];
     T cfl[NST];
     A cfu[NST][kScalarTaps ? KK : 1];
     auto issue = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
-        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * xplane, ci < nch ? xplane_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t pr = plane_rsrc(xs + (int64_t)ci * in_plane, ci < nch ? in_bytes : 0u);
 #pragma unroll
-        for (int rr = 0; rr < ROWS; ++rr)
-            if (row_needed<R, K, D>(rr)) load_vec<kXB>(pr, xb[rr], xw[ST][rr]);
+        for (int rr = 0; rr < LROWS; ++rr)
+            if (S2B || row_needed<R, K, D>(rr)) load_vec<kLB>(pr, lb[rr], xw[ST][rr]);
         const int cc = ci < nch ? ci : nch - 1;   // (the taps are read through plain pointers: stay inside)
         if constexpr (kScalarTaps) {
 #pragma unroll
-            for (int t = 0; t < KK; ++t) cfu[ST][t] = cfs[(int64_t)cc * KK + (BWD ? KK - 1 - t : t)];
+            for (int t = 0; t < KK; ++t) cfu[ST][t] = cfs[(int64_t)cc * KK + (kFlip ? KK - 1 - t : t)];
         } else {
             cfl[ST] = cfs[(int64_t)cc * KK + tsel];
         }
@@ -521,14 +565,6 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
 #pragma unroll
                     for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfw[r][t][k]));
         }
-        Row row[ROWS];
-#pragma unroll
-        for (int rr = 0; rr < ROWS; ++rr) {
-            if (!row_needed<R, K, D>(rr)) continue;
-#pragma unroll
-            for (int k = 0; k < NWX; ++k) row[rr].own[k] = xw[ST][rr][k];
-            row[rr].sides(ln.first, ln.last);
-        }
         A w[KK];
         if constexpr (kScalarTaps) {
 #pragma unroll
@@ -537,6 +573,54 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
             const A cfa = (A)ld(&cfl[ST]);
 #pragma unroll
             for (int t = 0; t < KK; ++t) w[t] = lane_broadcast<A>(cfa, t);
+        }
+        if constexpr (S2B) {
+            // feature gradient of the lane's two feature rows: the four parity classes of a
+            // feature pixel see one, two, two and four taps
+            using GRow = ExtRow<T, VX, 1, PAD>;
+            GRow g0, g1;
+#pragma unroll
+            for (int k = 0; k < NW; ++k) { g0.own[k] = xw[ST][0][k]; g1.own[k] = xw[ST][1][k]; }
+            g0.sides(ln.first, ln.last);
+            g1.sides(ln.first, ln.last);
+            // dO * comb(CF[i][j], SF[i][j]) with the spatial tap of slot (i, j)
+            auto term = [&](A gv, int i, int j, int e, A acc) __attribute__((always_inline)) {
+                const int t = i * K + j;
+                const A sv = elem<T>(sfw[0][t], e);
+                if constexpr (MUL) return fma_(w[t], fma_(gv, sv, A(0)), acc);
+                else return fma_(gv, sv, fma_(gv, w[t], acc));
+            };
+            A top[2 * VX], bot[2 * VX];
+#pragma unroll
+            for (int e = 0; e < VX; ++e) {
+                const A g00 = g0.at(e), g01 = g0.at(e + 1), g10 = g1.at(e), g11 = g1.at(e + 1);
+                top[2 * e] = term(g00, 1, 1, e, A(0));
+                top[2 * e + 1] = term(g00, 1, 2, e, term(g01, 1, 0, e, A(0)));
+                bot[2 * e] = term(g00, 2, 1, e, term(g10, 0, 1, e, A(0)));
+                bot[2 * e + 1] = term(g00, 2, 2, e, term(g01, 2, 0, e, term(g10, 0, 2, e, term(g11, 0, 0, e, A(0)))));
+            }
+            const __amdgpu_buffer_rsrc_t dr = plane_rsrc(os + (int64_t)ci * out_plane, ci < nch ? out_bytes : 0u);
+            if constexpr (sizeof(T) == 2) {
+                // (round the complete fp32 sums, the same way in every unrolled copy: see below)
+#pragma unroll
+                for (int e = 0; e < 2 * VX; ++e) {
+                    asm volatile("" : "+v"(top[e]));
+                    asm volatile("" : "+v"(bot[e]));
+                }
+            }
+            uint32_t ow[NWX];
+            pack<T, 2 * VX, A>(top, ow);
+            store_vec_nt<kXB>(dr, xb[1], ow);
+            pack<T, 2 * VX, A>(bot, ow);
+            store_vec_nt<kXB>(dr, xb[2], ow);
+        } else {
+        Row row[ROWS];
+#pragma unroll
+        for (int rr = 0; rr < ROWS; ++rr) {
+            if (!row_needed<R, K, D>(rr)) continue;
+#pragma unroll
+            for (int k = 0; k < NWX; ++k) row[rr].own[k] = xw[ST][rr][k];
+            row[rr].sides(ln.first, ln.last);
         }
         A acc[R][VX];
 #pragma unroll
@@ -562,7 +646,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
                             acc[r][e] = fma_(xv, sv, acc[r][e]);
                         }
                     }
-        const __amdgpu_buffer_rsrc_t orr = plane_rsrc(os + (int64_t)ci * plane, ci < nch ? plane_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t orr = plane_rsrc(os + (int64_t)ci * out_plane, ci < nch ? out_bytes : 0u);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             if constexpr (sizeof(T) == 2) {
@@ -577,6 +661,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
             pack<T, VX, A>(acc[r], ow);
             store_vec_nt<kVB>(orr, ob[r], ow);
         }
+        }   // (not the stride-2 gradient)
     };
 
     // Channel ci is computed from stage ci % NST while the loads of channel

@@ -46,15 +46,15 @@ hipError_t launch_kdv(const Problem &p, const RowsGeom &g, bool backward, const 
     return hipGetLastError();
 }
 
-// Stride 2, forward.
-template <typename T, int VX>
+// Stride 2: forward, or (BWD: x is dO, out is dX, even feature heights) the feature gradient.
+template <typename T, int VX, bool BWD>
 hipError_t launch_stride2_v(const Problem &p, const RowsGeom &g, const T *x, const T *cf,
                             const T *sf, T *out, hipStream_t st) {
     const dim3 grid(g.xcd_per * kXcd), block(kWave * g.wpb);
     const bool pad = rows_shift_in_as_is(g);
     constexpr int kWpe = sizeof(T) == 2 && VX >= 8 ? 2 : 3;
 #define DDF_ROWS_CASE(MUL_, PAD_)                                                               \
-    hipLaunchKernelGGL((k_rows<T, 3, 1, MUL_, false, VX, 1, PAD_, kStages, kWpe, 2>), grid,     \
+    hipLaunchKernelGGL((k_rows<T, 3, 1, MUL_, BWD, VX, 1, PAD_, kStages, kWpe, 2>), grid,       \
                        block, 0, st, g, x, cf, sf, out)
     if (p.mul) {
         if (pad) DDF_ROWS_CASE(true, true);
@@ -100,17 +100,24 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
     const uintptr_t mask = (uintptr_t)(vx * sizeof(T)) - 1;
     if ((((uintptr_t)x | (uintptr_t)sf | (uintptr_t)out) & mask) != 0) return hipErrorNotSupported;
     if (p.s == 2) {
-        // (feature vectors are twice as long and come in pieces of at most 16 bytes)
-        if (backward || ((uintptr_t)x & (std::min<uintptr_t>(2 * vx * sizeof(T), 16) - 1)) != 0)
+        // (feature vectors are twice as long and come in pieces of at most 16 bytes; the
+        // feature gradient writes rows 2y and 2y + 1 per result row: even heights)
+        const T *feat = backward ? out : x;
+        if (((uintptr_t)feat & (std::min<uintptr_t>(2 * vx * sizeof(T), 16) - 1)) != 0)
             return hipErrorNotSupported;
+        if (backward && !rows_stride2_feature_gradient(p)) return hipErrorNotSupported;
+#define DDF_S2_CASE(VX_)                                                                       \
+    return backward ? rows::launch_stride2_v<T, VX_, true>(p, g, x, cf, sf, out, st)           \
+                    : rows::launch_stride2_v<T, VX_, false>(p, g, x, cf, sf, out, st)
+        // (feature vectors of 16 bytes at most: vx <= 4 for fp16, 2 for fp32)
         if constexpr (sizeof(T) == 2) {
-            if (vx == 8) return rows::launch_stride2_v<T, 8>(p, g, x, cf, sf, out, st);
+            if (vx == 4) DDF_S2_CASE(4);
         }
         if constexpr (sizeof(T) != 8) {
-            if (vx == 1) return rows::launch_stride2_v<T, 1>(p, g, x, cf, sf, out, st);
-            if (vx == 4) return rows::launch_stride2_v<T, 4>(p, g, x, cf, sf, out, st);
-            if (vx == 2) return rows::launch_stride2_v<T, 2>(p, g, x, cf, sf, out, st);
+            if (vx == 1) DDF_S2_CASE(1);
+            if (vx == 2) DDF_S2_CASE(2);
         }
+#undef DDF_S2_CASE
         return hipErrorNotSupported;
     }
     if constexpr (sizeof(T) == 2) {
@@ -282,13 +289,10 @@ hipError_t rows_filters_launch(const Problem &p, const T *go, const T *x, const 
                                                                ws_sf, ws_cf, need, st)            \
                 : rows::launch_filters_stride2_v<T, VX_, false>(p, g, go, x, cf, sf, dx, dcf, dsf, \
                                                                 ws_sf, ws_cf, need, st)
-            if (vx == 4) DDF_S2_CASE(4);
-            else if (vx == 2) DDF_S2_CASE(2);
+            if (vx == 2) DDF_S2_CASE(2);
             else if (vx == 1) DDF_S2_CASE(1);
             if constexpr (sizeof(T) == 2) {
-                if (vx == 8 && !fused)
-                    err = rows::launch_filters_stride2_v<T, 8, false>(p, g, go, x, cf, sf, dx, dcf, dsf,
-                                                                      ws_sf, ws_cf, need, st);
+                if (vx == 4) DDF_S2_CASE(4);
             }
 #undef DDF_S2_CASE
         } else if (taprow) {

@@ -330,6 +330,24 @@ def test_needs_input_grad_subsets():
 
 @pytest.mark.parametrize('dtype', [torch.float32, torch.float16], ids=_ids)
 @pytest.mark.parametrize('combine', ['mul', 'add'])
+@pytest.mark.parametrize('shape', [(2, 24, 56, 56), (3, 20, 28, 28), (2, 9, 14, 14), (2, 6, 10, 6),
+                                   (1, 5, 8, 64), (2, 7, 32, 16), (1, 3, 2, 2), (2, 4, 12, 128)])
+def test_stride2_feature_gradient_alone(shape, combine, dtype):
+    """dX asked for on its own with stride 2 (what autograd does when the filters are
+    frozen): even heights run on the row-register kernel, which writes feature rows 2y
+    and 2y + 1 from the lane of result row y."""
+    from ddfnet_amd import _lib
+    N, C, H, W = shape
+    x, cf, sf, go = random_case(N, C, H, W, 3, 2, dtype, seed=17)
+    assert 'k_rows<dX' in _lib.describe(shape, 3, 1, 2, combine, dtype, _lib.NEED_DX)
+    _, dx, dcf, dsf = run_ddf(x, cf, sf, go, 3, 1, 2, combine, need=(True, False, False))
+    assert dcf is None and dsf is None
+    want = oracle.backward(go, x, cf, sf, 3, 1, 2, combine)[0]
+    assert rel_err(dx, want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16], ids=_ids)
+@pytest.mark.parametrize('combine', ['mul', 'add'])
 @pytest.mark.parametrize('shape,d', [((3, 40, 14, 14), 1), ((2, 24, 14, 14), 2), ((2, 9, 12, 16), 1),
                                      ((1, 130, 8, 8), 1), ((2, 20, 28, 28), 1), ((2, 12, 56, 56), 1)])
 def test_one_launch_backward_equals_separate_requests(shape, d, combine, dtype):
