@@ -551,9 +551,44 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
 #pragma unroll
             for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfw[r][t][k]));
 
+    // fp16, 3 x 3 without dilation: the taps of columns 0 and 1 of a filter row go through
+    // the two-element dot product (fp32 accumulation), whose operands are pairs of
+    // neighbouring feature pixels and, per pixel, the pair of combined filters
+    // comb(CF, SF) - formed by one packed fp16 operation, i.e. rounded to fp16 like the
+    // operands.  12 vector instructions per pixel and channel instead of 18.  For that
+    // the spatial taps are regrouped once: sfp[r][i][e] = taps (i, 0) and (i, 1) of pixel
+    // e, sfs[r][i][k] = tap (i, 2) of pixels 2k and 2k + 1.
+    // (Stride 2, forward: result pixel e takes the feature pixels 2e - 1, 2e and 2e + 1.)
+    constexpr bool kDot2 = sizeof(T) == 2 && K == 3 && D == 1 && VX >= 2 && (S == 1 || !BWD);
+    uint32_t sfp[kDot2 ? R : 1][K][kDot2 ? VX : 1], sfs[kDot2 ? R : 1][K][NW];
+    if constexpr (kDot2) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int i = 0; i < K; ++i)
+#pragma unroll
+                for (int k = 0; k < NW; ++k) {
+                    const uint32_t a = sfw[r][i * K][k], b = sfw[r][i * K + 1][k];
+                    sfp[r][i][2 * k] = (a & 0xffffu) | (b << 16);
+                    sfp[r][i][2 * k + 1] = (a >> 16) | (b & 0xffff0000u);
+                    sfs[r][i][k] = sfw[r][i * K + 2][k];
+                }
+    }
+
     auto compute = [&](auto st_tag, int ci) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
-        if constexpr (sizeof(T) == 2) {
+        if constexpr (kDot2) {
+            // (keep the regrouped taps as they are: see below)
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int i = 0; i < K; ++i) {
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) asm volatile("" : "+v"(sfp[r][i][e]));
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfs[r][i][k]));
+                }
+        } else if constexpr (sizeof(T) == 2) {
             // Keeps the packed taps packed: without this the compiler widens all
             // of them to fp32 ahead of the channel loop, twice the registers.
             // Widened at their one use per channel they fold into the
@@ -566,9 +601,20 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
                     for (int k = 0; k < NW; ++k) asm volatile("" : "+v"(sfw[r][t][k]));
         }
         A w[KK];
+        uint32_t wp[kDot2 ? K : 1], ws[kDot2 ? K : 1];   // channel taps (i, 0) | (i, 1), and (i, 2) twice
         if constexpr (kScalarTaps) {
 #pragma unroll
             for (int t = 0; t < KK; ++t) w[t] = cfu[ST][t];
+        } else if constexpr (kDot2) {
+            const uint32_t bits = (uint32_t)__builtin_bit_cast(unsigned short, cfl[ST]);
+            uint32_t b[KK];
+#pragma unroll
+            for (int t = 0; t < KK; ++t) b[t] = (uint32_t)__builtin_amdgcn_readlane((int)bits, t);
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                wp[i] = b[i * K] | (b[i * K + 1] << 16);
+                ws[i] = b[i * K + 2] | (b[i * K + 2] << 16);
+            }
         } else {
             const A cfa = (A)ld(&cfl[ST]);
 #pragma unroll
@@ -627,6 +673,52 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
         for (int r = 0; r < R; ++r)
 #pragma unroll
             for (int e = 0; e < VX; ++e) acc[r][e] = 0;
+        if constexpr (kDot2) {
+            // pairs of neighbouring feature pixels (e - 1, e) of every window row: the odd e
+            // are the row's own words, the even e straddle two words
+            uint32_t xp[ROWS][VX];
+#pragma unroll
+            for (int rr = 0; rr < ROWS; ++rr) {
+                if constexpr (S == 1) {
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) {
+                        const uint32_t below = k == 0 ? row[rr].left[Row::SW - 1] : row[rr].own[k - 1];
+                        xp[rr][2 * k] = __builtin_amdgcn_alignbit(row[rr].own[k], below, 16);
+                        xp[rr][2 * k + 1] = row[rr].own[k];
+                    }
+                } else {
+                    // (2e - 1, 2e): the last element of word e - 1 and the first of word e
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) {
+                        const uint32_t below = e == 0 ? row[rr].left[Row::SW - 1] : row[rr].own[e - 1];
+                        xp[rr][e] = __builtin_amdgcn_alignbit(row[rr].own[e], below, 16);
+                    }
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < K; ++i) {
+                const half2_t wpair = __builtin_bit_cast(half2_t, wp[i]);
+                const half2_t wlast = __builtin_bit_cast(half2_t, ws[i]);
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+#pragma unroll
+                    for (int e = 0; e < VX; ++e) {
+                        const half2_t sp = __builtin_bit_cast(half2_t, sfp[r][i][e]);
+                        const half2_t cb = MUL ? wpair * sp : wpair + sp;
+                        acc[r][e] = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, xp[r + i][e]), cb,
+                                                           acc[r][e], false);
+                    }
+#pragma unroll
+                    for (int k = 0; k < NW; ++k) {
+                        const half2_t sl = __builtin_bit_cast(half2_t, sfs[r][i][k]);
+                        const half2_t cb = MUL ? wlast * sl : wlast + sl;
+#pragma unroll
+                        for (int h = 0; h < 2; ++h)
+                            acc[r][2 * k + h] = fma_(row[r + i].at(S * (2 * k + h) + 1), (A)cb[h], acc[r][2 * k + h]);
+                    }
+                }
+            }
+        } else {
         // mul: x * sf is exact in the accumulator type for fp16 storage and goes
         // into one mixed-precision multiply; add: two multiply-adds
 #pragma unroll
@@ -646,6 +738,7 @@ __global__ __launch_bounds__(kWave * kMaxWpb, WPE) void k_rows(RowsGeom g, const
                             acc[r][e] = fma_(xv, sv, acc[r][e]);
                         }
                     }
+        }   // (not the dot-product path)
         const __amdgpu_buffer_rsrc_t orr = plane_rsrc(os + (int64_t)ci * out_plane, ci < nch ? out_bytes : 0u);
 #pragma unroll
         for (int r = 0; r < R; ++r) {

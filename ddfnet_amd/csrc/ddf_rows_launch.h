@@ -126,6 +126,7 @@ hipError_t rows_launch(const Problem &p, bool backward, const T *x, const T *cf,
         if (vx == 2 && r == 1) return rows::launch_v<T, 2, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 1 && r == 1) return rows::launch_v<T, 1, 1>(p, g, backward, x, cf, sf, out, st);
         if (vx == 8 && r == 2) return rows::launch_v<T, 8, 2>(p, g, backward, x, cf, sf, out, st);
+        if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
         if (vx == 2 && r == 2) return rows::launch_v<T, 2, 2>(p, g, backward, x, cf, sf, out, st);
     } else if constexpr (sizeof(T) == 4) {
         if (vx == 4 && r == 2) return rows::launch_v<T, 4, 2>(p, g, backward, x, cf, sf, out, st);
