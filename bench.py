@@ -101,6 +101,18 @@ def algorithmic_bytes(N, C, H, W, k, s, esz):
     }
 
 
+def rotating_sets(N, C, H, W, k, s, esz, set_bytes):
+    """Buffer sets to rotate over: enough that even the library call that touches the
+    fewest bytes of a set (the forward pass) goes through twice the last-level cache
+    before it sees a set again.  Sized by the whole set instead, a call timed on its own
+    finds part of its operands still cached: the 5x5 forward pass then reads 30 us where
+    the same kernel takes 38 us inside a step (kernel trace of both)."""
+    least = min(algorithmic_bytes(N, C, H, W, k, s, esz).values())
+    nsets = max(2, LLC_BYTES * 2 // least + 1)
+    free, _ = torch.cuda.mem_get_info()
+    return int(min(nsets, max(2, (free // 2) // set_bytes)))
+
+
 class Workset(object):
     """One rotating set of device buffers for a workload."""
 
@@ -223,9 +235,7 @@ def run_workload(name, steps, warmup, lib, verbose=True, copy_probe=False):
     esz = torch.empty(0, dtype=dtype).element_size()
     host = make_inputs(N, C, H, W, k, s, dtype)
     first = Workset(host)
-    nsets = max(2, LLC_BYTES * 2 // first.nbytes() + 1)
-    free, _ = torch.cuda.mem_get_info()
-    nsets = int(min(nsets, max(2, (free // 2) // first.nbytes())))
+    nsets = rotating_sets(N, C, H, W, k, s, esz, first.nbytes())
     sets = [first] + [Workset(host) for _ in range(nsets - 1)]
     ws_bytes = lib.backward_workspace_bytes((N, C, H, W), k, d, s, combine, dtype, 7)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda') if ws_bytes else None
@@ -288,7 +298,8 @@ def profile_phase(name, phase, steps, warmup, lib):
     N, C, H, W, k, d, s, combine, dtype = WORKLOADS[name]
     host = make_inputs(N, C, H, W, k, s, dtype)
     first = Workset(host)
-    nsets = max(2, LLC_BYTES * 2 // first.nbytes() + 1)
+    esz = torch.empty(0, dtype=dtype).element_size()
+    nsets = rotating_sets(N, C, H, W, k, s, esz, first.nbytes())
     sets = [first] + [Workset(host) for _ in range(nsets - 1)]
     ws_bytes = lib.backward_workspace_bytes((N, C, H, W), k, d, s, combine, dtype, 7)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda') if ws_bytes else None
@@ -301,7 +312,6 @@ def profile_phase(name, phase, steps, warmup, lib):
     for _ in range(4):
         b.copy_(a)
     torch.cuda.synchronize()
-    esz = torch.empty(0, dtype=dtype).element_size()
     need_of = {'fwd': 0, 'bwd': 7, 'dx': 1, 'dfilters': 6}
     return {'workload': name, 'phase': phase, 'calls': warmup + steps, 'us_per_call': round(ms * 1e3, 2),
             'kernels': lib.describe((N, C, H, W), k, d, s, combine, dtype, need_of[phase]),
