@@ -20,11 +20,17 @@
 #include <algorithm>
 
 #include "ddf_common.h"
+#include "ddf_rows.h"
 
 namespace ddf {
 int tune_int(const char *name, int fallback);
 
 namespace {
+using rows::kOutside;
+using rows::load_vec;
+using rows::plane_rsrc;
+using rows::store_vec_nt;
+using rows::vec_words;
 
 constexpr int kChunk = 256;   // channels whose weights sit in LDS at a time (64 per wave)
 
@@ -272,6 +278,201 @@ __global__ __launch_bounds__(4 * kWave) void k_spatial_branch_tiles(
     }
 }
 
+// ---------------------------------------------------------------------------
+// Spatial branch, 3 x 3 taps, as a stream over the channels (the kernel the
+// launcher prefers).  A lane owns VP neighbouring result pixels of one sample
+// (stride 1: the plane is one run of pixels, so a vector may cross image rows;
+// stride 2: the 2 * VP feature pixels under VP result pixels of one row come in
+// as one vector) and adds up KK taps for each.  The WAVES waves of a workgroup
+// cover the same pixels and a range of channels each, U at a time; their sums
+// meet in LDS at the end.  Like the operator's own kernels it has
+//   * every channel plane behind a buffer descriptor (an idle lane's offset and
+//     the planes past the last channel read zero, no bounds branch),
+//   * the loads of NST - 1 channel groups in flight while one is computed,
+//   * the weights - the same for every lane - in scalar registers.
+struct SpatialGeom {
+    int C, W, Wo;
+    int plane;      // H * W
+    int npix;       // Ho * Wo
+    int nvec;       // npix / VP
+    int lpt;        // lanes of a workgroup's pixel tile that have a vector
+    int ngroups;    // C / U
+    int gpw;        // channel groups per wave
+    int steps;      // gpw rounded up to a multiple of NST
+};
+
+template <typename T, int KK, int VP, int S, int WAVES, int U, int NST>
+__global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
+    SpatialGeom g, const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias,
+    T *__restrict__ sf, float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
+    constexpr int XE = S == 1 ? VP : (VP == 1 ? 1 : 2 * VP);   // feature elements a lane loads per channel
+    constexpr int kXB = XE * sizeof(T), NWX = vec_words(kXB);
+    constexpr int kOB = VP * sizeof(T), NWO = vec_words(kOB);
+    constexpr int WPU = U * sizeof(T) / 4;                     // 32-bit words of U weights
+    static_assert(U * sizeof(T) % 4 == 0 && U % 2 == 0, "weights come in whole words, channels in pairs");
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int head = blockIdx.y, heads = gridDim.y;
+    const int64_t n = blockIdx.z;
+    const int v = blockIdx.x * g.lpt + lane;
+    const bool live = lane < g.lpt && v < g.nvec;
+    const int p = v * VP;                                      // first of the lane's result pixels
+    int in_off = p;
+    if constexpr (S == 2) {
+        const int yo = p / g.Wo, xo = p - yo * g.Wo;
+        in_off = 2 * yo * g.W + 2 * xo;
+    }
+    const uint32_t xb = live ? (uint32_t)in_off * (uint32_t)sizeof(T) : kOutside;
+    const uint32_t plane_bytes = (uint32_t)g.plane * (uint32_t)sizeof(T);
+    // the sample's C planes behind one descriptor; a channel is a scalar offset into it
+    const __amdgpu_buffer_rsrc_t xr = plane_rsrc(x + n * g.C * (int64_t)g.plane, (uint32_t)g.C * plane_bytes);
+    const char *wg = reinterpret_cast<const char *>(w + (int64_t)head * KK * g.C);
+    const uint32_t row_bytes = (uint32_t)g.C * (uint32_t)sizeof(T);
+    const int j0 = wave * g.gpw;                               // the wave's first channel group
+
+    uint32_t xw[NST][U][NWX];
+    short xh[NST][U];                                          // (single fp16 elements: as loaded)
+    uint32_t ww[NST][KK][WPU];
+    // channel group i of this wave's gpw consecutive ones, stage ST (consecutive: a wave's
+    // weights of consecutive steps then share scalar-cache lines)
+    auto issue = [&](auto st_tag, int i) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        const bool have = i < g.gpw && j0 + i < g.ngroups;
+        // (a group the wave does not have: every lane's offset lies outside, the loads
+        // return zero; its weights are those of the wave's first group)
+        const int j = have ? j0 + i : (j0 < g.ngroups ? j0 : 0);
+        const uint32_t vb = have ? xb : kOutside;
+        const uint32_t cb = (uint32_t)(j * U) * plane_bytes;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if constexpr (kXB == 2) {
+                xh[ST][u] = __builtin_amdgcn_raw_buffer_load_b16(xr, (int)vb, (int)(cb + (uint32_t)u * plane_bytes), 0);
+            } else if constexpr (kXB == 4) {
+                xw[ST][u][0] = __builtin_amdgcn_raw_buffer_load_b32(xr, (int)vb, (int)(cb + (uint32_t)u * plane_bytes), 0);
+            } else if constexpr (kXB == 8) {
+                const auto q = __builtin_amdgcn_raw_buffer_load_b64(xr, (int)vb, (int)(cb + (uint32_t)u * plane_bytes), 0);
+                xw[ST][u][0] = q[0]; xw[ST][u][1] = q[1];
+            } else {
+                static_assert(kXB <= 16, "vectors of 16 bytes at most");
+                const auto q = __builtin_amdgcn_raw_buffer_load_b128(xr, (int)vb, (int)(cb + (uint32_t)u * plane_bytes), 0);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) xw[ST][u][k] = q[k];
+            }
+        }
+        const uint32_t wb = (uint32_t)(j * U) * (uint32_t)sizeof(T);
+#pragma unroll
+        for (int t = 0; t < KK; ++t)
+#pragma unroll
+            for (int q = 0; q < WPU; ++q)
+                ww[ST][t][q] = *reinterpret_cast<const uint32_t *>(wg + (wb + (uint32_t)t * row_bytes + 4u * q));
+    };
+    float acc[KK][VP];
+#pragma unroll
+    for (int t = 0; t < KK; ++t)
+#pragma unroll
+        for (int k = 0; k < VP; ++k) acc[t][k] = 0.f;
+    auto compute = [&](auto st_tag) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        if constexpr (sizeof(T) == 2) {
+            // two channels at a time: (x[c], x[c+1]) of a pixel against (w[c], w[c+1]), which is
+            // one word of the weight row as it lies in memory; fp32 sums
+#pragma unroll
+            for (int pr = 0; pr < U / 2; ++pr)
+#pragma unroll
+                for (int k = 0; k < VP; ++k) {
+                    constexpr uint32_t kLow = 0x05040100u, kHigh = 0x07060302u;
+                    rows::half2_t xp;
+                    if constexpr (kXB == 2) {
+                        xp[0] = __builtin_bit_cast(_Float16, xh[ST][2 * pr]);
+                        xp[1] = __builtin_bit_cast(_Float16, xh[ST][2 * pr + 1]);
+                    } else {
+                        const int e = S * k;
+                        xp = __builtin_bit_cast(rows::half2_t,
+                                                __builtin_amdgcn_perm(xw[ST][2 * pr + 1][e / 2], xw[ST][2 * pr][e / 2],
+                                                                      (e & 1) ? kHigh : kLow));
+                    }
+#pragma unroll
+                    for (int t = 0; t < KK; ++t)
+                        acc[t][k] = __builtin_amdgcn_fdot2(xp, __builtin_bit_cast(rows::half2_t, ww[ST][t][pr]),
+                                                           acc[t][k], false);
+                }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float xv[VP];
+#pragma unroll
+                for (int k = 0; k < VP; ++k) xv[k] = rows::elem<T>(xw[ST][u], S * k);
+#pragma unroll
+                for (int t = 0; t < KK; ++t) {
+                    const float wv = rows::elem<T>(ww[ST][t], u);
+#pragma unroll
+                    for (int k = 0; k < VP; ++k) acc[t][k] = fmaf(wv, xv[k], acc[t][k]);
+                }
+            }
+        }
+    };
+    // (in this order: the waits inside the walk count the loads that were issued later)
+    issue(std::integral_constant<int, 0>{}, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (NST > 2) issue(std::integral_constant<int, 1>{}, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (NST > 3) issue(std::integral_constant<int, 2>{}, 2);
+    __builtin_amdgcn_sched_barrier(0);
+    auto step = [&](auto st_tag, int i) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        issue(std::integral_constant<int, (ST + NST - 1) % NST>{}, i + NST - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(st_tag);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int i = 0; i < g.steps; i += NST) {
+        step(std::integral_constant<int, 0>{}, i);
+        if constexpr (NST > 1) step(std::integral_constant<int, 1>{}, i + 1);
+        if constexpr (NST > 2) step(std::integral_constant<int, 2>{}, i + 2);
+        if constexpr (NST > 3) step(std::integral_constant<int, 3>{}, i + 3);
+    }
+
+    if constexpr (WAVES > 1) {
+        // the other waves' sums reach wave 0 through LDS, [wave][tap][lane][pixel]
+        __shared__ __align__(16) float red[WAVES - 1][KK][kWave][VP];
+        if (wave > 0) {
+#pragma unroll
+            for (int t = 0; t < KK; ++t)
+#pragma unroll
+                for (int k = 0; k < VP; ++k) red[wave - 1][t][lane][k] = acc[t][k];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        // (one wave's sums at a time: unrolled, all of them would be in registers at once)
+#pragma unroll 1
+        for (int q = 0; q < WAVES - 1; ++q)
+#pragma unroll
+            for (int t = 0; t < KK; ++t)
+#pragma unroll
+                for (int k = 0; k < VP; ++k) acc[t][k] += red[q][t][lane][k];
+    }
+    TapParams<T, KK> params;
+    params.load(head, gain, gain_vec, offset_vec, bias);
+#pragma unroll
+    for (int k = 0; k < VP; ++k) {
+        float r[KK];
+#pragma unroll
+        for (int t = 0; t < KK; ++t) r[t] = acc[t][k];
+        normalise<T, KK>(r, params);
+#pragma unroll
+        for (int t = 0; t < KK; ++t) acc[t][k] = r[t];
+    }
+    T *on = sf + ((n * heads + head) * KK) * (int64_t)g.npix;
+    const __amdgpu_buffer_rsrc_t orr = plane_rsrc(on, (uint32_t)KK * (uint32_t)g.npix * (uint32_t)sizeof(T));
+    const uint32_t ob = live ? (uint32_t)p * (uint32_t)sizeof(T) : kOutside;
+#pragma unroll
+    for (int t = 0; t < KK; ++t) {
+        uint32_t ow[NWO];
+        rows::pack<T, VP, float>(acc[t], ow);
+        store_vec_nt<kOB>(orr, ob + (uint32_t)t * (uint32_t)g.npix * (uint32_t)sizeof(T), ow);
+    }
+}
+
 // Butterfly steps through the VALU's lane-permute path.  (Shuffles through the
 // LDS crossbar cost a round trip each and made these kernels several times slower.)
 template <int CTRL>
@@ -396,6 +597,88 @@ __global__ __launch_bounds__(kChannelThreads) void k_channel_branch(
 
 bool branch_kernel_size_built(int k) { return k == 3 || k == 5; }
 
+// Launch of k_spatial_stream; hipErrorNotSupported where it does not cover the problem
+// (the caller then takes the kernels above).
+template <typename T>
+hipError_t spatial_stream(const T *x, const T *w, const T *bias, T *sf, int64_t N, int64_t C, int64_t H,
+                          int64_t W, int head, int stride, double gain, const T *gain_vec,
+                          const T *offset_vec, hipStream_t st) {
+    constexpr int KK = 9, NST = 3;
+    constexpr int U = sizeof(T) == 2 ? 4 : 2;
+    constexpr int esz = (int)sizeof(T);
+    const int64_t Ho = H / stride, Wo = W / stride, npix = Ho * Wo;
+    if (tune_int("DDF_TUNE_SPATIAL_STREAM", 1) == 0) return hipErrorNotSupported;
+    if (stride != 1 && stride != 2) return hipErrorNotSupported;
+    if (C % U != 0 || ((uintptr_t)w % 4) != 0) return hipErrorNotSupported;
+    if (C * H * W * esz >= (1ll << 31) || KK * npix * esz >= (1ll << 31)) return hipErrorNotSupported;
+    // pixels per lane: the widest vector the shapes and addresses allow ...
+    auto fits = [&](int vp) {
+        if (npix % vp != 0 || ((uintptr_t)sf % (vp * esz)) != 0) return false;
+        if (stride == 1) return ((uintptr_t)x % (vp * esz)) == 0 && (H * W) % vp == 0;
+        if (vp == 1) return true;
+        return Wo % vp == 0 && W % vp == 0 && (H * W) % (2 * vp) == 0 && ((uintptr_t)x % (2 * vp * esz)) == 0;
+    };
+    const int vp_max = (stride == 1 ? 16 : 8) / esz;
+    // ... that still leaves enough waves to fill the machine: the waves of a workgroup
+    // share its pixels and split the channels, at least two pipeline rounds each
+    const int64_t want = tune_int("DDF_TUNE_SPATIAL_WANT", 2048);
+    int vp = 1, waves = 1;
+    for (int cand = vp_max; cand >= 1; cand /= 2) {
+        if (!fits(cand)) continue;
+        const int64_t nvec = npix / cand;
+        const int64_t tiles = cdiv(nvec, kWave) * N * head;
+        int wv = 1;
+        // (nearly a wave per SIMD with whole channel walks: better than splitting them)
+        if (tiles < tune_int("DDF_TUNE_SPATIAL_WHOLE", 768))
+            while (wv < 16 && wv * 2 * cand <= 32 && tiles * wv < want && (C / U) / (wv * 2) >= 2 * NST)
+                wv *= 2;
+        vp = cand;
+        waves = wv;
+        if (tiles * wv >= want || wv == 1) break;
+    }
+    const int fvp = tune_int("DDF_TUNE_SPATIAL_VP", 0), fwv = tune_int("DDF_TUNE_SPATIAL_WAVES", 0);
+    if (fvp > 0 && fvp <= vp_max && fits(fvp)) vp = fvp;
+    if (fwv > 0) waves = fwv;
+    if (vp * waves > 32 || (waves & (waves - 1)) != 0 || waves > 16) return hipErrorNotSupported;   // (the variants built)
+    SpatialGeom g;
+    g.C = (int)C; g.W = (int)W; g.Wo = (int)Wo;
+    g.plane = (int)(H * W);
+    g.npix = (int)npix;
+    g.nvec = (int)(npix / vp);
+    const int tiles = (int)cdiv(g.nvec, kWave);
+    g.lpt = (int)cdiv(g.nvec, tiles);                   // (tiles of equal size)
+    g.ngroups = (int)(C / U);
+    g.gpw = (int)cdiv(g.ngroups, waves);
+    g.steps = (int)cdiv(g.gpw, NST) * NST;
+    if (N > 65535 || head > 65535) return hipErrorNotSupported;
+    const dim3 grid((unsigned)tiles, (unsigned)head, (unsigned)N);
+#define DDF_STREAM_LAUNCH(VP_, S_, WAVES_)                                                        \
+    hipLaunchKernelGGL((k_spatial_stream<T, KK, VP_, S_, WAVES_, U, NST>), grid, dim3(WAVES_ * kWave), \
+                       0, st, g, x, w, bias, sf, (float)gain, gain_vec, offset_vec)
+#define DDF_STREAM_WAVES(VP_, S_)                                                                 \
+    do {                                                                                          \
+        if (waves == 1) DDF_STREAM_LAUNCH(VP_, S_, 1);                                            \
+        else if (waves == 2) DDF_STREAM_LAUNCH(VP_, S_, 2);                                       \
+        else if (waves == 4) DDF_STREAM_LAUNCH(VP_, S_, 4);                                       \
+        else if (waves == 8 && VP_ <= 4) DDF_STREAM_LAUNCH((VP_ <= 4 ? VP_ : 1), S_, 8);          \
+        else if (waves == 16 && VP_ <= 2) DDF_STREAM_LAUNCH((VP_ <= 2 ? VP_ : 1), S_, 16);        \
+        else return hipErrorNotSupported;                                                         \
+    } while (0)
+    if (stride == 1) {
+        if (vp == 8) { if constexpr (esz == 2) DDF_STREAM_WAVES(8, 1); else return hipErrorNotSupported; }
+        else if (vp == 4) DDF_STREAM_WAVES(4, 1);
+        else if (vp == 2) DDF_STREAM_WAVES(2, 1);
+        else DDF_STREAM_WAVES(1, 1);
+    } else {
+        if (vp == 4) { if constexpr (esz == 2) DDF_STREAM_WAVES(4, 2); else return hipErrorNotSupported; }
+        else if (vp == 2) DDF_STREAM_WAVES(2, 2);
+        else DDF_STREAM_WAVES(1, 2);
+    }
+#undef DDF_STREAM_WAVES
+#undef DDF_STREAM_LAUNCH
+    return hipGetLastError();
+}
+
 template <typename T>
 hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t N, int64_t C,
                           int64_t H, int64_t W, int head, int k, int stride, double gain,
@@ -403,6 +686,11 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
     const int64_t Ho = H / stride, Wo = W / stride;
     if (N == 0 || C == 0 || Ho * Wo == 0 || head == 0) return hipSuccess;
     if (N > 65535 || head > 65535 || C > (1 << 24) || H * W >= (1ll << 31)) return hipErrorNotSupported;
+    if (k == 3) {
+        const hipError_t err = spatial_stream<T>(x, w, bias, sf, N, C, H, W, head, stride, gain, gain_vec,
+                                                 offset_vec, st);
+        if (err != hipErrorNotSupported) return err;
+    }
     const int waves = k == 3 ? 8 : 4;
     // channels staged in LDS at a time: all of them up to kChunk, a multiple of 8 per wave
     // (and so of the 16 the tile kernel keeps in flight)
