@@ -429,6 +429,63 @@ def model_inference(batch=128, steps=10, warmup=3):
             'ddf_layers': layers}
 
 
+def branch_table(lib, batch=128, iters=100):
+    """The two filter-branch launches of DDFPack at the sixteen DDF layers of
+    ddf_mul_resnet50 (ddf/ddf.py:176-192, inference, fp16), each timed on its
+    own between stream events with feature maps rotating beyond the last-level
+    cache; torch's global average pool over the same feature maps for scale.
+    GB/s: feature bytes the spatial branch must read (every second row under
+    stride 2) plus the taps it writes."""
+    dt = torch.float16
+    layers = ((64, 56, 1, 3), (128, 56, 2, 1), (128, 28, 1, 3), (256, 28, 2, 1), (256, 14, 1, 5),
+              (512, 14, 2, 1), (512, 7, 1, 2))
+
+    def timed(fns):
+        n = len(fns)
+        for i in range(n + 3):
+            fns[i % n]()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for i in range(iters):
+            fns[i % n]()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / iters * 1e3
+
+    rows, total = [], {'spatial_us': 0.0, 'channel_us': 0.0, 'pool_us': 0.0}
+    torch.manual_seed(0)
+    for c, hw, s, count in layers:
+        mid = int(c * 0.2)
+        nset = max(2, int(600e6 / (batch * c * hw * hw * 2)) + 1)
+        w1 = torch.randn(mid, c, device='cuda', dtype=dt) * 0.1
+        b1 = torch.randn(mid, device='cuda', dtype=dt)
+        w2 = torch.randn(c * 9, mid, device='cuda', dtype=dt) * 0.1
+        b2 = torch.randn(c * 9, device='cuda', dtype=dt)
+        gv = torch.ones(c * 9, device='cuda', dtype=dt)
+        ov = torch.zeros(c * 9, device='cuda', dtype=dt)
+        w = torch.randn(9, c, device='cuda', dtype=dt) * 0.1
+        b = torch.randn(9, device='cuda', dtype=dt)
+        xs = [torch.randn(batch, c, hw, hw, device='cuda', dtype=dt) for _ in range(nset)]
+        ps = [torch.randn(batch, c, device='cuda', dtype=dt) for _ in range(nset)]
+        ch = timed([(lambda q=q: lib.channel_branch(q, w1, b1, w2, b2, 3, 1.0, gv, ov)) for q in ps])
+        sp = timed([(lambda x=x: lib.spatial_branch(x, w, b, 1, 3, s, 1.0, None, None)) for x in xs])
+        pool = timed([(lambda x=x: x.mean((2, 3))) for x in xs])
+        nbytes = batch * c * hw * hw * 2 // s + batch * 9 * (hw // s) ** 2 * 2
+        rows.append({'shape': [batch, c, hw, hw], 'stride': s, 'layers': count,
+                     'spatial_us': round(sp, 1), 'spatial_gbps': round(nbytes / sp / 1e3, 1),
+                     'channel_us': round(ch, 1), 'torch_mean_us': round(pool, 1)})
+        total['spatial_us'] += count * sp
+        total['channel_us'] += count * ch
+        total['pool_us'] += count * pool
+        del xs
+    torch.cuda.empty_cache()
+    out = {'per_batch_of_%d' % batch: {k: round(v, 1) for k, v in total.items()}, 'layers': rows}
+    log('[branches] per batch of %d, 16 layers: spatial %.0f us, channel %.0f us (torch mean over the same maps %.0f us)' % (
+        batch, total['spatial_us'], total['channel_us'], total['pool_us']))
+    return out
+
+
 def test_time_table(iters=20, warmup=5):
     """The reference's own micro-benchmark (test_time.py:54-145): a 3x3
     convolution, a depthwise 3x3 convolution, a DDFPack layer and the bare ddf
@@ -693,6 +750,7 @@ def main():
             mi['model'], mi['batch'], mi['dtype'], mi['images_per_s'], mi['ms_per_batch'],
             mi['ddf_ms_per_batch']))
     if not args.only_headline:
+        line['model_inference']['filter_branches'] = branch_table(lib)
         line['ddfpack_train'] = pack_train_table()
         line['up_forward'] = up_forward_table(lib)
     elif args.up_pack:

@@ -90,7 +90,8 @@ def test_spatial_branch_unaligned_views(dtype, tol):
 
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.float16, 6e-3)])
 @pytest.mark.parametrize('n,c,k', [(3, 16, 3), (128, 64, 3), (5, 128, 3), (4, 256, 3), (3, 512, 3),
-                                   (2, 70, 5), (7, 300, 3), (2, 1024, 3)])
+                                   (2, 70, 5), (7, 300, 3), (2, 1024, 3), (3, 64, 5), (6, 96, 3),
+                                   (130, 512, 3), (9, 256, 5)])
 def test_channel_branch_matches_fp64(n, c, k, dtype, tol):
     torch.manual_seed(n + c)
     mid = int(c * 0.2)
