@@ -97,11 +97,24 @@ bool cut_channels_filters(RowsGeom &t, int64_t N, int C) {
     const int target = tune_int("DDF_TUNE_ROWSF_WAVES", 2048);
     const int64_t want_split = std::max<int64_t>(1, (target + base * rows::kFilterWaves - 1) /
                                                         (base * rows::kFilterWaves));
-    int cpb = (int)((C + want_split - 1) / want_split);
-    int cpw = (cpb + rows::kFilterWaves - 1) / rows::kFilterWaves;
-    // whole rounds of the kernel's channel pipeline and whole dCF flush groups
-    cpw = (cpw + rows::kFlushChannels - 1) / rows::kFlushChannels * rows::kFlushChannels;
-    cpw = std::max(cpw, tune_int("DDF_TUNE_ROWSF_MIN_CPW", 2 * rows::kFlushChannels));
+    // Channels per wave for `split` channel ranges: whole rounds of the kernel's channel
+    // pipeline and whole dCF flush groups.
+    auto cpw_of = [&](int64_t split) {
+        const int cpb = (int)((C + split - 1) / split);
+        int w = (cpb + rows::kFilterWaves - 1) / rows::kFilterWaves;
+        w = (w + rows::kFlushChannels - 1) / rows::kFlushChannels * rows::kFlushChannels;
+        return std::max(w, tune_int("DDF_TUNE_ROWSF_MIN_CPW", 2 * rows::kFlushChannels));
+    };
+    // One split fewer where that turns a ragged second round of waves into a single round
+    // of longer walks (rounds of `target` resident waves times channels per wave is what
+    // the launch takes): 32 x 128 x 56 x 56 at stride 2 runs 1 792 waves of 16 channels
+    // 5 % faster than 2 688 of 12.
+    auto cost_of = [&](int w) {
+        const int64_t waves = base * rows::kFilterWaves * ((C + (int64_t)w * rows::kFilterWaves - 1) / ((int64_t)w * rows::kFilterWaves));
+        return ((waves + target - 1) / target) * w;
+    };
+    int cpw = cpw_of(want_split);
+    if (want_split > 1 && cost_of(cpw_of(want_split - 1)) < cost_of(cpw)) cpw = cpw_of(want_split - 1);
     const int forced = tune_int("DDF_TUNE_ROWSF_CPW", 0);
     if (forced) cpw = std::min(forced, C);
     t.cpw = std::max(1, cpw);
