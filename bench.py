@@ -319,6 +319,50 @@ def profile_phase(name, phase, steps, warmup, lib):
             'copy_probe_bytes': 4 * a.numel() * 4}
 
 
+BRANCH_LAYERS = ((64, 56, 1, 3), (128, 56, 2, 1), (128, 28, 1, 3), (256, 28, 2, 1), (256, 14, 1, 5),
+                 (512, 14, 2, 1), (512, 7, 1, 2))   # (C, H = W, stride, layers of that shape in ddf_mul_resnet50)
+
+
+def profile_branch(index, which, steps, warmup, lib, batch=128):
+    """One filter-branch launch shape on its own, for runs under rocprofv3:
+    warmup + steps launches of the spatial (or channel) branch kernel at layer
+    shape BRANCH_LAYERS[index], fp16, feature maps rotating beyond the
+    last-level cache, then a plain 256 MiB device copy (the yardstick the fetch /
+    write counters are scaled by)."""
+    dt = torch.float16
+    c, hw, s, count = BRANCH_LAYERS[index]
+    mid = int(c * 0.2)
+    torch.manual_seed(0)
+    nset = max(2, int(600e6 / (batch * c * hw * hw * 2)) + 1)
+    if which == 'spatial':
+        w = torch.randn(9, c, device='cuda', dtype=dt) * 0.1
+        b = torch.randn(9, device='cuda', dtype=dt)
+        xs = [torch.randn(batch, c, hw, hw, device='cuda', dtype=dt) for _ in range(nset)]
+        run = lambda i: lib.spatial_branch(xs[i % nset], w, b, 1, 3, s, 1.0, None, None)
+        nbytes = batch * c * hw * hw * 2 // s + batch * 9 * (hw // s) ** 2 * 2
+    else:
+        w1 = torch.randn(mid, c, device='cuda', dtype=dt) * 0.1
+        b1 = torch.randn(mid, device='cuda', dtype=dt)
+        w2 = torch.randn(c * 9, mid, device='cuda', dtype=dt) * 0.1
+        b2 = torch.randn(c * 9, device='cuda', dtype=dt)
+        gv = torch.ones(c * 9, device='cuda', dtype=dt)
+        ov = torch.zeros(c * 9, device='cuda', dtype=dt)
+        ps = [torch.randn(batch, c, device='cuda', dtype=dt) for _ in range(nset)]
+        run = lambda i: lib.channel_branch(ps[i % nset], w1, b1, w2, b2, 3, 1.0, gv, ov)
+        nbytes = 2 * (batch * c + mid * c + c * 9 * mid + batch * c * 9)
+    for i in range(warmup):
+        run(i)
+    ms = timed(run, steps)
+    a = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device='cuda')
+    b_ = torch.empty_like(a)
+    for _ in range(4):
+        b_.copy_(a)
+    torch.cuda.synchronize()
+    return {'branch': which, 'shape': [batch, c, hw, hw], 'stride': s, 'layers': count,
+            'calls': warmup + steps, 'us_per_call': round(ms * 1e3, 2), 'algorithmic_bytes': nbytes,
+            'copy_probe_bytes': 4 * a.numel() * 4}
+
+
 def device_copy_ceiling(step_bytes):
     """What a plain device-to-device copy reaches on this box: the practical
     ceiling beside the 8 TB/s of the data sheet.  Once at 256 MiB, once moving as
@@ -437,8 +481,7 @@ def branch_table(lib, batch=128, iters=100):
     GB/s: feature bytes the spatial branch must read (every second row under
     stride 2) plus the taps it writes."""
     dt = torch.float16
-    layers = ((64, 56, 1, 3), (128, 56, 2, 1), (128, 28, 1, 3), (256, 28, 2, 1), (256, 14, 1, 5),
-              (512, 14, 2, 1), (512, 7, 1, 2))
+    layers = BRANCH_LAYERS
 
     def timed(fns):
         n = len(fns)
@@ -695,6 +738,10 @@ def main():
     ap.add_argument('--profile-model', action='store_true',
                     help='run only the ResNet-50 inference (warm-up, a half-second gap, then --steps '
                          'batches): the unit the model summary in profiles/ is collected on')
+    ap.add_argument('--profile-branch', default=None, metavar='KIND:INDEX',
+                    help='run only the spatial or channel branch launch of one ResNet-50 layer shape '
+                         '(spatial:0 .. spatial:6, channel:0 .. channel:6): the unit the branch summary in '
+                         'profiles/ is collected on')
     ap.add_argument('--copy-probe', action='store_true',
                     help='also run a plain 256 MiB device copy (calibrates hardware counters)')
     args = ap.parse_args()
@@ -709,6 +756,11 @@ def main():
 
     if args.profile_model:
         print(json.dumps(profile_model(batches=args.steps)))
+        return
+    if args.profile_branch:
+        kind, index = args.profile_branch.split(':')
+        assert kind in ('spatial', 'channel') and 0 <= int(index) < len(BRANCH_LAYERS)
+        print(json.dumps(profile_branch(int(index), kind, args.steps, args.warmup, lib)))
         return
     if args.profile_phase:
         print(json.dumps(profile_phase(args.workload, args.profile_phase, args.steps, args.warmup, lib)))
