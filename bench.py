@@ -477,7 +477,8 @@ def branch_table(lib, batch=128, iters=100):
     """The two filter-branch launches of DDFPack at the sixteen DDF layers of
     ddf_mul_resnet50 (ddf/ddf.py:176-192, inference, fp16), each timed on its
     own between stream events with feature maps rotating beyond the last-level
-    cache; torch's global average pool over the same feature maps for scale.
+    cache, and torch's global average pool over the same feature maps; then the
+    pair the module runs instead, with the pooling on the spatial branch's launch.
     GB/s: feature bytes the spatial branch must read (every second row under
     stride 2) plus the taps it writes."""
     dt = torch.float16
@@ -496,7 +497,8 @@ def branch_table(lib, batch=128, iters=100):
         torch.cuda.synchronize()
         return start.elapsed_time(stop) / iters * 1e3
 
-    rows, total = [], {'spatial_us': 0.0, 'channel_us': 0.0, 'pool_us': 0.0}
+    rows, total = [], {'spatial_us': 0.0, 'channel_us': 0.0, 'pool_us': 0.0, 'spatial_with_pool_us': 0.0,
+                       'channel_from_parts_us': 0.0}
     torch.manual_seed(0)
     for c, hw, s, count in layers:
         mid = int(c * 0.2)
@@ -514,18 +516,30 @@ def branch_table(lib, batch=128, iters=100):
         ch = timed([(lambda q=q: lib.channel_branch(q, w1, b1, w2, b2, 3, 1.0, gv, ov)) for q in ps])
         sp = timed([(lambda x=x: lib.spatial_branch(x, w, b, 1, 3, s, 1.0, None, None)) for x in xs])
         pool = timed([(lambda x=x: x.mean((2, 3))) for x in xs])
+        # the same with the pooling riding on the spatial branch's launch
+        sp_pool = timed([(lambda x=x: lib.spatial_branch_pool(x, w, b, 1, 3, s, 1.0, None, None)) for x in xs])
+        parts = [lib.spatial_branch_pool(x, w, b, 1, 3, s, 1.0, None, None)[1] for x in xs[:2]]
+        ch_parts = timed([(lambda q=q: lib.channel_branch_parts(q, 1.0 / (hw * hw), w1, b1, w2, b2, 3, 1.0, gv, ov))
+                          for q in parts])
         nbytes = batch * c * hw * hw * 2 // s + batch * 9 * (hw // s) ** 2 * 2
         rows.append({'shape': [batch, c, hw, hw], 'stride': s, 'layers': count,
                      'spatial_us': round(sp, 1), 'spatial_gbps': round(nbytes / sp / 1e3, 1),
-                     'channel_us': round(ch, 1), 'torch_mean_us': round(pool, 1)})
+                     'channel_us': round(ch, 1), 'torch_mean_us': round(pool, 1),
+                     'spatial_with_pool_us': round(sp_pool, 1), 'channel_from_parts_us': round(ch_parts, 1)})
         total['spatial_us'] += count * sp
         total['channel_us'] += count * ch
         total['pool_us'] += count * pool
-        del xs
+        total['spatial_with_pool_us'] += count * sp_pool
+        total['channel_from_parts_us'] += count * ch_parts
+        del xs, parts
     torch.cuda.empty_cache()
     out = {'per_batch_of_%d' % batch: {k: round(v, 1) for k, v in total.items()}, 'layers': rows}
-    log('[branches] per batch of %d, 16 layers: spatial %.0f us, channel %.0f us (torch mean over the same maps %.0f us)' % (
-        batch, total['spatial_us'], total['channel_us'], total['pool_us']))
+    log('[branches] per batch of %d, 16 layers: pool %.0f + channel %.0f + spatial %.0f = %.0f us; with the pooling '
+        'on the spatial launch: channel %.0f + spatial %.0f = %.0f us' % (
+            batch, total['pool_us'], total['channel_us'], total['spatial_us'],
+            total['pool_us'] + total['channel_us'] + total['spatial_us'],
+            total['channel_from_parts_us'], total['spatial_with_pool_us'],
+            total['channel_from_parts_us'] + total['spatial_with_pool_us']))
     return out
 
 

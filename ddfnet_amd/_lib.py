@@ -16,6 +16,7 @@ DTYPE = {torch.float16: 0, torch.float32: 1, torch.float64: 2}
 COMBINE = {'mul': 0, 'add': 1}
 VARIANT = {'': 0, 'o': 1, 'f': 2}
 NEED_DX, NEED_DCF, NEED_DSF = 1, 2, 4
+ERR_UNSUPPORTED = 2   # DDF_ERR_UNSUPPORTED
 
 # name -> (restype, argtypes); must list every symbol of include/ddf_hip.h
 _vp, _i64, _i, _u, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
@@ -40,6 +41,10 @@ SYMBOLS = {
                                [_vp] * 2 + [_i, _vp]),
     'ddf_hip_channel_branch': (_i, [_vp] * 6 + [_i64] * 3 + [_i, ctypes.c_double] + [_vp] * 2 +
                                [_i, _vp]),
+    'ddf_hip_spatial_branch_pool': (_i, [_vp] * 5 + [_i64, ctypes.POINTER(ctypes.c_int)] + [_i64] * 4 +
+                                    [_i] * 3 + [ctypes.c_double] + [_vp] * 2 + [_i, _vp]),
+    'ddf_hip_channel_branch_parts': (_i, [_vp, _i, ctypes.c_double] + [_vp] * 5 + [_i64] * 3 +
+                                     [_i, ctypes.c_double] + [_vp] * 2 + [_i, _vp]),
     'ddf_hip_up_forward': (_i, [_vp] * 4 + [_i64] * 4 + [_i] * 5 + [_vp]),
     'ddf_hip_up_backward_workspace_bytes': (_sz, [_i64] * 4 + [_i] * 5 + [_u]),
     'ddf_hip_up_backward': (_i, [_vp] * 8 + [_sz] + [_i64] * 4 + [_i] * 5 + [_u, _vp]),
@@ -217,6 +222,47 @@ def channel_branch(pooled, weight1, bias1, weight2, bias2, k, gain, gain_vec=Non
         rc = lib().ddf_hip_channel_branch(
             _ptr(pooled), _ptr(weight1), _ptr(bias1), _ptr(weight2), _ptr(bias2), _ptr(cf), N, C,
             mid, k, float(gain), _ptr(gain_vec), _ptr(offset_vec), DTYPE[pooled.dtype], _stream())
+    check(rc)
+    return cf
+
+
+def spatial_branch_pool(features, weight, bias, head, k, stride, gain, gain_vec=None, offset_vec=None):
+    """spatial_branch that also leaves partial sums of every feature plane (what the
+    global average pool in front of the channel branch needs); returns
+    (taps, parts) with parts an fp32 (N, tiles, C) tensor, or None where the
+    library has no kernel for it (then pool and call the plain entry points)."""
+    N, C, H, W = features.shape
+    ho, wo = H // stride, W // stride
+    if N * C * ho * wo * head == 0:
+        return None
+    sf = features.new_empty((N, head * k * k, ho, wo))
+    cap_tiles = (ho * wo + 63) // 64 * 4
+    parts = torch.empty((N * cap_tiles * C,), dtype=torch.float32, device=features.device)
+    nparts = ctypes.c_int(0)
+    with on_device_of(features):
+        rc = lib().ddf_hip_spatial_branch_pool(
+            _ptr(features), _ptr(weight), _ptr(bias), _ptr(sf), _ptr(parts), parts.numel(),
+            ctypes.byref(nparts), N, C, H, W, head, k, stride, float(gain), _ptr(gain_vec),
+            _ptr(offset_vec), DTYPE[features.dtype], _stream())
+    if rc == ERR_UNSUPPORTED:
+        return None
+    check(rc)
+    return sf, parts[:N * nparts.value * C].view(N, nparts.value, C)
+
+
+def channel_branch_parts(parts, scale, weight1, bias1, weight2, bias2, k, gain, gain_vec=None,
+                         offset_vec=None):
+    """channel_branch on pooled = scale * parts.sum(1), parts an fp32 (N, tiles, C)
+    tensor as spatial_branch_pool returns it; the filters come out in the
+    weights' dtype."""
+    N, nparts, C = parts.shape
+    mid = weight1.shape[0]
+    cf = weight1.new_empty((N, C, k, k))
+    with on_device_of(parts):
+        rc = lib().ddf_hip_channel_branch_parts(
+            _ptr(parts), nparts, float(scale), _ptr(weight1), _ptr(bias1), _ptr(weight2), _ptr(bias2),
+            _ptr(cf), N, C, mid, k, float(gain), _ptr(gain_vec), _ptr(offset_vec),
+            DTYPE[weight1.dtype], _stream())
     check(rc)
     return cf
 

@@ -542,10 +542,12 @@ int ddf_hip_filter_norm_backward(const void *grad_y, const void *x, void *grad_x
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_filter_norm_backward launch");
 }
 
-int ddf_hip_spatial_branch(const void *features, const void *weight, const void *bias,
-                           void *spatial_filter, int64_t N, int64_t C, int64_t H, int64_t W,
-                           int head, int kernel_size, int stride, double gain,
-                           const void *gain_vec, const void *offset_vec, int dtype, void *stream) {
+namespace {
+int spatial_branch_impl(const void *features, const void *weight, const void *bias,
+                        void *spatial_filter, float *pool_parts, int64_t pool_capacity, int *n_parts,
+                        int64_t N, int64_t C, int64_t H, int64_t W,
+                        int head, int kernel_size, int stride, double gain,
+                        const void *gain_vec, const void *offset_vec, int dtype, void *stream) {
     if (N < 0 || C < 0 || H < 0 || W < 0 || head < 0) return fail(DDF_ERR_BAD_ARG, "negative tensor size");
     if (stride < 1) return fail(DDF_ERR_BAD_ARG, "stride must be >= 1 (got %d)", stride);
     if (dtype != DDF_F16 && dtype != DDF_F32)
@@ -560,26 +562,54 @@ int ddf_hip_spatial_branch(const void *features, const void *weight, const void 
             ? ddf::spatial_branch<__half>((const __half *)features, (const __half *)weight,
                                           (const __half *)bias, (__half *)spatial_filter, N, C, H, W,
                                           head, kernel_size, stride, gain, (const __half *)gain_vec,
-                                          (const __half *)offset_vec, st)
+                                          (const __half *)offset_vec, st, pool_parts, pool_capacity, n_parts)
             : ddf::spatial_branch<float>((const float *)features, (const float *)weight,
                                          (const float *)bias, (float *)spatial_filter, N, C, H, W, head,
                                          kernel_size, stride, gain, (const float *)gain_vec,
-                                         (const float *)offset_vec, st);
+                                         (const float *)offset_vec, st, pool_parts, pool_capacity, n_parts);
     if (err == hipErrorNotSupported) return fail(DDF_ERR_UNSUPPORTED, "spatial branch: sizes not covered");
+    if (err == hipErrorInvalidValue && pool_parts)
+        return fail(DDF_ERR_WORKSPACE, "spatial branch: the buffer of partial sums is too small");
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_spatial_branch launch");
 }
+}  // namespace
 
-int ddf_hip_channel_branch(const void *pooled, const void *weight1, const void *bias1,
-                           const void *weight2, const void *bias2, void *channel_filter, int64_t N,
-                           int64_t C, int64_t mid, int kernel_size, double gain,
+int ddf_hip_spatial_branch(const void *features, const void *weight, const void *bias,
+                           void *spatial_filter, int64_t N, int64_t C, int64_t H, int64_t W,
+                           int head, int kernel_size, int stride, double gain,
                            const void *gain_vec, const void *offset_vec, int dtype, void *stream) {
+    return spatial_branch_impl(features, weight, bias, spatial_filter, nullptr, 0, nullptr, N, C, H, W, head,
+                               kernel_size, stride, gain, gain_vec, offset_vec, dtype, stream);
+}
+
+int ddf_hip_spatial_branch_pool(const void *features, const void *weight, const void *bias,
+                                void *spatial_filter, float *pool_parts, int64_t pool_capacity,
+                                int *n_parts, int64_t N, int64_t C, int64_t H, int64_t W, int head,
+                                int kernel_size, int stride, double gain, const void *gain_vec,
+                                const void *offset_vec, int dtype, void *stream) {
+    if (!pool_parts || !n_parts || pool_capacity < 0)
+        return fail(DDF_ERR_BAD_ARG, "ddf_hip_spatial_branch_pool: null buffer of partial sums");
+    *n_parts = 0;
+    if (N > 0 && C > 0 && head > 0 && stride >= 1 && (H / stride) * (W / stride) == 0)
+        return fail(DDF_ERR_UNSUPPORTED, "spatial branch: nothing to pool into");
+    return spatial_branch_impl(features, weight, bias, spatial_filter, pool_parts, pool_capacity, n_parts, N, C,
+                               H, W, head, kernel_size, stride, gain, gain_vec, offset_vec, dtype, stream);
+}
+
+namespace {
+int channel_branch_impl(const void *pooled, const float *parts, int n_parts, double scale,
+                        const void *weight1, const void *bias1,
+                        const void *weight2, const void *bias2, void *channel_filter, int64_t N,
+                        int64_t C, int64_t mid, int kernel_size, double gain,
+                        const void *gain_vec, const void *offset_vec, int dtype, void *stream) {
     if (N < 0 || C < 0 || mid < 0) return fail(DDF_ERR_BAD_ARG, "negative tensor size");
     if (dtype != DDF_F16 && dtype != DDF_F32)
         return fail(DDF_ERR_UNSUPPORTED, "the branch kernels cover fp16 and fp32 (dtype %d)", dtype);
     if (!ddf::branch_kernel_size_built(kernel_size))
         return fail(DDF_ERR_UNSUPPORTED, "the branch kernels cover kernel sizes 3 and 5 (got %d)", kernel_size);
     if (N * C == 0) return DDF_OK;
-    if (!pooled || !weight1 || !weight2 || !channel_filter) return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    if ((!pooled && !parts) || !weight1 || !weight2 || !channel_filter) return fail(DDF_ERR_BAD_ARG, "null tensor pointer");
+    if (parts && n_parts < 1) return fail(DDF_ERR_BAD_ARG, "n_parts must be >= 1 (got %d)", n_parts);
     hipStream_t st = (hipStream_t)stream;
     const hipError_t err =
         dtype == DDF_F16
@@ -587,14 +617,33 @@ int ddf_hip_channel_branch(const void *pooled, const void *weight1, const void *
                                           (const __half *)bias1, (const __half *)weight2,
                                           (const __half *)bias2, (__half *)channel_filter, N, C, mid,
                                           kernel_size, gain, (const __half *)gain_vec,
-                                          (const __half *)offset_vec, st)
+                                          (const __half *)offset_vec, st, parts, n_parts, scale)
             : ddf::channel_branch<float>((const float *)pooled, (const float *)weight1,
                                          (const float *)bias1, (const float *)weight2,
                                          (const float *)bias2, (float *)channel_filter, N, C, mid,
                                          kernel_size, gain, (const float *)gain_vec,
-                                         (const float *)offset_vec, st);
+                                         (const float *)offset_vec, st, parts, n_parts, scale);
     if (err == hipErrorNotSupported) return fail(DDF_ERR_UNSUPPORTED, "channel branch: sizes not covered");
     return err == hipSuccess ? DDF_OK : fail_hip(err, "ddf_hip_channel_branch launch");
+}
+}  // namespace
+
+int ddf_hip_channel_branch(const void *pooled, const void *weight1, const void *bias1,
+                           const void *weight2, const void *bias2, void *channel_filter, int64_t N,
+                           int64_t C, int64_t mid, int kernel_size, double gain,
+                           const void *gain_vec, const void *offset_vec, int dtype, void *stream) {
+    return channel_branch_impl(pooled, nullptr, 0, 1.0, weight1, bias1, weight2, bias2, channel_filter, N, C,
+                               mid, kernel_size, gain, gain_vec, offset_vec, dtype, stream);
+}
+
+int ddf_hip_channel_branch_parts(const float *pool_parts, int n_parts, double scale,
+                                 const void *weight1, const void *bias1, const void *weight2,
+                                 const void *bias2, void *channel_filter, int64_t N, int64_t C,
+                                 int64_t mid, int kernel_size, double gain, const void *gain_vec,
+                                 const void *offset_vec, int dtype, void *stream) {
+    if (!pool_parts) return fail(DDF_ERR_BAD_ARG, "ddf_hip_channel_branch_parts: null partial sums");
+    return channel_branch_impl(nullptr, pool_parts, n_parts, scale, weight1, bias1, weight2, bias2,
+                               channel_filter, N, C, mid, kernel_size, gain, gain_vec, offset_vec, dtype, stream);
 }
 
 int ddf_hip_up_forward(const void *features, const void *const *channel_filters,

@@ -301,11 +301,47 @@ struct SpatialGeom {
     int steps;      // gpw rounded up to a multiple of NST
 };
 
-template <typename T, int KK, int VP, int S, int WAVES, int U, int NST>
+// Sums of U (2 or 4) values per lane over each row of 16 lanes of a wave: every lane
+// ends up with its row's total of value number (lane % U).  The first steps halve the
+// number of values a lane carries instead of adding U full sums side by side: lane
+// pairs exchange the value the other keeps (quad permutes); then the quads of a row add
+// up by rotation.  (The four rows of a wave are left apart: bringing them together takes
+// lane-indexed reads through the LDS unit, whose counter the kernel's scalar weight
+// loads share - waiting for one drains the other's prefetch.)
+template <int CTRL>
+__device__ __forceinline__ float from_permuted(float x) {
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+template <int U>
+__device__ __forceinline__ float row_sums(const float (&v)[U], int lane) {
+    static_assert(U == 2 || U == 4, "two or four values per lane");
+    const bool b0 = lane & 1, b1 = lane & 2;
+    float k = (b0 ? v[1] : v[0]) + from_permuted<0xB1 /* quad_perm [1,0,3,2] */>(b0 ? v[0] : v[1]);
+    if constexpr (U == 4) {
+        const float k1 = (b0 ? v[3] : v[2]) + from_permuted<0xB1>(b0 ? v[2] : v[3]);
+        k = (b1 ? k1 : k) + from_permuted<0x4E /* quad_perm [2,3,0,1] */>(b1 ? k : k1);
+    } else {
+        k += from_permuted<0x4E>(k);
+    }
+    k += from_permuted<0x124 /* row_ror:4 */>(k);
+    k += from_permuted<0x128 /* row_ror:8 */>(k);
+    return k;
+}
+
+// POOL: the kernel also leaves, per sample, pixel tile and channel, the sum of the
+// feature map over the pixels of a quarter of the tile (the lanes of one row of 16) in
+// pool_part[((n * tiles + tile) * 4 + row) * C + c] (fp32) -
+// the global average pool in front of the channel branch, from the values this kernel
+// has in registers anyway.  Under stride 2 (even H and W) the lane also loads the
+// feature row below its own, and both columns where it otherwise takes one; those lines
+// come in with their neighbours in any case.
+template <typename T, int KK, int VP, int S, int WAVES, int U, int NST, bool POOL = false>
 __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
     SpatialGeom g, const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias,
-    T *__restrict__ sf, float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
-    constexpr int XE = S == 1 ? VP : (VP == 1 ? 1 : 2 * VP);   // feature elements a lane loads per channel
+    T *__restrict__ sf, float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec,
+    float *__restrict__ pool_part) {
+    // feature elements a lane loads per channel (pooling under stride 2: both columns)
+    constexpr int XE = S == 1 ? VP : (VP == 1 && !POOL ? 1 : 2 * VP);
     constexpr int kXB = XE * sizeof(T), NWX = vec_words(kXB);
     constexpr int kOB = VP * sizeof(T), NWO = vec_words(kOB);
     constexpr int WPU = U * sizeof(T) / 4;                     // 32-bit words of U weights
@@ -331,6 +367,7 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
     const int j0 = wave * g.gpw;                               // the wave's first channel group
 
     uint32_t xw[NST][U][NWX];
+    uint32_t xlow[POOL && S == 2 ? NST : 1][U][NWX];           // (pooling under stride 2: the row below)
     short xh[NST][U];                                          // (single fp16 elements: as loaded)
     uint32_t ww[NST][KK][WPU];
     // channel group i of this wave's gpw consecutive ones, stage ST (consecutive: a wave's
@@ -358,6 +395,12 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
 #pragma unroll
                 for (int k = 0; k < 4; ++k) xw[ST][u][k] = q[k];
             }
+            if constexpr (POOL && S == 2) {
+                if (head == 0)
+                    load_vec<kXB>(xr, vb == kOutside ? kOutside : vb + (uint32_t)g.W * (uint32_t)sizeof(T) +
+                                                                       cb + (uint32_t)u * plane_bytes,
+                                  xlow[ST][u]);
+            }
         }
         const uint32_t wb = (uint32_t)(j * U) * (uint32_t)sizeof(T);
 #pragma unroll
@@ -371,8 +414,43 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
     for (int t = 0; t < KK; ++t)
 #pragma unroll
         for (int k = 0; k < VP; ++k) acc[t][k] = 0.f;
-    auto compute = [&](auto st_tag) __attribute__((always_inline)) {
+    auto compute = [&](auto st_tag, int i) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
+        if constexpr (POOL) {
+            // (head 0 of a sample does it for all heads.  No branch around the arithmetic: it
+            // would cut the step into blocks, and the waits the compiler then places at their
+            // joins cost more than the sums of a group the wave does not have.)
+            const bool keep = head == 0 && i < g.gpw && j0 + i < g.ngroups;
+            {
+                // (one partial sum per row of 16 lanes: four per tile)
+                float *dst = pool_part + (((n * gridDim.x + blockIdx.x) * 4 + (lane >> 4)) * g.C + (int64_t)(j0 + i) * U);
+                float psum[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    float ps = 0.f;
+                    if constexpr (sizeof(T) == 2 && kXB == 2) {
+                        ps = (float)__builtin_bit_cast(_Float16, xh[ST][u]);
+                    } else if constexpr (sizeof(T) == 2) {
+                        const rows::half2_t ones = {(_Float16)1, (_Float16)1};
+#pragma unroll
+                        for (int k = 0; k < NWX; ++k) {
+                            ps = __builtin_amdgcn_fdot2(__builtin_bit_cast(rows::half2_t, xw[ST][u][k]), ones, ps, false);
+                            if constexpr (S == 2)
+                                ps = __builtin_amdgcn_fdot2(__builtin_bit_cast(rows::half2_t, xlow[ST][u][k]), ones, ps, false);
+                        }
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < NWX; ++k) {
+                            ps += __uint_as_float(xw[ST][u][k]);
+                            if constexpr (S == 2) ps += __uint_as_float(xlow[ST][u][k]);
+                        }
+                    }
+                    psum[u] = ps;
+                }
+                const float tot = row_sums<U>(psum, lane);
+                if (keep && (lane & 15) < U) dst[lane & 15] = tot;
+            }
+        }
         if constexpr (sizeof(T) == 2) {
             // two channels at a time: (x[c], x[c+1]) of a pixel against (w[c], w[c+1]), which is
             // one word of the weight row as it lies in memory; fp32 sums
@@ -422,7 +500,7 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
         constexpr int ST = decltype(st_tag)::value;
         issue(std::integral_constant<int, (ST + NST - 1) % NST>{}, i + NST - 1);
         __builtin_amdgcn_sched_barrier(0);
-        compute(st_tag);
+        compute(st_tag, i);
         __builtin_amdgcn_sched_barrier(0);
     };
     for (int i = 0; i < g.steps; i += NST) {
@@ -502,7 +580,8 @@ template <typename T, int KK, int BLOCK, int NS>
 __global__ __launch_bounds__(kChannelThreads) void k_channel_branch(
     const T *__restrict__ pooled, const T *__restrict__ w1, const T *__restrict__ b1,
     const T *__restrict__ w2, const T *__restrict__ b2, T *__restrict__ cf, int N, int C, int mid,
-    float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec) {
+    float gain, const T *__restrict__ gain_vec, const T *__restrict__ offset_vec,
+    const float *__restrict__ parts, int nparts, float scale) {
     extern __shared__ float branch_smem[];
     float *v = branch_smem;            // [NS][C]
     float *h = v + NS * C;             // [NS][mid]
@@ -511,9 +590,19 @@ __global__ __launch_bounds__(kChannelThreads) void k_channel_branch(
     const int64_t n0 = (int64_t)blockIdx.y * NS;
     const int ns = min(NS, N - (int)n0);   // samples of this workgroup (the others: copies of the last)
     const int cb = blockIdx.x * BLOCK;
+    // the pooled vectors: given, or scale * the sum of nparts partial sums per value
+    // (parts[(n * nparts + p) * C + c], what k_spatial_stream leaves)
     for (int i = threadIdx.x; i < NS * C; i += kChannelThreads) {
         const int s = i / C, c = i - s * C;
-        v[i] = ld(pooled + (n0 + min(s, ns - 1)) * C + c);
+        const int64_t n = n0 + min(s, ns - 1);
+        if (parts) {
+            float a = 0.f;
+#pragma unroll 4
+            for (int q = 0; q < nparts; ++q) a += parts[(n * nparts + q) * C + c];
+            v[i] = a * scale;
+        } else {
+            v[i] = ld(pooled + n * C + c);
+        }
     }
     __syncthreads();
     // Dot products with sixteen lanes along a weight row and four rows per wave at a
@@ -602,7 +691,8 @@ bool branch_kernel_size_built(int k) { return k == 3 || k == 5; }
 template <typename T>
 hipError_t spatial_stream(const T *x, const T *w, const T *bias, T *sf, int64_t N, int64_t C, int64_t H,
                           int64_t W, int head, int stride, double gain, const T *gain_vec,
-                          const T *offset_vec, hipStream_t st) {
+                          const T *offset_vec, hipStream_t st, float *pool_part = nullptr,
+                          int64_t pool_capacity = 0, int *pool_parts = nullptr) {
     constexpr int KK = 9, NST = 3;
     constexpr int U = sizeof(T) == 2 ? 4 : 2;
     constexpr int esz = (int)sizeof(T);
@@ -612,8 +702,11 @@ hipError_t spatial_stream(const T *x, const T *w, const T *bias, T *sf, int64_t 
     if (C % U != 0 || ((uintptr_t)w % 4) != 0) return hipErrorNotSupported;
     if (C * H * W * esz >= (1ll << 31) || KK * npix * esz >= (1ll << 31)) return hipErrorNotSupported;
     // pixels per lane: the widest vector the shapes and addresses allow ...
+    const bool pool = pool_part != nullptr;
+    if (pool && stride == 2 && (H % 2 != 0 || W % 2 != 0)) return hipErrorNotSupported;   // (pixels no lane covers)
     auto fits = [&](int vp) {
         if (npix % vp != 0 || ((uintptr_t)sf % (vp * esz)) != 0) return false;
+        if (pool && stride == 2 && vp == 1) return ((uintptr_t)x % (2 * esz)) == 0;   // (pairs of columns)
         if (stride == 1) return ((uintptr_t)x % (vp * esz)) == 0 && (H * W) % vp == 0;
         if (vp == 1) return true;
         return Wo % vp == 0 && W % vp == 0 && (H * W) % (2 * vp) == 0 && ((uintptr_t)x % (2 * vp * esz)) == 0;
@@ -622,7 +715,7 @@ hipError_t spatial_stream(const T *x, const T *w, const T *bias, T *sf, int64_t 
     // ... that still leaves enough waves to fill the machine: the waves of a workgroup
     // share its pixels and split the channels, at least two pipeline rounds each
     const int64_t want = tune_int("DDF_TUNE_SPATIAL_WANT", 2048);
-    int vp = 1, waves = 1;
+    int vp = 0, waves = 1;
     for (int cand = vp_max; cand >= 1; cand /= 2) {
         if (!fits(cand)) continue;
         const int64_t nvec = npix / cand;
@@ -639,6 +732,7 @@ hipError_t spatial_stream(const T *x, const T *w, const T *bias, T *sf, int64_t 
     const int fvp = tune_int("DDF_TUNE_SPATIAL_VP", 0), fwv = tune_int("DDF_TUNE_SPATIAL_WAVES", 0);
     if (fvp > 0 && fvp <= vp_max && fits(fvp)) vp = fvp;
     if (fwv > 0) waves = fwv;
+    if (vp == 0) return hipErrorNotSupported;
     if (vp * waves > 32 || (waves & (waves - 1)) != 0 || waves > 16) return hipErrorNotSupported;   // (the variants built)
     SpatialGeom g;
     g.C = (int)C; g.W = (int)W; g.Wo = (int)Wo;
@@ -651,10 +745,23 @@ hipError_t spatial_stream(const T *x, const T *w, const T *bias, T *sf, int64_t 
     g.gpw = (int)cdiv(g.ngroups, waves);
     g.steps = (int)cdiv(g.gpw, NST) * NST;
     if (N > 65535 || head > 65535) return hipErrorNotSupported;
+    if (pool) {
+        if (N * tiles * 4 * C > pool_capacity) return hipErrorInvalidValue;
+        *pool_parts = tiles * 4;
+    }
     const dim3 grid((unsigned)tiles, (unsigned)head, (unsigned)N);
 #define DDF_STREAM_LAUNCH(VP_, S_, WAVES_)                                                        \
-    hipLaunchKernelGGL((k_spatial_stream<T, KK, VP_, S_, WAVES_, U, NST>), grid, dim3(WAVES_ * kWave), \
-                       0, st, g, x, w, bias, sf, (float)gain, gain_vec, offset_vec)
+    do {                                                                                          \
+        if (pool) {                                                                               \
+            hipLaunchKernelGGL((k_spatial_stream<T, KK, VP_, S_, WAVES_, U, NST, true>), grid,    \
+                               dim3(WAVES_ * kWave), 0, st, g, x, w, bias, sf, (float)gain,       \
+                               gain_vec, offset_vec, pool_part);                                  \
+            break;                                                                                \
+        }                                                                                         \
+        hipLaunchKernelGGL((k_spatial_stream<T, KK, VP_, S_, WAVES_, U, NST, false>), grid,       \
+                           dim3(WAVES_ * kWave), 0, st, g, x, w, bias, sf, (float)gain, gain_vec, \
+                           offset_vec, (float *)nullptr);                                         \
+    } while (0)
 #define DDF_STREAM_WAVES(VP_, S_)                                                                 \
     do {                                                                                          \
         if (waves == 1) DDF_STREAM_LAUNCH(VP_, S_, 1);                                            \
@@ -682,15 +789,17 @@ hipError_t spatial_stream(const T *x, const T *w, const T *bias, T *sf, int64_t 
 template <typename T>
 hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t N, int64_t C,
                           int64_t H, int64_t W, int head, int k, int stride, double gain,
-                          const T *gain_vec, const T *offset_vec, hipStream_t st) {
+                          const T *gain_vec, const T *offset_vec, hipStream_t st, float *pool_part,
+                          int64_t pool_capacity, int *pool_parts) {
     const int64_t Ho = H / stride, Wo = W / stride;
     if (N == 0 || C == 0 || Ho * Wo == 0 || head == 0) return hipSuccess;
     if (N > 65535 || head > 65535 || C > (1 << 24) || H * W >= (1ll << 31)) return hipErrorNotSupported;
     if (k == 3) {
         const hipError_t err = spatial_stream<T>(x, w, bias, sf, N, C, H, W, head, stride, gain, gain_vec,
-                                                 offset_vec, st);
+                                                 offset_vec, st, pool_part, pool_capacity, pool_parts);
         if (err != hipErrorNotSupported) return err;
     }
+    if (pool_part) return hipErrorNotSupported;   // (only the streaming kernel pools)
     const int waves = k == 3 ? 8 : 4;
     // channels staged in LDS at a time: all of them up to kChunk, a multiple of 8 per wave
     // (and so of the 16 the tile kernel keeps in flight)
@@ -756,7 +865,8 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
 template <typename T>
 hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2, const T *b2,
                           T *cf, int64_t N, int64_t C, int64_t mid, int k, double gain,
-                          const T *gain_vec, const T *offset_vec, hipStream_t st) {
+                          const T *gain_vec, const T *offset_vec, hipStream_t st, const float *parts,
+                          int nparts, double scale) {
     if (N == 0 || C == 0) return hipSuccess;
     const int kk = k * k;
     // (wide layers: fewer, larger blocks, as every block of a sample recomputes the hidden vector)
@@ -773,7 +883,7 @@ hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2
 #define DDF_CHANNEL_LAUNCH(KK_, BLOCK_, NS_)                                                     \
     hipLaunchKernelGGL((k_channel_branch<T, KK_, BLOCK_, NS_>), grid, dim3(kChannelThreads), lds, \
                        st, pooled, w1, b1, w2, b2, cf, (int)N, (int)C, (int)mid, (float)gain,    \
-                       gain_vec, offset_vec)
+                       gain_vec, offset_vec, parts, nparts, (float)scale)
 #define DDF_CHANNEL_CASE(KK_, BLOCK_)                                                            \
     do {                                                                                         \
         if (ns == 4) DDF_CHANNEL_LAUNCH(KK_, BLOCK_, 4);                                         \
@@ -793,10 +903,10 @@ hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2
 #define DDF_INSTANTIATE_BRANCHES(T)                                                              \
     template hipError_t spatial_branch<T>(const T *, const T *, const T *, T *, int64_t, int64_t, \
                                           int64_t, int64_t, int, int, int, double, const T *,    \
-                                          const T *, hipStream_t);                               \
+                                          const T *, hipStream_t, float *, int64_t, int *);      \
     template hipError_t channel_branch<T>(const T *, const T *, const T *, const T *, const T *, \
                                           T *, int64_t, int64_t, int64_t, int, double, const T *, \
-                                          const T *, hipStream_t);
+                                          const T *, hipStream_t, const float *, int, double);
 DDF_INSTANTIATE_BRANCHES(__half)
 DDF_INSTANTIATE_BRANCHES(float)
 #undef DDF_INSTANTIATE_BRANCHES

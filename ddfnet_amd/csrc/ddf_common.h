@@ -94,13 +94,21 @@ hipError_t filter_norm_backward(const T *dy, const T *x, T *dx, T *terms, int64_
 // hipErrorNotSupported: kernel size or sizes not covered, nothing launched.
 bool branch_kernel_size_built(int k);
 template <typename T>
+// pool_part (may be null): the launch also leaves the sums of the feature map over
+// the pixels of each of *pool_parts parts of a plane, fp32, [(n * parts + p) * C + c]; at most
+// pool_capacity floats.  hipErrorNotSupported where no kernel does that.
 hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t N, int64_t C,
                           int64_t H, int64_t W, int head, int k, int stride, double gain,
-                          const T *gain_vec, const T *offset_vec, hipStream_t st);
+                          const T *gain_vec, const T *offset_vec, hipStream_t st,
+                          float *pool_part = nullptr, int64_t pool_capacity = 0,
+                          int *pool_parts = nullptr);
+// parts (may be null): the pooled vectors are scale * the sums of nparts such partial
+// sums instead of `pooled`.
 template <typename T>
 hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2, const T *b2,
                           T *cf, int64_t N, int64_t C, int64_t mid, int k, double gain,
-                          const T *gain_vec, const T *offset_vec, hipStream_t st);
+                          const T *gain_vec, const T *offset_vec, hipStream_t st,
+                          const float *parts = nullptr, int nparts = 0, double scale = 1.0);
 
 // All scale*scale sub-pixel branches of an up-sampling DDF in one launch,
 // written into the pixel-shuffled (N, C, H*scale, W*scale) result; cf / sf are

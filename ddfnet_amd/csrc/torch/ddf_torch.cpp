@@ -357,7 +357,7 @@ at::Tensor ddf_pack_forward(const at::Tensor &features, const at::Tensor &conv_w
                             double channel_gain, const c10::optional<at::Tensor> &channel_gain_vec,
                             const c10::optional<at::Tensor> &channel_offset_vec,
                             int64_t kernel_size, int64_t dilation, int64_t stride, int64_t head,
-                            const std::string &kernel_combine) {
+                            const std::string &kernel_combine, bool fuse_pool) {
     TORCH_CHECK(features.is_cuda() && features.dim() == 4, "features must be a 4-d device tensor");
     const int dt = dtype_code(features.scalar_type());
     TORCH_CHECK(dt == DDF_F16 || dt == DDF_F32, "ddf_pack_forward covers fp16 and fp32");
@@ -378,17 +378,41 @@ at::Tensor ddf_pack_forward(const at::Tensor &features, const at::Tensor &conv_w
 
     c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(x.device());
     hipStream_t st = current_stream(x);
-    const at::Tensor pooled = at::mean(x, {2, 3});
     at::Tensor cf = at::empty({b, c, kernel_size, kernel_size}, x.options());
-    check_status(ddf_hip_channel_branch(
-        pooled.data_ptr(), fc1_weight.data_ptr(), ptr_or_null(fc1_bias), fc2_weight.data_ptr(),
-        ptr_or_null(fc2_bias), cf.data_ptr(), b, c, mid, (int)kernel_size, channel_gain,
-        ptr_or_null(channel_gain_vec), ptr_or_null(channel_offset_vec), dt, st));
     at::Tensor sf = at::empty({b, head * kk, ho, wo}, x.options());
-    check_status(ddf_hip_spatial_branch(
-        x.data_ptr(), conv_weight.data_ptr(), ptr_or_null(conv_bias), sf.data_ptr(), b, c, h, w,
-        (int)head, (int)kernel_size, (int)stride, spatial_gain, ptr_or_null(spatial_gain_vec),
-        ptr_or_null(spatial_offset_vec), dt, st));
+    // The spatial branch reads every feature plane anyway: where its kernel can, it leaves
+    // the planes' partial sums and the channel branch pools from those (one launch and
+    // one read of the feature map fewer); else pool first.
+    bool pooled_on_the_way = false;
+    if (fuse_pool && b * c * ho * wo > 0) {
+        const int64_t cap = b * c * ((ho * wo + 63) / 64) * 4;
+        at::Tensor parts = at::empty({cap}, x.options().dtype(at::kFloat));
+        int n_parts = 0;
+        const int rc = ddf_hip_spatial_branch_pool(
+            x.data_ptr(), conv_weight.data_ptr(), ptr_or_null(conv_bias), sf.data_ptr(),
+            parts.data_ptr<float>(), cap, &n_parts, b, c, h, w, (int)head, (int)kernel_size, (int)stride,
+            spatial_gain, ptr_or_null(spatial_gain_vec), ptr_or_null(spatial_offset_vec), dt, st);
+        if (rc != DDF_ERR_UNSUPPORTED) {
+            check_status(rc);
+            check_status(ddf_hip_channel_branch_parts(
+                parts.data_ptr<float>(), n_parts, 1.0 / (double)(h * w), fc1_weight.data_ptr(),
+                ptr_or_null(fc1_bias), fc2_weight.data_ptr(), ptr_or_null(fc2_bias), cf.data_ptr(), b, c, mid,
+                (int)kernel_size, channel_gain, ptr_or_null(channel_gain_vec),
+                ptr_or_null(channel_offset_vec), dt, st));
+            pooled_on_the_way = true;
+        }
+    }
+    if (!pooled_on_the_way) {
+        const at::Tensor pooled = at::mean(x, {2, 3});
+        check_status(ddf_hip_channel_branch(
+            pooled.data_ptr(), fc1_weight.data_ptr(), ptr_or_null(fc1_bias), fc2_weight.data_ptr(),
+            ptr_or_null(fc2_bias), cf.data_ptr(), b, c, mid, (int)kernel_size, channel_gain,
+            ptr_or_null(channel_gain_vec), ptr_or_null(channel_offset_vec), dt, st));
+        check_status(ddf_hip_spatial_branch(
+            x.data_ptr(), conv_weight.data_ptr(), ptr_or_null(conv_bias), sf.data_ptr(), b, c, h, w,
+            (int)head, (int)kernel_size, (int)stride, spatial_gain, ptr_or_null(spatial_gain_vec),
+            ptr_or_null(spatial_offset_vec), dt, st));
+    }
     at::Tensor out = at::empty({b, c, ho, wo}, x.options());
     // heads are folded into the batch: (b * head, c / head, h, w)
     check_status(ddf_hip_forward(x.data_ptr(), cf.data_ptr(), sf.data_ptr(), out.data_ptr(), b * head,
@@ -408,6 +432,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
           py::arg("spatial_filters"), py::arg("kernel_size") = 3, py::arg("dilation") = 1,
           py::arg("scale_factor") = 2, py::arg("kernel_combine") = "mul");
     m.def("ddf_pack_forward", &ddf_pack_forward,
-          "DDFPack.forward without gradients: pool, channel branch, spatial branch, operator");
+          "DDFPack.forward without gradients: spatial branch (pooling on the way where it can), "
+          "channel branch, operator");
     m.def("library_version", []() { return ddf_hip_version(); });
 }

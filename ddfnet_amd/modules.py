@@ -174,6 +174,8 @@ class DDFPack(nn.Module):
         self.kernel_combine = kernel_combine
         # (training: normalisation + operator as one autograd node; off = op by op)
         self.fuse_spatial_norm = True
+        # inference: the global average pool rides on the spatial branch's launch
+        self.fuse_pool = True
         self.spatial_branch = build_spatial_branch(
             in_channels, kernel_size, head, nonlinearity, stride)
         self.channel_branch = build_channel_branch(
@@ -243,24 +245,30 @@ class DDFPack(nn.Module):
             return None
         ext = functional.extension()
         if ext is not None:
-            # the same four launches without the interpreter in between
+            # the same launches without the interpreter in between
             return ext.ddf_pack_forward(
                 x, conv.weight, conv.bias,
                 1.0 if sp_norm.runing_std else sp_norm.std, tensors[6], tensors[7],
                 fc1.weight, fc1.bias, fc2.weight, fc2.bias,
                 1.0 if ch_norm.runing_std else ch_norm.std, tensors[8], tensors[9],
-                k, self.dilation, self.stride, self.head, self.kernel_combine)
+                k, self.dilation, self.stride, self.head, self.kernel_combine, self.fuse_pool)
         x = x.contiguous()
-        cf = _lib.channel_branch(
-            x.mean((2, 3)), fc1.weight, fc1.bias, fc2.weight, fc2.bias, k,
-            1.0 if ch_norm.runing_std else ch_norm.std,
-            ch_norm.std if ch_norm.runing_std else None,
-            ch_norm.mean if ch_norm.runing_mean else None)
-        sf = _lib.spatial_branch(
-            x, conv.weight, conv.bias, self.head, k, self.stride,
-            1.0 if sp_norm.runing_std else sp_norm.std,
-            sp_norm.std if sp_norm.runing_std else None,
-            sp_norm.mean if sp_norm.runing_mean else None)
+        ch_args = (fc1.weight, fc1.bias, fc2.weight, fc2.bias, k,
+                   1.0 if ch_norm.runing_std else ch_norm.std,
+                   ch_norm.std if ch_norm.runing_std else None,
+                   ch_norm.mean if ch_norm.runing_mean else None)
+        sp_args = (conv.weight, conv.bias, self.head, k, self.stride,
+                   1.0 if sp_norm.runing_std else sp_norm.std,
+                   sp_norm.std if sp_norm.runing_std else None,
+                   sp_norm.mean if sp_norm.runing_mean else None)
+        # the spatial branch reads every feature plane anyway: where its kernel can, it
+        # leaves the planes' partial sums and the channel branch pools from those
+        pooled = _lib.spatial_branch_pool(x, *sp_args) if self.fuse_pool else None
+        if pooled is not None:
+            sf, parts = pooled
+            return _lib.channel_branch_parts(parts, 1.0 / (x.size(2) * x.size(3)), *ch_args), sf
+        cf = _lib.channel_branch(x.mean((2, 3)), *ch_args)
+        sf = _lib.spatial_branch(x, *sp_args)
         return cf, sf
 
     def forward(self, x):

@@ -272,6 +272,39 @@ int ddf_hip_channel_branch(const void *pooled, const void *weight1,
                            const void *offset_vec, int dtype, void *stream);
 
 /*
+ * The two branches with the global average pool between them folded in
+ * (DDFPack.forward computes the channel filter from the pooled features,
+ * ddf/ddf.py:183-185 and :213-219; no counterpart as a function in the reference).
+ * ddf_hip_spatial_branch_pool is ddf_hip_spatial_branch that also leaves, from
+ * the feature values it has in registers anyway, partial sums of every feature
+ * plane: pool_parts[(n * *n_parts + p) * C + c], fp32, is the sum of
+ * features[n, c] over the pixels of part p.  The caller provides room for
+ * pool_capacity floats (N * C * 4 * ceil((H/stride) * (W/stride) / 64) is always
+ * enough) and gets the number of parts back in *n_parts.
+ * ddf_hip_channel_branch_parts is ddf_hip_channel_branch with the pooled
+ * vector given as scale * (sum of n_parts such partial sums), scale = 1 / (H*W).
+ * One launch and one full read of the feature map fewer per layer than
+ * pooling first.  DDF_ERR_UNSUPPORTED (then pool and call the plain entry
+ * points): kernel size other than 3, odd H or W under stride 2, or a shape the
+ * streaming kernel turns down; DDF_ERR_WORKSPACE: pool_capacity too small.
+ */
+int ddf_hip_spatial_branch_pool(const void *features, const void *weight,
+                                const void *bias, void *spatial_filter,
+                                float *pool_parts, int64_t pool_capacity,
+                                int *n_parts, int64_t N, int64_t C, int64_t H,
+                                int64_t W, int head, int kernel_size, int stride,
+                                double gain, const void *gain_vec,
+                                const void *offset_vec, int dtype, void *stream);
+int ddf_hip_channel_branch_parts(const float *pool_parts, int n_parts,
+                                 double scale, const void *weight1,
+                                 const void *bias1, const void *weight2,
+                                 const void *bias2, void *channel_filter,
+                                 int64_t N, int64_t C, int64_t mid,
+                                 int kernel_size, double gain,
+                                 const void *gain_vec, const void *offset_vec,
+                                 int dtype, void *stream);
+
+/*
  * Up-sampling DDF forward (DDFUpPack.forward, ddf/ddf.py:257-272): the
  * reference calls `ddf` once per sub-pixel branch b = 0 .. scale*scale-1 on
  * the same features with that branch's filters (ddf.py:264-269), stacks the

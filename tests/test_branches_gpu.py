@@ -106,3 +106,62 @@ def test_channel_branch_matches_fp64(n, c, k, dtype, tol):
     ref = channel_reference(*(t.cpu() for t in (pooled, w1, b1, w2, b2)), k, 1.0, gv.cpu(), ov.cpu())
     err = ((out.double().cpu() - ref).abs().max() / ref.abs().max()).item()
     assert err < tol, err
+
+
+POOL_CASES = [(2, 64, 56, 56, 1, 1), (2, 128, 56, 56, 2, 1), (2, 128, 28, 28, 1, 1), (2, 256, 28, 28, 2, 1),
+              (2, 256, 14, 14, 1, 1), (2, 512, 14, 14, 2, 1), (2, 512, 7, 7, 1, 1), (3, 16, 12, 14, 1, 1),
+              (3, 16, 12, 14, 2, 1), (3, 16, 9, 11, 1, 4), (2, 36, 10, 18, 2, 3), (1, 8, 5, 3, 1, 1),
+              (2, 20, 40, 24, 2, 2), (40, 32, 28, 28, 1, 1), (2, 64, 30, 32, 1, 2), (2, 24, 6, 20, 2, 1)]
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.float16])
+@pytest.mark.parametrize('case', POOL_CASES, ids=lambda c: 'x'.join(map(str, c)))
+def test_spatial_branch_pool(case, dtype):
+    """ddf_hip_spatial_branch_pool: the same taps as ddf_hip_spatial_branch, bit for
+    bit, and partial sums that add up to the feature planes' sums (the global
+    average pool of ddf/ddf.py:184 times H * W)."""
+    n, c, h, w_, s, head = case
+    torch.manual_seed(7)
+    x = torch.randn(n, c, h, w_, device='cuda').to(dtype)
+    w = (torch.randn(head * 9, c, device='cuda') * 0.2).to(dtype)
+    b = torch.randn(head * 9, device='cuda').to(dtype)
+    both = _lib.spatial_branch_pool(x, w, b, head, 3, s, 0.7, None, None)
+    assert both is not None
+    sf, parts = both
+    assert parts.dtype == torch.float32 and parts.shape[0] == n and parts.shape[2] == c
+    assert torch.equal(sf, _lib.spatial_branch(x, w, b, head, 3, s, 0.7, None, None))
+    sums = x.double().sum((2, 3)).cpu()
+    scale = x.double().abs().sum((2, 3)).cpu().max()
+    assert ((parts.double().sum(1).cpu() - sums).abs().max() / scale).item() < 1e-6
+
+
+def test_spatial_branch_pool_turns_down_what_it_cannot_cover():
+    x = torch.randn(2, 16, 9, 8, device='cuda')
+    w5 = torch.randn(25, 16, device='cuda')
+    w3 = torch.randn(9, 16, device='cuda')
+    assert _lib.spatial_branch_pool(x, w5, None, 1, 5, 1, 1.0) is None      # 5 x 5 taps
+    assert _lib.spatial_branch_pool(x, w3, None, 1, 3, 2, 1.0) is None      # odd height under stride 2
+    assert _lib.spatial_branch_pool(x[:, :, :8].contiguous(), w3, None, 1, 3, 2, 1.0) is not None
+    assert _lib.spatial_branch_pool(x[:, :15].contiguous(), w3[:, :15].contiguous(), None, 1, 3, 1, 1.0) is None   # odd channel count
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.float16, 6e-3)])
+@pytest.mark.parametrize('n,c,k,tiles', [(3, 16, 3, 1), (128, 64, 3, 13), (5, 128, 3, 4), (4, 256, 3, 2),
+                                         (3, 512, 3, 7), (2, 70, 5, 3)])
+def test_channel_branch_parts_matches_fp64(n, c, k, tiles, dtype, tol):
+    torch.manual_seed(n + c)
+    mid = int(c * 0.2)
+    parts = torch.randn(n, tiles, c, device='cuda')
+    scale = 1.0 / 37
+    w1 = (torch.randn(mid, c, device='cuda') * 0.2).to(dtype)
+    b1 = torch.randn(mid, device='cuda').to(dtype)
+    w2 = (torch.randn(c * k * k, mid, device='cuda') * 0.3).to(dtype)
+    b2 = torch.randn(c * k * k, device='cuda').to(dtype)
+    gv = (torch.rand(c * k * k, device='cuda') + 0.5).to(dtype)
+    ov = torch.randn(c * k * k, device='cuda').to(dtype)
+    out = _lib.channel_branch_parts(parts, scale, w1, b1, w2, b2, k, 1.0, gv, ov)
+    assert out.dtype == dtype
+    pooled = parts.double().sum(1).cpu() * scale
+    ref = channel_reference(pooled, *(t.cpu() for t in (w1, b1, w2, b2)), k, 1.0, gv.cpu(), ov.cpu())
+    err = ((out.double().cpu() - ref).abs().max() / ref.abs().max()).item()
+    assert err < tol, err
