@@ -334,12 +334,14 @@ def profile_branch(index, which, steps, warmup, lib, batch=128):
     mid = int(c * 0.2)
     torch.manual_seed(0)
     nset = max(2, int(600e6 / (batch * c * hw * hw * 2)) + 1)
-    if which == 'spatial':
+    if which in ('spatial', 'spatial_pool'):
         w = torch.randn(9, c, device='cuda', dtype=dt) * 0.1
         b = torch.randn(9, device='cuda', dtype=dt)
         xs = [torch.randn(batch, c, hw, hw, device='cuda', dtype=dt) for _ in range(nset)]
-        run = lambda i: lib.spatial_branch(xs[i % nset], w, b, 1, 3, s, 1.0, None, None)
-        nbytes = batch * c * hw * hw * 2 // s + batch * 9 * (hw // s) ** 2 * 2
+        call = lib.spatial_branch if which == 'spatial' else lib.spatial_branch_pool
+        run = lambda i: call(xs[i % nset], w, b, 1, 3, s, 1.0, None, None)
+        # (what the branch needs; the pooled variant needs every row under stride 2 as well)
+        nbytes = batch * c * hw * hw * 2 // (s if which == 'spatial' else 1) + batch * 9 * (hw // s) ** 2 * 2
     else:
         w1 = torch.randn(mid, c, device='cuda', dtype=dt) * 0.1
         b1 = torch.randn(mid, device='cuda', dtype=dt)
@@ -754,7 +756,7 @@ def main():
                          'batches): the unit the model summary in profiles/ is collected on')
     ap.add_argument('--profile-branch', default=None, metavar='KIND:INDEX',
                     help='run only the spatial or channel branch launch of one ResNet-50 layer shape '
-                         '(spatial:0 .. spatial:6, channel:0 .. channel:6): the unit the branch summary in '
+                         '(spatial:0 .. spatial:6, spatial_pool:0 .. 6, channel:0 .. channel:6): the unit the branch summary in '
                          'profiles/ is collected on')
     ap.add_argument('--copy-probe', action='store_true',
                     help='also run a plain 256 MiB device copy (calibrates hardware counters)')
@@ -773,7 +775,7 @@ def main():
         return
     if args.profile_branch:
         kind, index = args.profile_branch.split(':')
-        assert kind in ('spatial', 'channel') and 0 <= int(index) < len(BRANCH_LAYERS)
+        assert kind in ('spatial', 'spatial_pool', 'channel') and 0 <= int(index) < len(BRANCH_LAYERS)
         print(json.dumps(profile_branch(int(index), kind, args.steps, args.warmup, lib)))
         return
     if args.profile_phase:
