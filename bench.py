@@ -741,8 +741,9 @@ def main():
     ap.add_argument('--all', action='store_true', help='(default now; kept for old command lines)')
     ap.add_argument('--model', action='store_true', help='(default now; kept for old command lines)')
     ap.add_argument('--test-time', action='store_true',
-                    help="also run the reference's micro-benchmark table (conv, depthwise conv, "
-                         "DDFPack, ddf at seven 256-channel shapes)")
+                    help="with --only-headline: also run the reference's micro-benchmark table (conv, "
+                         "depthwise conv, DDFPack, ddf at seven 256-channel shapes; part of the default "
+                         "line otherwise)")
     ap.add_argument('--up-pack', action='store_true',
                     help='with --only-headline: also time the fused up-sampling forward against its '
                          'composition (part of the default line otherwise)')
@@ -823,7 +824,7 @@ def main():
         line['up_forward'] = up_forward_table(lib)
     elif args.up_pack:
         line['up_forward'] = up_forward_table(lib)
-    if args.test_time:
+    if args.test_time or not args.only_headline:
         line['test_time'] = test_time_table()
     if not args.no_cpu:
         line['cpu_baseline'] = cpu_baseline(args.workload)
