@@ -26,9 +26,11 @@ The same line carries the other benchmark configurations
 dilated 5x5 shapes, two more ResNet stages), ddf_mul_resnet50 inference
 (``model_inference``: fp16, batch 128, 224x224, random weights: images/s and
 per-layer GB/s of the DDF layers, operands rotating beyond the last-level
-cache), a DDFPack layer as a training unit (``ddfpack_train``), the fused
-up-sampling forward (``up_forward``) and the CPU baseline; ``--only-headline``
-leaves all but the last out.
+cache; ``filter_branches``: the two branch launches of DDFPack at those layers,
+with and without the pooling on the spatial branch's launch), a DDFPack layer
+as a training unit (``ddfpack_train``), the fused up-sampling forward
+(``up_forward``), the reference's own micro-benchmark table (``test_time``) and
+the CPU baseline; ``--only-headline`` leaves all but the last out.
 
 Prints ONE JSON line on stdout; everything else goes to stderr.
 """
