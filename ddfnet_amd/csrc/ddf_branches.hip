@@ -376,7 +376,7 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
         constexpr int ST = decltype(st_tag)::value;
         const bool have = i < g.gpw && j0 + i < g.ngroups;
         // (a group the wave does not have: every lane's offset lies outside, the loads
-        // return zero; its weights are those of the wave's first group)
+        // return zero - whatever weights they then meet)
         const int j = have ? j0 + i : (j0 < g.ngroups ? j0 : 0);
         const uint32_t vb = have ? xb : kOutside;
         const uint32_t cb = (uint32_t)(j * U) * plane_bytes;
@@ -402,6 +402,14 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
                                   xlow[ST][u]);
             }
         }
+    };
+    // The weights of group i, stage ST.  They are requested one step ahead only (a scalar
+    // load is back well within a step), so two of the NST register sets are alive at any
+    // time: with all of them the pooled variants run out of scalar registers.
+    auto issue_weights = [&](auto st_tag, int i) __attribute__((always_inline)) {
+        constexpr int ST = decltype(st_tag)::value;
+        const bool have = i < g.gpw && j0 + i < g.ngroups;
+        const int j = have ? j0 + i : (j0 < g.ngroups ? j0 : 0);
         const uint32_t wb = (uint32_t)(j * U) * (uint32_t)sizeof(T);
 #pragma unroll
         for (int t = 0; t < KK; ++t)
@@ -431,13 +439,20 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
                     if constexpr (sizeof(T) == 2 && kXB == 2) {
                         ps = (float)__builtin_bit_cast(_Float16, xh[ST][u]);
                     } else if constexpr (sizeof(T) == 2) {
+                        // (every word on its own, then a tree of additions: one accumulator for
+                        // all words is a chain of dependent dot products, each waiting out the
+                        // latency of the one before)
                         const rows::half2_t ones = {(_Float16)1, (_Float16)1};
+                        float part[NWX];
 #pragma unroll
                         for (int k = 0; k < NWX; ++k) {
-                            ps = __builtin_amdgcn_fdot2(__builtin_bit_cast(rows::half2_t, xw[ST][u][k]), ones, ps, false);
+                            part[k] = __builtin_amdgcn_fdot2(__builtin_bit_cast(rows::half2_t, xw[ST][u][k]), ones, 0.f, false);
                             if constexpr (S == 2)
-                                ps = __builtin_amdgcn_fdot2(__builtin_bit_cast(rows::half2_t, xlow[ST][u][k]), ones, ps, false);
+                                part[k] = __builtin_amdgcn_fdot2(__builtin_bit_cast(rows::half2_t, xlow[ST][u][k]), ones, part[k], false);
                         }
+                        if constexpr (NWX == 4) ps = (part[0] + part[1]) + (part[2] + part[3]);
+                        else if constexpr (NWX == 2) ps = part[0] + part[1];
+                        else ps = part[0];
                     } else {
 #pragma unroll
                         for (int k = 0; k < NWX; ++k) {
@@ -491,6 +506,7 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
     };
     // (in this order: the waits inside the walk count the loads that were issued later)
     issue(std::integral_constant<int, 0>{}, 0);
+    issue_weights(std::integral_constant<int, 0>{}, 0);
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (NST > 2) issue(std::integral_constant<int, 1>{}, 1);
     __builtin_amdgcn_sched_barrier(0);
@@ -499,6 +515,7 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
     auto step = [&](auto st_tag, int i) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         issue(std::integral_constant<int, (ST + NST - 1) % NST>{}, i + NST - 1);
+        issue_weights(std::integral_constant<int, (ST + 1) % NST>{}, i + 1);
         __builtin_amdgcn_sched_barrier(0);
         compute(st_tag, i);
         __builtin_amdgcn_sched_barrier(0);
