@@ -62,11 +62,23 @@ bool cut_channels_forward(RowsGeom &t, int64_t N, int C, int nst, int64_t plane,
     const int target = tune_int("DDF_TUNE_ROWS_WAVES", 8192);
     const int64_t want_split = std::max<int64_t>(1, (target + base - 1) / base);
     int cpw = (int)(C / want_split);
-    // Small planes (up to 32 x 32) walk four rounds at least where that still leaves a
-    // thousand waves: with operands that really come from memory, walks of 12 channels
-    // beat walks of 6 by 10-15 % at 7 x 7 and 14 x 14 (the spatial taps a wave loads first
-    // are paid for once per walk); larger planes and small batches lose by it.
-    const int rounds = (plane <= 1024 && (int64_t)C * base >= 1024 * 4 * nst) ? 4 : 2;
+    // Small planes (up to 32 x 32) walk more rounds where that still leaves a wave per
+    // SIMD: the spatial taps a wave loads first are paid for once per walk.  Measured with
+    // operands that really come from memory (fp16 and fp32, batches of 8 to 256): planes
+    // up to 16 x 16 want walks of 12 channels once those leave a thousand waves (10-15 %
+    // over walks of 6) and of 24 once those leave some three thousand (7-9 % more); planes
+    // up to 32 x 32 want the longest of 18, 12 and 9 that leaves a thousand (6-11 % over
+    // 12 at 28 x 28).  Larger planes and small batches lose by longer walks.
+    auto waves_with = [&](int rnds) { return base * ((C + rnds * nst - 1) / (rnds * nst)); };
+    int rounds = 2;
+    if (plane <= 256) {
+        if (waves_with(8) >= 2816) rounds = 8;
+        else if (waves_with(4) >= 1024) rounds = 4;
+    } else if (plane <= 1024) {
+        if (waves_with(6) >= 1024) rounds = 6;
+        else if (waves_with(4) >= 1024) rounds = 4;
+        else if (waves_with(3) >= 900) rounds = 3;
+    }
     const int min_cpw = tune_int("DDF_TUNE_ROWS_MIN_CPW", std::max(rounds * nst, (min_walk + nst - 1) / nst * nst));
     cpw = std::max(cpw / nst * nst, min_cpw);
     const int forced = tune_int("DDF_TUNE_ROWS_CPW", 0);
