@@ -18,6 +18,7 @@
 // Both kernels are bound by memory and launch latency, not by arithmetic: the
 // spatial branch does KK multiply-adds per 4-byte (2-byte) load.
 #include <algorithm>
+#include <type_traits>
 
 #include "ddf_common.h"
 #include "ddf_rows.h"
@@ -699,6 +700,196 @@ __global__ __launch_bounds__(kChannelThreads) void k_channel_branch(
     }
 }
 
+
+// ---- the channel branch on the matrix cores (fp16) ---------------------------
+//
+// Both 1x1 convolutions are matrix products with the batch as one dimension:
+//   hidden[m, n] = relu(b1[m] + sum_c w1[m, c] * v[n, c])           (mid x C) . (C x N)
+//   taps[r, n]   = b2[r] + sum_m w2[r, m] * hidden[m, n]            (C*KK x mid) . (mid x N)
+// v_mfma_f32_16x16x32_f16 takes, per lane l of a wave, eight values of a row of A
+// (row l % 16, positions 8 * (l / 16) + 0..7 of the 32 the step covers: one
+// 16-byte load from a row-major weight matrix) and the eight values of column
+// l % 16 of B at the same positions, and leaves D[4 * (l / 16) + 0..3][l % 16].
+// A workgroup takes sixteen samples (the columns) and `block` channels:
+//   * the pooled vectors go to LDS as [32 channels][sample][32], rounded to fp16
+//     (what the reference's half-precision pooling returns);
+//   * the hidden layer goes to LDS as [32 values][sample][32], rounded to fp16 (as
+//     the reference's first convolution does);
+//   * the rows of tile j of the second product are (channel c0 + i, tap j), so a
+//     lane ends up with all KK taps of four channels of one sample and
+//     normalises them in registers: 4 * KK contiguous values to store.
+// mid is no multiple of 32 (nor of 16): the last tile of hidden values starts at
+// mid - 32 (mid - 16 for the rows of the first product) and overlaps the one
+// before it; the overlapping positions of its B operand are zero (they are
+// counted in the tile before), so every weight that is read is a weight of the
+// row it is used for.  Rows of w2 start at any even byte address: its loads are
+// 16 bytes at 2-byte alignment.
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ half8_t load_half8_any(const __half *p) {
+    half8_t v;
+    __builtin_memcpy(&v, p, sizeof(v));
+    return v;
+}
+__device__ __forceinline__ half8_t load_half8(const __half *p) {
+    return *reinterpret_cast<const half8_t *>(p);
+}
+__device__ __forceinline__ half4_t load_half4(const __half *p) {
+    return *reinterpret_cast<const half4_t *>(p);
+}
+
+constexpr int kMmaSamples = 16;
+constexpr int kMmaStep = 32;                          // values of the summed dimension per instruction
+constexpr int kMmaTile = kMmaSamples * kMmaStep;      // halves of one [sample][32] tile in LDS
+
+template <int KK, int WAVES>
+__global__ __launch_bounds__(WAVES * kWave) void k_channel_branch_mma(
+    const __half *__restrict__ pooled, const __half *__restrict__ w1, const __half *__restrict__ b1,
+    const __half *__restrict__ w2, const __half *__restrict__ b2, __half *__restrict__ cf, int N, int C,
+    int mid, int block, float gain, const __half *__restrict__ gain_vec,
+    const __half *__restrict__ offset_vec, const float *__restrict__ parts, int nparts, float scale) {
+    extern __shared__ __align__(16) _Float16 mma_smem[];
+    _Float16 *pv = mma_smem;                        // [C / 32][16 samples][32]: pooled vectors
+    _Float16 *hv = pv + (C / kMmaStep) * kMmaTile;  // [tiles of mid][16 samples][32]: hidden vectors
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int col = lane & 15, quad = lane >> 4;
+    const int n0 = blockIdx.y * kMmaSamples;
+    const int cb = blockIdx.x * block;
+    const int rtiles = (mid + 15) >> 4;             // tiles of sixteen rows of w1
+    const int ktiles = (mid + kMmaStep - 1) / kMmaStep;   // steps of the second product
+    const int klast = mid - kMmaStep;               // where the last of them starts
+
+    // pooled vectors of the sixteen samples: four channels per item
+    const int c4s = C >> 2;
+    for (int i = threadIdx.x; i < kMmaSamples * c4s; i += WAVES * kWave) {
+        const int s = i / c4s, c4 = i - s * c4s;
+        const int64_t n = min(n0 + s, N - 1);
+        half4_t v;
+        if (parts) {
+            const float4_t *src = reinterpret_cast<const float4_t *>(parts + n * nparts * C) + c4;
+            float4_t a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+            for (int q = 0; q < nparts; ++q) a += src[(int64_t)q * c4s];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = (_Float16)(a[e] * scale);
+        } else {
+            v = load_half4(pooled + n * C + c4 * 4);
+        }
+        *reinterpret_cast<half4_t *>(pv + ((c4 >> 3) * kMmaSamples + s) * kMmaStep + (c4 & 7) * 4) = v;
+    }
+    // the last tile of the hidden layer starts out as zeros (its overlap with the tile before stays zero)
+    for (int i = threadIdx.x; i < kMmaTile / 2; i += WAVES * kWave)
+        reinterpret_cast<uint32_t *>(hv + (ktiles - 1) * kMmaTile)[i] = 0u;
+    __syncthreads();
+
+    // hidden layer: tiles of sixteen rows of w1
+    for (int t = wave; t < rtiles; t += WAVES) {
+        const int mbase = min(t * 16, mid - 16);
+        const __half *arow = w1 + (int64_t)(mbase + col) * C + quad * 8;
+        const _Float16 *brow = pv + col * kMmaStep + quad * 8;
+        float4_t acc = {0.f, 0.f, 0.f, 0.f};
+        // (the matrix instruction is convergent, which rules out unrolling with a
+        // remainder: chunks of a fixed number of steps, all loads of a chunk first)
+        int kb = 0;
+        auto chunk = [&](auto steps) {
+            constexpr int U = decltype(steps)::value;
+            half8_t a[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) a[u] = load_half8(arow + (kb + u) * kMmaStep);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                    a[u], *reinterpret_cast<const half8_t *>(brow + (kb + u) * kMmaTile), acc, 0, 0, 0);
+            kb += U;
+        };
+        const int nk = C / kMmaStep;
+        while (nk - kb >= 16) chunk(std::integral_constant<int, 16>());
+        if (nk - kb >= 8) chunk(std::integral_constant<int, 8>());
+        if (nk - kb >= 4) chunk(std::integral_constant<int, 4>());
+        while (kb < nk) chunk(std::integral_constant<int, 1>());
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int m = mbase + quad * 4 + e;
+            if (m < t * 16) continue;    // (the last tile's overlap: those rows belong to the tile before)
+            const float bias = b1 ? ld(b1 + m) : 0.f;
+            const int kt = min(m / kMmaStep, ktiles - 1);
+            hv[(kt * kMmaSamples + col) * kMmaStep + m - min(kt * kMmaStep, klast)] =
+                (_Float16)fmaxf(acc[e] + bias, 0.f);
+        }
+    }
+    __syncthreads();
+
+    // taps: per wave sixteen channels x KK taps x sixteen samples
+    const int n = n0 + col;
+    for (int ct = wave; ct * 16 < block && cb + ct * 16 < C; ct += WAVES) {
+        const int c0 = cb + ct * 16;
+        // gains, offsets and biases of this lane's four channels: 4 * KK contiguous values each
+        const int64_t pbase = (int64_t)(c0 + quad * 4) * KK;
+        half4_t pg[KK], po[KK], pb[KK];
+#pragma unroll
+        for (int j = 0; j < KK; ++j) {
+            pg[j] = po[j] = pb[j] = half4_t{0, 0, 0, 0};
+            if (gain_vec) pg[j] = load_half4(gain_vec + pbase + 4 * j);
+            if (offset_vec) po[j] = load_half4(offset_vec + pbase + 4 * j);
+            if (b2) pb[j] = load_half4(b2 + pbase + 4 * j);
+        }
+        float4_t acc[KK];
+#pragma unroll
+        for (int j = 0; j < KK; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        const __half *arow = w2 + (int64_t)(c0 + col) * KK * mid + quad * 8;
+        const _Float16 *brow = hv + col * kMmaStep + quad * 8;
+        int t = 0;
+        auto tiles = [&](auto count) {
+            constexpr int U = decltype(count)::value;
+            half8_t a[U][KK];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int kbase = min((t + u) * kMmaStep, klast);
+#pragma unroll
+                for (int j = 0; j < KK; ++j) a[u][j] = load_half8_any(arow + j * mid + kbase);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const half8_t b = *reinterpret_cast<const half8_t *>(brow + (t + u) * kMmaTile);
+#pragma unroll
+                for (int j = 0; j < KK; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[u][j], b, acc[j], 0, 0, 0);
+            }
+            t += U;
+        };
+        constexpr int kDeep = KK <= 9 ? 4 : 1;
+        while (ktiles - t >= kDeep) tiles(std::integral_constant<int, kDeep>());
+        if (kDeep > 2 && ktiles - t >= 2) tiles(std::integral_constant<int, 2>());
+        if (kDeep > 1 && t < ktiles) tiles(std::integral_constant<int, 1>());
+        if (n >= N) continue;
+        half4_t out[KK];   // channel e of the lane's four: values [e * KK, (e + 1) * KK) of the 4 * KK
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float u[KK];
+            TapParams<__half, KK> params;
+#pragma unroll
+            for (int j = 0; j < KK; ++j) {
+                const int at = e * KK + j;
+                u[j] = acc[j][e];
+                params.gain[j] = gain_vec ? (float)pg[at >> 2][at & 3] : gain;
+                params.offset[j] = offset_vec ? (float)po[at >> 2][at & 3] : 0.f;
+                params.bias[j] = b2 ? (float)pb[at >> 2][at & 3] : 0.f;
+            }
+            normalise<__half, KK>(u, params);
+#pragma unroll
+            for (int j = 0; j < KK; ++j) {
+                const int at = e * KK + j;
+                out[at >> 2][at & 3] = (_Float16)u[j];
+            }
+        }
+        half4_t *op = reinterpret_cast<half4_t *>(cf + ((int64_t)n * C + c0 + quad * 4) * KK);
+#pragma unroll
+        for (int j = 0; j < KK; ++j) op[j] = out[j];
+    }
+}
+
 }  // namespace
 
 bool branch_kernel_size_built(int k) { return k == 3 || k == 5; }
@@ -879,6 +1070,46 @@ hipError_t spatial_branch(const T *x, const T *w, const T *bias, T *sf, int64_t 
     return hipGetLastError();
 }
 
+// The matrix-core kernel where it applies (fp16, a hidden layer of at least one
+// step of the matrix instruction, whole steps of channels, operands aligned for
+// its vector loads); hipErrorNotSupported otherwise.
+template <typename T>
+hipError_t channel_branch_mma(const T *, const T *, const T *, const T *, const T *, T *, int64_t, int64_t,
+                              int64_t, int, double, const T *, const T *, hipStream_t, const float *, int,
+                              double) {
+    return hipErrorNotSupported;
+}
+template <>
+hipError_t channel_branch_mma<__half>(const __half *pooled, const __half *w1, const __half *b1,
+                                      const __half *w2, const __half *b2, __half *cf, int64_t N, int64_t C,
+                                      int64_t mid, int k, double gain, const __half *gain_vec,
+                                      const __half *offset_vec, hipStream_t st, const float *parts,
+                                      int nparts, double scale) {
+    if (tune_int("DDF_TUNE_CHANNEL_MMA", 1) == 0) return hipErrorNotSupported;
+    auto aligned = [](const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; };
+    const size_t lds = (size_t)(C / kMmaStep + cdiv(mid, kMmaStep)) * kMmaTile * sizeof(__half);
+    if ((k != 3 && k != 5) || mid < kMmaStep || C % kMmaStep != 0 || lds > 64 * 1024 ||
+        N > (int64_t)65535 * kMmaSamples || C * k * k * mid >= ((int64_t)1 << 31))
+        return hipErrorNotSupported;
+    if (!aligned(w1, 16) || !aligned(cf, 8) || !aligned(b2, 8) || !aligned(gain_vec, 8) ||
+        !aligned(offset_vec, 8) || !aligned(w2, 2) || (parts ? !aligned(parts, 16) : !aligned(pooled, 8)))
+        return hipErrorNotSupported;
+    const int waves = tune_int("DDF_TUNE_CHANNEL_MMA_WAVES", 8) == 8 ? 8 : 4;
+    int block = tune_int("DDF_TUNE_CHANNEL_MMA_BLOCK", 16);
+    block = std::max(16, block / 16 * 16);
+    const dim3 grid((unsigned)cdiv(C, block), (unsigned)cdiv(N, kMmaSamples));
+#define DDF_MMA_LAUNCH(KK_, WAVES_)                                                                  \
+    hipLaunchKernelGGL((k_channel_branch_mma<KK_, WAVES_>), grid, dim3(WAVES_ * kWave), lds, st, pooled, \
+                       w1, b1, w2, b2, cf, (int)N, (int)C, (int)mid, block, (float)gain, gain_vec,      \
+                       offset_vec, parts, nparts, (float)scale)
+    if (k == 3 && waves == 8) DDF_MMA_LAUNCH(9, 8);
+    else if (k == 3) DDF_MMA_LAUNCH(9, 4);
+    else if (waves == 8) DDF_MMA_LAUNCH(25, 8);
+    else DDF_MMA_LAUNCH(25, 4);
+#undef DDF_MMA_LAUNCH
+    return hipGetLastError();
+}
+
 template <typename T>
 hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2, const T *b2,
                           T *cf, int64_t N, int64_t C, int64_t mid, int k, double gain,
@@ -886,6 +1117,10 @@ hipError_t channel_branch(const T *pooled, const T *w1, const T *b1, const T *w2
                           int nparts, double scale) {
     if (N == 0 || C == 0) return hipSuccess;
     const int kk = k * k;
+    if (hipError_t e = channel_branch_mma(pooled, w1, b1, w2, b2, cf, N, C, mid, k, gain, gain_vec,
+                                          offset_vec, st, parts, nparts, scale);
+        e != hipErrorNotSupported)
+        return e;
     // (wide layers: fewer, larger blocks, as every block of a sample recomputes the hidden vector)
     const int block = C >= 512 ? 128 : 64;
     // samples per workgroup: as many as keep every compute unit busy and fit the LDS
