@@ -753,94 +753,166 @@ __global__ __launch_bounds__(WAVES * kWave) void k_channel_branch_mma(
     extern __shared__ __align__(16) _Float16 mma_smem[];
     _Float16 *pv = mma_smem;                        // [C / 32][16 samples][32]: pooled vectors
     _Float16 *hv = pv + (C / kMmaStep) * kMmaTile;  // [tiles of mid][16 samples][32]: hidden vectors
-    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int col = lane & 15, quad = lane >> 4;
     const int n0 = blockIdx.y * kMmaSamples;
     const int cb = blockIdx.x * block;
     const int rtiles = (mid + 15) >> 4;             // tiles of sixteen rows of w1
     const int ktiles = (mid + kMmaStep - 1) / kMmaStep;   // steps of the second product
     const int klast = mid - kMmaStep;               // where the last of them starts
+    const int nk = C / kMmaStep;                    // steps of the first product
 
-    // pooled vectors of the sixteen samples: four channels per item
-    const int c4s = C >> 2;
-    for (int i = threadIdx.x; i < kMmaSamples * c4s; i += WAVES * kWave) {
-        const int s = i / c4s, c4 = i - s * c4s;
-        const int64_t n = min(n0 + s, N - 1);
-        half4_t v;
-        if (parts) {
-            const float4_t *src = reinterpret_cast<const float4_t *>(parts + n * nparts * C) + c4;
-            float4_t a = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-            for (int q = 0; q < nparts; ++q) a += src[(int64_t)q * c4s];
+    // All waves: the pooled vectors of the sixteen samples into LDS, four channels per
+    // item (given, or scale * the sum of nparts partial sums per value), and zeros in
+    // the last tile of the hidden layer (its overlap with the tile before stays zero).
+    auto pooled_vectors = [&]() {
+        const int c4s = C >> 2;
+        for (int i = threadIdx.x; i < kMmaSamples * c4s; i += WAVES * kWave) {
+            const int s = i / c4s, c4 = i - s * c4s;
+            const int64_t n = min(n0 + s, N - 1);
+            half4_t v;
+            if (parts) {
+                const float4_t *src = reinterpret_cast<const float4_t *>(parts + n * nparts * C) + c4;
+                float4_t a = {0.f, 0.f, 0.f, 0.f};
+                // four partial sums requested together (the fence keeps the compiler from
+                // taking them one round trip at a time to save registers)
+                int q = 0;
+                for (; q + 4 <= nparts; q += 4) {
+                    const float4_t x0 = src[(int64_t)q * c4s], x1 = src[(int64_t)(q + 1) * c4s],
+                                   x2 = src[(int64_t)(q + 2) * c4s], x3 = src[(int64_t)(q + 3) * c4s];
+                    __builtin_amdgcn_sched_barrier(0);
+                    a += (x0 + x1) + (x2 + x3);
+                }
+                for (; q < nparts; ++q) a += src[(int64_t)q * c4s];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = (_Float16)(a[e] * scale);
-        } else {
-            v = load_half4(pooled + n * C + c4 * 4);
+                for (int e = 0; e < 4; ++e) v[e] = (_Float16)(a[e] * scale);
+            } else {
+                v = load_half4(pooled + n * C + c4 * 4);
+            }
+            *reinterpret_cast<half4_t *>(pv + ((c4 >> 3) * kMmaSamples + s) * kMmaStep + (c4 & 7) * 4) = v;
         }
-        *reinterpret_cast<half4_t *>(pv + ((c4 >> 3) * kMmaSamples + s) * kMmaStep + (c4 & 7) * 4) = v;
-    }
-    // the last tile of the hidden layer starts out as zeros (its overlap with the tile before stays zero)
-    for (int i = threadIdx.x; i < kMmaTile / 2; i += WAVES * kWave)
-        reinterpret_cast<uint32_t *>(hv + (ktiles - 1) * kMmaTile)[i] = 0u;
-    __syncthreads();
+        for (int i = threadIdx.x; i < kMmaTile / 2; i += WAVES * kWave)
+            reinterpret_cast<uint32_t *>(hv + (ktiles - 1) * kMmaTile)[i] = 0u;
+    };
 
-    // hidden layer: tiles of sixteen rows of w1
-    for (int t = wave; t < rtiles; t += WAVES) {
-        const int mbase = min(t * 16, mid - 16);
-        const __half *arow = w1 + (int64_t)(mbase + col) * C + quad * 8;
-        const _Float16 *brow = pv + col * kMmaStep + quad * 8;
-        float4_t acc = {0.f, 0.f, 0.f, 0.f};
-        // (the matrix instruction is convergent, which rules out unrolling with a
-        // remainder: chunks of a fixed number of steps, all loads of a chunk first)
-        int kb = 0;
-        auto chunk = [&](auto steps) {
-            constexpr int U = decltype(steps)::value;
-            half8_t a[U];
+    // The first waves compute taps (a tile of sixteen channels at a time), the others
+    // the hidden layer; each kind asks for the first weights it will need before
+    // anything else (they depend on nothing, and are there by the time the operand
+    // from LDS is).  The two kinds run separate code, so each has the whole register
+    // file for what it keeps in flight; both pass the same two barriers.
+    const int tap_waves = min(min(block, C - cb) >> 4, WAVES - 1);
+    if (wave >= tap_waves) {
+        // ---- hidden layer: tiles of sixteen rows of w1 ----
+        constexpr int kPre1 = 16;
+        const int hidden_waves = WAVES - tap_waves;
+        const int t0 = wave - tap_waves;
+        half8_t apre[kPre1];
+        auto request = [&](int t) {
+            const __half *arow = w1 + (int64_t)(min(t * 16, mid - 16) + col) * C + quad * 8;
 #pragma unroll
-            for (int u = 0; u < U; ++u) a[u] = load_half8(arow + (kb + u) * kMmaStep);
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                    a[u], *reinterpret_cast<const half8_t *>(brow + (kb + u) * kMmaTile), acc, 0, 0, 0);
-            kb += U;
+            for (int u = 0; u < kPre1; ++u) apre[u] = load_half8(arow + min(u, nk - 1) * kMmaStep);
         };
-        const int nk = C / kMmaStep;
-        while (nk - kb >= 16) chunk(std::integral_constant<int, 16>());
-        if (nk - kb >= 8) chunk(std::integral_constant<int, 8>());
-        if (nk - kb >= 4) chunk(std::integral_constant<int, 4>());
-        while (kb < nk) chunk(std::integral_constant<int, 1>());
+        if (t0 < rtiles) request(t0);
+        pooled_vectors();
+        __syncthreads();
+        for (int t = t0; t < rtiles; t += hidden_waves) {
+            if (t != t0) request(t);
+            const int mbase = min(t * 16, mid - 16);
+            const __half *arow = w1 + (int64_t)(mbase + col) * C + quad * 8;
+            const _Float16 *brow = pv + col * kMmaStep + quad * 8;
+            float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int m = mbase + quad * 4 + e;
-            if (m < t * 16) continue;    // (the last tile's overlap: those rows belong to the tile before)
-            const float bias = b1 ? ld(b1 + m) : 0.f;
-            const int kt = min(m / kMmaStep, ktiles - 1);
-            hv[(kt * kMmaSamples + col) * kMmaStep + m - min(kt * kMmaStep, klast)] =
-                (_Float16)fmaxf(acc[e] + bias, 0.f);
+            for (int u = 0; u < kPre1; ++u) {
+                if (u < nk)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        apre[u], *reinterpret_cast<const half8_t *>(brow + u * kMmaTile), acc, 0, 0, 0);
+            }
+            // (the matrix instruction is convergent, which rules out unrolling with a
+            // remainder: chunks of a fixed number of steps, all loads of a chunk first)
+            int kb = kPre1;
+            auto chunk = [&](auto steps) {
+                constexpr int U = decltype(steps)::value;
+                half8_t a[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) a[u] = load_half8(arow + (kb + u) * kMmaStep);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                        a[u], *reinterpret_cast<const half8_t *>(brow + (kb + u) * kMmaTile), acc, 0, 0, 0);
+                kb += U;
+            };
+            while (nk - kb >= 16) chunk(std::integral_constant<int, 16>());
+            if (nk - kb >= 8) chunk(std::integral_constant<int, 8>());
+            if (nk - kb >= 4) chunk(std::integral_constant<int, 4>());
+            while (kb < nk) chunk(std::integral_constant<int, 1>());
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int m = mbase + quad * 4 + e;
+                if (m < t * 16) continue;    // (the last tile's overlap: those rows belong to the tile before)
+                const float bias = b1 ? ld(b1 + m) : 0.f;
+                const int kt = min(m / kMmaStep, ktiles - 1);
+                hv[(kt * kMmaSamples + col) * kMmaStep + m - min(kt * kMmaStep, klast)] =
+                    (_Float16)fmaxf(acc[e] + bias, 0.f);
+            }
         }
+        __syncthreads();
+        return;
     }
-    __syncthreads();
 
-    // taps: per wave sixteen channels x KK taps x sixteen samples
-    const int n = n0 + col;
-    for (int ct = wave; ct * 16 < block && cb + ct * 16 < C; ct += WAVES) {
-        const int c0 = cb + ct * 16;
+    // ---- taps: per wave sixteen channels x KK taps x sixteen samples ----
+    constexpr int kPre = KK <= 9 ? 2 : 1;           // steps of the second product requested up front
+    half4_t pg[KK], po[KK], pb[KK];
+    half8_t apre[kPre][KK];
+    auto request = [&](int c0) {
         // gains, offsets and biases of this lane's four channels: 4 * KK contiguous values each
         const int64_t pbase = (int64_t)(c0 + quad * 4) * KK;
-        half4_t pg[KK], po[KK], pb[KK];
 #pragma unroll
-        for (int j = 0; j < KK; ++j) {
-            pg[j] = po[j] = pb[j] = half4_t{0, 0, 0, 0};
-            if (gain_vec) pg[j] = load_half4(gain_vec + pbase + 4 * j);
-            if (offset_vec) po[j] = load_half4(offset_vec + pbase + 4 * j);
-            if (b2) pb[j] = load_half4(b2 + pbase + 4 * j);
+        for (int j = 0; j < KK; ++j) pg[j] = po[j] = pb[j] = half4_t{0, 0, 0, 0};
+        if (gain_vec) {
+#pragma unroll
+            for (int j = 0; j < KK; ++j) pg[j] = load_half4(gain_vec + pbase + 4 * j);
         }
+        if (offset_vec) {
+#pragma unroll
+            for (int j = 0; j < KK; ++j) po[j] = load_half4(offset_vec + pbase + 4 * j);
+        }
+        if (b2) {
+#pragma unroll
+            for (int j = 0; j < KK; ++j) pb[j] = load_half4(b2 + pbase + 4 * j);
+        }
+        const __half *arow = w2 + (int64_t)(c0 + col) * KK * mid + quad * 8;
+#pragma unroll
+        for (int u = 0; u < kPre; ++u) {
+            const int kbase = min(u * kMmaStep, klast);    // (steps past the last one: the last one again, unused)
+#pragma unroll
+            for (int j = 0; j < KK; ++j) apre[u][j] = load_half8_any(arow + j * mid + kbase);
+        }
+    };
+    request(cb + wave * 16);
+    pooled_vectors();
+    __syncthreads();
+    __syncthreads();
+    const int n = n0 + col;
+    for (int ct = wave; ct * 16 < block && cb + ct * 16 < C; ct += tap_waves) {
+        const int c0 = cb + ct * 16;
+        if (ct != wave) request(c0);
         float4_t acc[KK];
 #pragma unroll
         for (int j = 0; j < KK; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
         const __half *arow = w2 + (int64_t)(c0 + col) * KK * mid + quad * 8;
         const _Float16 *brow = hv + col * kMmaStep + quad * 8;
-        int t = 0;
+#pragma unroll
+        for (int u = 0; u < kPre; ++u) {
+            if (u < ktiles) {
+                const half8_t b = *reinterpret_cast<const half8_t *>(brow + u * kMmaTile);
+#pragma unroll
+                for (int j = 0; j < KK; ++j)
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(apre[u][j], b, acc[j], 0, 0, 0);
+            }
+        }
+        int t = kPre;
         auto tiles = [&](auto count) {
             constexpr int U = decltype(count)::value;
             half8_t a[U][KK];
@@ -850,6 +922,7 @@ __global__ __launch_bounds__(WAVES * kWave) void k_channel_branch_mma(
 #pragma unroll
                 for (int j = 0; j < KK; ++j) a[u][j] = load_half8_any(arow + j * mid + kbase);
             }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const half8_t b = *reinterpret_cast<const half8_t *>(brow + (t + u) * kMmaTile);
@@ -859,10 +932,8 @@ __global__ __launch_bounds__(WAVES * kWave) void k_channel_branch_mma(
             }
             t += U;
         };
-        constexpr int kDeep = KK <= 9 ? 4 : 1;
-        while (ktiles - t >= kDeep) tiles(std::integral_constant<int, kDeep>());
-        if (kDeep > 2 && ktiles - t >= 2) tiles(std::integral_constant<int, 2>());
-        if (kDeep > 1 && t < ktiles) tiles(std::integral_constant<int, 1>());
+        while (ktiles - t >= kPre) tiles(std::integral_constant<int, kPre>());
+        if (kPre > 1 && t < ktiles) tiles(std::integral_constant<int, 1>());
         if (n >= N) continue;
         half4_t out[KK];   // channel e of the lane's four: values [e * KK, (e + 1) * KK) of the 4 * KK
 #pragma unroll
@@ -1094,7 +1165,8 @@ hipError_t channel_branch_mma<__half>(const __half *pooled, const __half *w1, co
     if (!aligned(w1, 16) || !aligned(cf, 8) || !aligned(b2, 8) || !aligned(gain_vec, 8) ||
         !aligned(offset_vec, 8) || !aligned(w2, 2) || (parts ? !aligned(parts, 16) : !aligned(pooled, 8)))
         return hipErrorNotSupported;
-    const int waves = tune_int("DDF_TUNE_CHANNEL_MMA_WAVES", 8) == 8 ? 8 : 4;
+    // (25 taps: the accumulators and parameters of a tile need the registers of a wave alone on its SIMD)
+    const int waves = k == 3 && tune_int("DDF_TUNE_CHANNEL_MMA_WAVES", 8) == 8 ? 8 : 4;
     int block = tune_int("DDF_TUNE_CHANNEL_MMA_BLOCK", 16);
     block = std::max(16, block / 16 * 16);
     const dim3 grid((unsigned)cdiv(C, block), (unsigned)cdiv(N, kMmaSamples));
@@ -1104,7 +1176,6 @@ hipError_t channel_branch_mma<__half>(const __half *pooled, const __half *w1, co
                        offset_vec, parts, nparts, (float)scale)
     if (k == 3 && waves == 8) DDF_MMA_LAUNCH(9, 8);
     else if (k == 3) DDF_MMA_LAUNCH(9, 4);
-    else if (waves == 8) DDF_MMA_LAUNCH(25, 8);
     else DDF_MMA_LAUNCH(25, 4);
 #undef DDF_MMA_LAUNCH
     return hipGetLastError();
