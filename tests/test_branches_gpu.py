@@ -91,7 +91,11 @@ def test_spatial_branch_unaligned_views(dtype, tol):
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.float16, 6e-3)])
 @pytest.mark.parametrize('n,c,k', [(3, 16, 3), (128, 64, 3), (5, 128, 3), (4, 256, 3), (3, 512, 3),
                                    (2, 70, 5), (7, 300, 3), (2, 1024, 3), (3, 64, 5), (6, 96, 3),
-                                   (130, 512, 3), (9, 256, 5)])
+                                   (130, 512, 3), (9, 256, 5),
+                                   # fp16 on the matrix cores: hidden layers of exactly one step, of a
+                                   # step and a few values, of several steps; batches that end inside a tile
+                                   (16, 160, 3), (4, 192, 3), (20, 320, 3), (2, 448, 5), (33, 1024, 3),
+                                   (17, 1280, 3)])
 def test_channel_branch_matches_fp64(n, c, k, dtype, tol):
     torch.manual_seed(n + c)
     mid = int(c * 0.2)
@@ -106,6 +110,21 @@ def test_channel_branch_matches_fp64(n, c, k, dtype, tol):
     ref = channel_reference(*(t.cpu() for t in (pooled, w1, b1, w2, b2)), k, 1.0, gv.cpu(), ov.cpu())
     err = ((out.double().cpu() - ref).abs().max() / ref.abs().max()).item()
     assert err < tol, err
+
+
+@pytest.mark.parametrize('n,c,k', [(5, 256, 3), (18, 512, 3), (3, 160, 5), (4, 64, 3)])
+def test_channel_branch_without_biases_and_vectors(n, c, k):
+    """Scalar gain, no offset, no biases (fp16: the matrix-core kernel where the shape allows it)."""
+    torch.manual_seed(c)
+    mid = int(c * 0.2)
+    pooled = torch.randn(n, c, device='cuda').half()
+    w1 = (torch.randn(mid, c, device='cuda') * 0.2).half()
+    w2 = (torch.randn(c * k * k, mid, device='cuda') * 0.3).half()
+    out = _lib.channel_branch(pooled, w1, None, w2, None, k, 0.7, None, None)
+    zeros1, zeros2 = torch.zeros(mid), torch.zeros(c * k * k)
+    ref = channel_reference(pooled.cpu(), w1.cpu(), zeros1, w2.cpu(), zeros2, k, 0.7, None, None)
+    err = ((out.double().cpu() - ref).abs().max() / ref.abs().max()).item()
+    assert err < 6e-3, err
 
 
 POOL_CASES = [(2, 64, 56, 56, 1, 1), (2, 128, 56, 56, 2, 1), (2, 128, 28, 28, 1, 1), (2, 256, 28, 28, 2, 1),
@@ -147,7 +166,8 @@ def test_spatial_branch_pool_turns_down_what_it_cannot_cover():
 
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.float16, 6e-3)])
 @pytest.mark.parametrize('n,c,k,tiles', [(3, 16, 3, 1), (128, 64, 3, 13), (5, 128, 3, 4), (4, 256, 3, 2),
-                                         (3, 512, 3, 7), (2, 70, 5, 3)])
+                                         (3, 512, 3, 7), (2, 70, 5, 3), (19, 160, 3, 1), (128, 512, 3, 4),
+                                         (33, 256, 3, 16), (5, 192, 5, 6), (40, 1024, 3, 28)])
 def test_channel_branch_parts_matches_fp64(n, c, k, tiles, dtype, tol):
     torch.manual_seed(n + c)
     mid = int(c * 0.2)
