@@ -423,16 +423,34 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
     for (int t = 0; t < KK; ++t)
 #pragma unroll
         for (int k = 0; k < VP; ++k) acc[t][k] = 0.f;
+    // POOL: where this lane's sums of the wave's first channel group go (one partial sum
+    // per row of 16 lanes: four per tile), and how many groups the wave keeps sums of (head
+    // 0 of a sample does it for all heads).  Worked out here and pinned: formed inside the
+    // walk they take a scalar load of a launch dimension, and the wait for it also waits
+    // for the weights that were just requested for the next step.  The sums go out through
+    // a buffer descriptor of the tile's 4 * C values, lanes with nothing to write at an
+    // offset outside it: a store under a branch leaves the compiler unable to count the
+    // loads in flight where the branch joins, and it then waits for all of them.
+    // (Collecting the sums in LDS and writing them after the walk was no faster.)
+    __amdgpu_buffer_rsrc_t pool_rsrc = plane_rsrc(nullptr, 0u);
+    uint32_t pool_off = kOutside;
+    int pool_groups = 0;
+    if constexpr (POOL) {
+        pool_rsrc = plane_rsrc(pool_part + ((n * gridDim.x + blockIdx.x) * 4) * g.C,
+                               (uint32_t)(4 * g.C) * (uint32_t)sizeof(float));
+        if (head == 0 && (lane & 15) < U)
+            pool_off = (uint32_t)((lane >> 4) * g.C + j0 * U + (lane & 15)) * (uint32_t)sizeof(float);
+        pool_groups = head == 0 ? min(g.gpw, g.ngroups - j0) : 0;
+        asm volatile("" : "+v"(pool_off), "+s"(pool_groups));
+    }
     auto compute = [&](auto st_tag, int i) __attribute__((always_inline)) {
         constexpr int ST = decltype(st_tag)::value;
         if constexpr (POOL) {
-            // (head 0 of a sample does it for all heads.  No branch around the arithmetic: it
-            // would cut the step into blocks, and the waits the compiler then places at their
-            // joins cost more than the sums of a group the wave does not have.)
-            const bool keep = head == 0 && i < g.gpw && j0 + i < g.ngroups;
+            // (No branch around the arithmetic: it would cut the step into blocks, and the
+            // waits the compiler then places at their joins cost more than the sums of a
+            // group the wave does not have.)
+            const bool keep = i < pool_groups;
             {
-                // (one partial sum per row of 16 lanes: four per tile)
-                float *dst = pool_part + (((n * gridDim.x + blockIdx.x) * 4 + (lane >> 4)) * g.C + (int64_t)(j0 + i) * U);
                 float psum[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
@@ -464,7 +482,9 @@ __global__ __launch_bounds__(WAVES * kWave) void k_spatial_stream(
                     psum[u] = ps;
                 }
                 const float tot = row_sums<U>(psum, lane);
-                if (keep && (lane & 15) < U) dst[lane & 15] = tot;
+                __builtin_amdgcn_raw_buffer_store_b32(
+                    __float_as_uint(tot), pool_rsrc,
+                    (int)(keep ? pool_off + (uint32_t)(i * U) * (uint32_t)sizeof(float) : kOutside), 0, 0);
             }
         }
         if constexpr (sizeof(T) == 2) {

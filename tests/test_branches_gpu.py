@@ -127,6 +127,38 @@ def test_channel_branch_without_biases_and_vectors(n, c, k):
     assert err < 6e-3, err
 
 
+def test_channel_branch_operands_at_odd_addresses():
+    """Weights, biases and vectors that start 2 bytes into their allocations (views of
+    larger tensors): whichever kernel takes the call, the taps are the same as from
+    aligned copies."""
+    torch.manual_seed(3)
+    n, c, k = 20, 256, 3
+    mid = int(c * 0.2)
+
+    def shifted(t):
+        store = torch.empty(t.numel() + 1, device='cuda', dtype=t.dtype)
+        view = store[1:].view(t.shape)
+        view.copy_(t)
+        return view
+
+    pooled = torch.randn(n, c, device='cuda').half()
+    w1 = (torch.randn(mid, c, device='cuda') * 0.2).half()
+    b1 = torch.randn(mid, device='cuda').half()
+    w2 = (torch.randn(c * k * k, mid, device='cuda') * 0.3).half()
+    b2 = torch.randn(c * k * k, device='cuda').half()
+    gv = (torch.rand(c * k * k, device='cuda') + 0.5).half()
+    ov = torch.randn(c * k * k, device='cuda').half()
+    want = _lib.channel_branch(pooled, w1, b1, w2, b2, k, 1.0, gv, ov)
+    ref = channel_reference(*(t.cpu() for t in (pooled, w1, b1, w2, b2)), k, 1.0, gv.cpu(), ov.cpu())
+    scale = ref.abs().max()
+    for which in range(7):
+        args = [pooled, w1, b1, w2, b2, gv, ov]
+        args[which] = shifted(args[which])
+        out = _lib.channel_branch(args[0], args[1], args[2], args[3], args[4], k, 1.0, args[5], args[6])
+        assert ((out.double().cpu() - ref).abs().max() / scale).item() < 6e-3, which
+        assert ((out.float() - want.float()).abs().max() / scale).item() < 2e-3, which
+
+
 POOL_CASES = [(2, 64, 56, 56, 1, 1), (2, 128, 56, 56, 2, 1), (2, 128, 28, 28, 1, 1), (2, 256, 28, 28, 2, 1),
               (2, 256, 14, 14, 1, 1), (2, 512, 14, 14, 2, 1), (2, 512, 7, 7, 1, 1), (3, 16, 12, 14, 1, 1),
               (3, 16, 12, 14, 2, 1), (3, 16, 9, 11, 1, 4), (2, 36, 10, 18, 2, 3), (1, 8, 5, 3, 1, 1),
