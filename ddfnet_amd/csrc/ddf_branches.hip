@@ -11,7 +11,9 @@
 //     cf[n, c, t] = norm_t( b2[c*KK + t] + sum_m w2[c*KK + t, m] * relu(b1[m] + sum_c' w1[m, c'] * v[n, c']) )
 //   the two 1x1 convolutions on the pooled (n, c) vector are small matrix
 //   products; one workgroup computes the hidden vector of its sample and 64
-//   (wide layers: 128) channels' filters, and normalises them in place.
+//   (wide layers: 128) channels' filters, and normalises them in place
+//   (k_channel_branch), or, in fp16 with a hidden layer of 32 values or more,
+//   sixteen samples x sixteen channels on the matrix cores (k_channel_branch_mma).
 //
 // norm_t(u) = gain_t * (u_t - mean(u)) / (std(u) + 1e-10) + offset_t with the
 // unbiased standard deviation over the KK taps, as in ddf_filter_norm.hip.
