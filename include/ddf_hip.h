@@ -263,6 +263,11 @@ int ddf_hip_spatial_branch(const void *features, const void *weight,
  * filters.  gain / gain_vec / offset_vec as in ddf_hip_filter_norm with
  * groups = C.  Inference path, as above.  DDF_ERR_UNSUPPORTED: kernel size
  * other than 3 or 5, fp64, or C + mid beyond what one workgroup's LDS holds.
+ * fp16 with mid >= 32 and C a multiple of 32 runs on the matrix cores (operands
+ * aligned for vector loads: weight1 to 16 bytes, pooled, bias2, gain_vec,
+ * offset_vec and channel_filter to 8; anything else takes the vector-ALU
+ * kernel): sums in fp32, the pooled and hidden vectors rounded to fp16 as the
+ * reference's half-precision modules round them.
  */
 int ddf_hip_channel_branch(const void *pooled, const void *weight1,
                            const void *bias1, const void *weight2,
